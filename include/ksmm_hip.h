@@ -1,0 +1,133 @@
+/* C ABI of libksmm_hip.so: Kronecker-sparse matrix multiplication on MI355X (gfx950).
+ *
+ * A factor with pattern (a, b, c, d) holds a*b*c*d weights and maps a*c*d input features to
+ * a*b*d output features:
+ *
+ *     y[a_i, b_i, d_i, n] = scale * sum_{c_i} W[a_i, b_i, c_i, d_i] * x[a_i, c_i, d_i, n]
+ *
+ * Tensors are plain device pointers:
+ *   x  input,  bs_last ? (a*c*d, batch) : (batch, a*c*d), row-major, contiguous
+ *   w  weight in the reference's "kernel" format (a*d*c, b), row-major: element
+ *      (a_i, b_i, c_i, d_i) at row (a_i*d + d_i)*c + c_i, column b_i
+ *      (reference: src/ksmm_py/layer/kronecker_sparse/interface.py:65-69)
+ *   y  output, bs_last ? (a*b*d, batch) : (batch, a*b*d); never aliases x
+ * All accumulation is fp32.  Supported (x, w, y) element types:
+ *   (F32, F32, F32)   (F16, F16, F16)   (FP8_E4M3, FP8_E4M3, F16)   (F16, FP8_E4M3, F16)
+ * FP8_E4M3 is the OCP e4m3fn encoding (torch.float8_e4m3fn); `scale` carries the product of
+ * the per-tensor dequantisation scales and is applied to the fp32 accumulator before the
+ * result is rounded to the output type.
+ *
+ * The library never allocates device memory and keeps no mutable global state.  All
+ * launches go to the stream the caller passes (a hipStream_t cast to void*; NULL is the
+ * legacy default stream).  Every entry point returns KSMM_OK or a negative error code;
+ * ksmm_strerror() names it.  Only ksmm_factor_forward*, ksmm_chain_forward* touch the GPU.
+ */
+#ifndef KSMM_HIP_H
+#define KSMM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KSMM_VERSION 1
+
+typedef enum ksmm_dtype {
+    KSMM_F32 = 0,
+    KSMM_F16 = 1,
+    KSMM_FP8_E4M3 = 2
+} ksmm_dtype;
+
+typedef enum ksmm_status {
+    KSMM_OK = 0,
+    KSMM_ERR_NULL_POINTER = -1,   /* x, w or y is NULL                                        */
+    KSMM_ERR_BAD_PATTERN = -2,    /* a, b, c or d < 1                                         */
+    KSMM_ERR_BAD_BATCH = -3,      /* batch < 1                                                */
+    KSMM_ERR_BAD_DTYPE = -4,      /* (x, w, y) type combination not in the list above         */
+    KSMM_ERR_TOO_LARGE = -5,      /* a tensor has 2^31 elements or more                       */
+    KSMM_ERR_BAD_ALGO = -6,       /* forced kernel id unknown, or it cannot run this problem  */
+    KSMM_ERR_LAUNCH = -7,         /* HIP reported an error at launch                          */
+    KSMM_ERR_CHAIN_MISMATCH = -8, /* output size of factor i != input size of factor i+1      */
+    KSMM_ERR_WORKSPACE = -9,      /* workspace missing or smaller than ksmm_chain_workspace   */
+    KSMM_ERR_BAD_CHAIN = -10,     /* n_factors < 1 or > KSMM_MAX_FACTORS                      */
+    KSMM_ERR_ALIAS = -11          /* y overlaps x                                             */
+} ksmm_status;
+
+/* Kernel families.  KSMM_ALGO_AUTO lets the tile table decide. */
+typedef enum ksmm_algo {
+    KSMM_ALGO_AUTO = 0,
+    KSMM_ALGO_GENERIC = 1, /* one thread per output element group; any shape              */
+    KSMM_ALGO_WAVE = 2,    /* weights stationary in registers, one wavefront per group    */
+    KSMM_ALGO_TILE = 3     /* LDS-staged MFMA tiles                                       */
+} ksmm_algo;
+
+/* What the tile table chose for a problem.  Replaces the reference's generated
+ * `best_kernel_bs_{first,last}_{float,half}` if-chains
+ * (src/ksmm_py/layer/kronecker_sparse/kernel_bs_first_float.cuh:8-21) and the rows of
+ * kernel_bs_*.best (batch a b c d TILEX TILEK TILEY TX TY VSIZE ms std mse). */
+typedef struct ksmm_tile {
+    int algo;         /* ksmm_algo actually used                                           */
+    int variant;      /* index of the template instance inside that family                 */
+    int tile_m;       /* outputs of one (a_i, d_i) block computed by a workgroup           */
+    int tile_n;       /* batch columns per workgroup iteration                             */
+    int tile_k;       /* slab of c staged per step                                         */
+    int tile_d;       /* consecutive d_i handled by one workgroup                          */
+    int threads;      /* workgroup size                                                    */
+    int lds_bytes;    /* LDS per workgroup                                                 */
+    int64_t grid;     /* number of workgroups                                              */
+} ksmm_tile;
+
+typedef struct ksmm_factor_desc {
+    const void *w;    /* kernel-format weight (a*d*c, b)                                   */
+    int a, b, c, d;
+    int w_dtype;      /* ksmm_dtype                                                        */
+    float scale;      /* multiplies this factor's fp32 accumulator                         */
+} ksmm_factor_desc;
+
+#define KSMM_MAX_FACTORS 16
+
+int ksmm_version(void);
+const char *ksmm_strerror(int status);
+
+/* Host-only argument check (no GPU needed).  Mirrors the checks of the reference binding
+ * (src/ksmm_py/layer/kronecker_sparse/kernel.cpp:36-42, kernel.cu:123-125), as codes. */
+int ksmm_validate(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                  int y_dtype, int bs_last);
+
+/* Tile-table lookup (host only).  `algo` = KSMM_ALGO_AUTO or a forced family. */
+int ksmm_query_tile(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                    int y_dtype, int bs_last, int algo, ksmm_tile *out);
+
+/* One factor.  Replaces `kernel.forward(input, factor, bs_last, a, b, c, d, dtype, vsize)`
+ * (src/ksmm_py/layer/kronecker_sparse/kernel.cpp:25-45 -> kernel.cu:40-127); the caller
+ * allocates y. */
+int ksmm_factor_forward(const void *x, const void *w, void *y, int64_t batch, int a, int b,
+                        int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                        float scale, void *stream);
+
+/* Same, with the kernel family (and optionally a variant, -1 = table default) forced; used
+ * by the tuner and by tests that must exercise one family. */
+int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batch, int a,
+                             int b, int c, int d, int x_dtype, int w_dtype, int y_dtype,
+                             int bs_last, float scale, int algo, int variant, void *stream);
+
+/* Bytes of device workspace ksmm_chain_forward needs for these factors (two ping-pong
+ * intermediates; 0 for a single factor).  Intermediates have type y_dtype. */
+int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
+                             int y_dtype);
+
+/* A chain K_n ... K_1 x: factors[0] acts first.  Replaces the Python loop of
+ * KSLinear.forward_bs_first / forward_bs_last
+ * (src/ksmm_py/layer/kronecker_sparse/interface.py:193-211, 269-291).  The first factor
+ * reads x in x_dtype; intermediates and y have y_dtype.  `fuse` != 0 allows kernels that
+ * keep intermediates in LDS when the table has one for this chain. */
+int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
+                       void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
+                       int y_dtype, int bs_last, int fuse, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KSMM_HIP_H */

@@ -1,0 +1,183 @@
+// C ABI of libksmm_hip.so: argument checks, kernel-family dispatch, factor chains.
+#include <string.h>
+
+#include "ksmm_common.h"
+
+using namespace ksmm;
+
+namespace {
+
+bool dtype_known(int dt) { return dt == KSMM_F32 || dt == KSMM_F16 || dt == KSMM_FP8_E4M3; }
+
+int check_shape(int64_t batch, int a, int b, int c, int d, int xd, int wd, int yd)
+{
+    if (a < 1 || b < 1 || c < 1 || d < 1) return KSMM_ERR_BAD_PATTERN;
+    if (batch < 1) return KSMM_ERR_BAD_BATCH;
+    if (!dtype_known(xd) || !dtype_known(wd) || !dtype_known(yd)) return KSMM_ERR_BAD_DTYPE;
+    if (combo_of(xd, wd, yd) < 0) return KSMM_ERR_BAD_DTYPE;
+    const int64_t lim = 0x7fffffffLL;
+    // products are checked step by step so that they cannot wrap
+    int64_t acd = (int64_t)a * c;
+    if (acd > lim) return KSMM_ERR_TOO_LARGE;
+    acd *= d;
+    int64_t abd = (int64_t)a * b;
+    if (abd > lim) return KSMM_ERR_TOO_LARGE;
+    abd *= d;
+    if (acd > lim || abd > lim) return KSMM_ERR_TOO_LARGE;
+    if (acd * batch > lim || abd * batch > lim) return KSMM_ERR_TOO_LARGE;
+    int64_t nnz = (int64_t)a * b;
+    nnz *= c;
+    if (nnz > lim) return KSMM_ERR_TOO_LARGE;
+    nnz *= d;
+    if (nnz > lim) return KSMM_ERR_TOO_LARGE;
+    return KSMM_OK;
+}
+
+// Family order for KSMM_ALGO_AUTO: the table inside each family decides whether it takes the
+// problem; the generic family always does.
+int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *tile)
+{
+    switch (algo) {
+    case KSMM_ALGO_GENERIC: return generic_run(p, variant, launch, tile);
+    case KSMM_ALGO_WAVE: return wave_run(p, variant, launch, tile);
+    case KSMM_ALGO_TILE: return tile_run(p, variant, launch, tile);
+    case KSMM_ALGO_AUTO: {
+        int rc = wave_run(p, -1, launch, tile);
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        rc = tile_run(p, -1, launch, tile);
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        return generic_run(p, -1, launch, tile);
+    }
+    default: return KSMM_ERR_BAD_ALGO;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ksmm_version(void) { return KSMM_VERSION; }
+
+const char *ksmm_strerror(int status)
+{
+    switch (status) {
+    case KSMM_OK: return "ok";
+    case KSMM_ERR_NULL_POINTER: return "null tensor pointer";
+    case KSMM_ERR_BAD_PATTERN: return "pattern (a,b,c,d) must be four positive integers";
+    case KSMM_ERR_BAD_BATCH: return "batch size must be positive";
+    case KSMM_ERR_BAD_DTYPE: return "unsupported data type combination";
+    case KSMM_ERR_TOO_LARGE: return "tensor too large (2^31 elements or more)";
+    case KSMM_ERR_BAD_ALGO: return "kernel family/variant unknown or not applicable to this problem";
+    case KSMM_ERR_LAUNCH: return "HIP kernel launch failed";
+    case KSMM_ERR_CHAIN_MISMATCH: return "consecutive factors have incompatible sizes";
+    case KSMM_ERR_WORKSPACE: return "workspace missing or too small";
+    case KSMM_ERR_BAD_CHAIN: return "bad number of factors";
+    case KSMM_ERR_ALIAS: return "output overlaps input";
+    default: return "unknown ksmm status";
+    }
+}
+
+int ksmm_validate(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                  int y_dtype, int bs_last)
+{
+    (void)bs_last;
+    return check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
+}
+
+int ksmm_query_tile(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                    int y_dtype, int bs_last, int algo, ksmm_tile *out)
+{
+    if (!out) return KSMM_ERR_NULL_POINTER;
+    int rc = check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    Problem p{nullptr, nullptr, nullptr, batch, a, b, c, d, x_dtype, w_dtype, y_dtype,
+              bs_last ? 1 : 0, 1.f, nullptr};
+    memset(out, 0, sizeof(*out));
+    return dispatch(p, algo, -1, false, out);
+}
+
+int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batch, int a,
+                             int b, int c, int d, int x_dtype, int w_dtype, int y_dtype,
+                             int bs_last, float scale, int algo, int variant, void *stream)
+{
+    int rc = check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    if (!x || !w || !y) return KSMM_ERR_NULL_POINTER;
+    const char *xb = (const char *)x, *yb = (const char *)y;
+    const int64_t xbytes = (int64_t)a * c * d * batch * (int64_t)dtype_size(x_dtype);
+    const int64_t ybytes = (int64_t)a * b * d * batch * (int64_t)dtype_size(y_dtype);
+    if (xb < yb + ybytes && yb < xb + xbytes) return KSMM_ERR_ALIAS;
+    Problem p{x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last ? 1 : 0, scale,
+              (hipStream_t)stream};
+    return dispatch(p, algo, variant, true, nullptr);
+}
+
+int ksmm_factor_forward(const void *x, const void *w, void *y, int64_t batch, int a, int b,
+                        int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                        float scale, void *stream)
+{
+    return ksmm_factor_forward_algo(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last,
+                                    scale, KSMM_ALGO_AUTO, -1, stream);
+}
+
+static int check_chain(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype)
+{
+    if (!f) return KSMM_ERR_NULL_POINTER;
+    if (n < 1 || n > KSMM_MAX_FACTORS) return KSMM_ERR_BAD_CHAIN;
+    for (int i = 0; i < n; ++i) {
+        // the first factor reads x_dtype, later ones read the intermediate type y_dtype
+        int rc = check_shape(batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
+                             f[i].w_dtype, y_dtype);
+        if (rc != KSMM_OK) return rc;
+        if (i > 0 && (int64_t)f[i].a * f[i].c * f[i].d != (int64_t)f[i - 1].a * f[i - 1].b * f[i - 1].d)
+            return KSMM_ERR_CHAIN_MISMATCH;
+    }
+    return KSMM_OK;
+}
+
+int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
+                             int y_dtype)
+{
+    if (!factors) return KSMM_ERR_NULL_POINTER;
+    if (n_factors < 1 || n_factors > KSMM_MAX_FACTORS) return KSMM_ERR_BAD_CHAIN;
+    if (batch < 1) return KSMM_ERR_BAD_BATCH;
+    if (!dtype_known(y_dtype)) return KSMM_ERR_BAD_DTYPE;
+    int64_t widest = 0;
+    for (int i = 0; i + 1 < n_factors; ++i) {
+        if (factors[i].a < 1 || factors[i].b < 1 || factors[i].d < 1) return KSMM_ERR_BAD_PATTERN;
+        int64_t o = (int64_t)factors[i].a * factors[i].b * factors[i].d;
+        if (o > widest) widest = o;
+    }
+    // two buffers, each rounded up to 256 bytes so that both stay 256-byte aligned
+    int64_t one = (widest * batch * (int64_t)dtype_size(y_dtype) + 255) / 256 * 256;
+    return n_factors > 1 ? 2 * one : 0;
+}
+
+int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
+                       void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
+                       int y_dtype, int bs_last, int fuse, void *stream)
+{
+    int rc = check_chain(factors, n_factors, batch, x_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    if (!x || !y) return KSMM_ERR_NULL_POINTER;
+    for (int i = 0; i < n_factors; ++i)
+        if (!factors[i].w) return KSMM_ERR_NULL_POINTER;
+    (void)fuse;
+    const int64_t need = ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
+    if (n_factors > 1 && (!workspace || workspace_bytes < need)) return KSMM_ERR_WORKSPACE;
+    char *buf[2] = {(char *)workspace, (char *)workspace + need / 2};
+    const void *cur = x;
+    int cur_dtype = x_dtype;
+    for (int i = 0; i < n_factors; ++i) {
+        void *dst = (i == n_factors - 1) ? y : (void *)buf[i & 1];
+        rc = ksmm_factor_forward_algo(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b,
+                                      factors[i].c, factors[i].d, cur_dtype, factors[i].w_dtype,
+                                      y_dtype, bs_last, factors[i].scale, KSMM_ALGO_AUTO, -1, stream);
+        if (rc != KSMM_OK) return rc;
+        cur = dst;
+        cur_dtype = y_dtype;
+    }
+    return KSMM_OK;
+}
+
+}  // extern "C"

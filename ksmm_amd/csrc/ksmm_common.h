@@ -1,0 +1,95 @@
+// Shared device/host helpers for the KS kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ksmm_hip.h"
+
+namespace ksmm {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+struct fp8_t {  // OCP e4m3fn storage
+    uint8_t bits;
+};
+
+// e4m3fn -> fp16 is exact: shift the 7 magnitude bits into the fp16 exponent/mantissa
+// fields and rescale by 2^8 (the difference of the exponent biases, 15 - 7).  Sub-normals
+// of e4m3fn land on fp16 sub-normals before the rescale, so they come out exact as well.
+__device__ __forceinline__ half_t fp8_to_half(uint8_t v)
+{
+    uint16_t h = (uint16_t)(((uint16_t)(v & 0x80u) << 8) | ((uint16_t)(v & 0x7fu) << 7));
+    return __builtin_bit_cast(half_t, h) * (half_t)256.0f;
+}
+
+// Two e4m3fn bytes (bits 0-7 and 8-15 of `v`) -> packed fp16 pair.
+__device__ __forceinline__ half2_t fp8x2_to_half2(uint32_t v)
+{
+    // bytes -> high byte of each 16-bit lane: 0x b1 00 b0 00
+    uint32_t u = __builtin_amdgcn_perm(0u, v, 0x010c000cu);
+    uint32_t t = ((u >> 1) & 0x3f803f80u) | (u & 0x80008000u);
+    half2_t h = __builtin_bit_cast(half2_t, t);
+    half2_t k = {(half_t)256.0f, (half_t)256.0f};
+    return h * k;
+}
+
+template <typename T> struct elem;
+template <> struct elem<float> {
+    static constexpr int dtype = KSMM_F32;
+    __device__ static __forceinline__ float load(const float *p) { return *p; }
+    __device__ static __forceinline__ void store(float *p, float v) { *p = v; }
+};
+template <> struct elem<half_t> {
+    static constexpr int dtype = KSMM_F16;
+    __device__ static __forceinline__ float load(const half_t *p) { return (float)*p; }
+    __device__ static __forceinline__ void store(half_t *p, float v) { *p = (half_t)v; }
+};
+template <> struct elem<fp8_t> {
+    static constexpr int dtype = KSMM_FP8_E4M3;
+    __device__ static __forceinline__ float load(const fp8_t *p) { return (float)fp8_to_half(p->bits); }
+};
+
+static inline size_t dtype_size(int dt)
+{
+    return dt == KSMM_F32 ? 4 : dt == KSMM_F16 ? 2 : 1;
+}
+
+// One factor problem, as the launchers see it.
+struct Problem {
+    const void *x;
+    const void *w;
+    void *y;
+    int64_t batch;
+    int a, b, c, d;
+    int x_dtype, w_dtype, y_dtype;
+    int bs_last;
+    float scale;
+    hipStream_t stream;
+};
+
+// dtype combination index: 0 f32, 1 f16, 2 fp8*fp8->f16, 3 f16*fp8->f16, -1 unsupported
+static inline int combo_of(int xd, int wd, int yd)
+{
+    if (xd == KSMM_F32 && wd == KSMM_F32 && yd == KSMM_F32) return 0;
+    if (xd == KSMM_F16 && wd == KSMM_F16 && yd == KSMM_F16) return 1;
+    if (xd == KSMM_FP8_E4M3 && wd == KSMM_FP8_E4M3 && yd == KSMM_F16) return 2;
+    if (xd == KSMM_F16 && wd == KSMM_FP8_E4M3 && yd == KSMM_F16) return 3;
+    return -1;
+}
+
+// Launchers, one per kernel family.  Each fills `tile` and, when `launch` is true, enqueues
+// the kernel on p.stream.  They return KSMM_ERR_BAD_ALGO when the family (or the requested
+// variant) cannot run the problem.
+int generic_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
+int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
+int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
+
+}  // namespace ksmm

@@ -1,0 +1,4 @@
+#include "ksmm_common.h"
+namespace ksmm {
+int tile_run(const Problem &, int, bool, ksmm_tile *) { return KSMM_ERR_BAD_ALGO; }
+}

@@ -1,0 +1,135 @@
+"""``Kernel.forward``: the per-factor entry point ``KSLinear(algo='kernel')`` calls.
+
+Same positional signature as the reference's
+``Kernel.forward(input, factor, bs_last, a, b, c, d, dtype, vsize)``
+(src/ksmm_py/layer/kronecker_sparse/kernel.py:61-73).  Instead of rewriting ``.cuh`` files
+and JIT-compiling per (pattern, batch), it calls the prebuilt C ABI (include/ksmm_hip.h)
+with raw device pointers on the current PyTorch stream.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+_DTYPES = {
+    torch.float32: _lib.KSMM_F32,
+    torch.float16: _lib.KSMM_F16,
+    torch.float8_e4m3fn: _lib.KSMM_FP8_E4M3,
+}
+
+
+def dtype_code(dt):
+    try:
+        return _DTYPES[dt]
+    except KeyError:
+        # kernel.cu:123-125: assert(0 && "Unsupported data type")
+        raise AssertionError("Unsupported data type %s" % (dt,))
+
+
+def _check_input(t, name):
+    # kernel.cpp:19-23
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+
+
+def _stream_ptr(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+class Kernel:
+    """Namespace with the reference's static-method calling convention (forward only)."""
+
+    @staticmethod
+    def forward(input, factor, bs_last, a, b, c, d, dtype=None, vsize=4, scale=1.0,
+                algo=_lib.ALGO_AUTO, variant=-1, out=None):
+        """y = K x for one factor.
+
+        ``input``: (a*c*d, batch) if ``bs_last`` else (batch, a*c*d); ``factor``: kernel
+        format (a*d*c, b).  ``dtype`` is accepted for signature compatibility: the element
+        types are taken from the tensors.  ``vsize`` is accepted and ignored (vector widths
+        are part of the tile table).  fp8 inputs/weights produce an fp16 result scaled by
+        ``scale``.
+        """
+        lib = _lib.load()
+        _check_input(input, "input")
+        _check_input(factor, "factor")
+        bs_last = bool(bs_last)
+        in_size = a * c * d
+        out_size = a * b * d
+        # kernel.cpp:38-42
+        assert input.dim() == 2 and factor.dim() == 2
+        assert in_size == input.size(0 if bs_last else 1)
+        assert factor.size(0) == input.size(0 if bs_last else 1)
+        assert b == factor.size(1)
+        batch = input.size(1 if bs_last else 0)
+        xd, wd = dtype_code(input.dtype), dtype_code(factor.dtype)
+        out_dtype = torch.float16 if wd == _lib.KSMM_FP8_E4M3 else input.dtype
+        shape = (out_size, batch) if bs_last else (batch, out_size)
+        if out is None:
+            out = torch.empty(shape, dtype=out_dtype, device=input.device)
+        else:
+            assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
+        with torch.cuda.device(input.device):
+            rc = lib.ksmm_factor_forward_algo(
+                input.data_ptr(), factor.data_ptr(), out.data_ptr(), batch, a, b, c, d, xd, wd,
+                dtype_code(out_dtype), int(bs_last), float(scale), int(algo), int(variant),
+                _stream_ptr(input))
+        _lib.check(rc)
+        return out
+
+    @staticmethod
+    def chain_forward(input, factors, patterns, bs_last, scales=None, fuse=True, workspace=None):
+        """All factors of a KSLinear in one call (factor-chain launcher)."""
+        lib = _lib.load()
+        _check_input(input, "input")
+        n = len(factors)
+        assert n == len(patterns) and 1 <= n <= _lib.MAX_FACTORS
+        bs_last = bool(bs_last)
+        descs = (_lib.KsmmFactorDesc * n)()
+        any_fp8 = False
+        for i, (f, p) in enumerate(zip(factors, patterns)):
+            _check_input(f, "factor")
+            a, b, c, d = p
+            assert f.dim() == 2 and f.size(0) == a * c * d and f.size(1) == b
+            descs[i].w = f.data_ptr()
+            descs[i].a, descs[i].b, descs[i].c, descs[i].d = a, b, c, d
+            descs[i].w_dtype = dtype_code(f.dtype)
+            descs[i].scale = 1.0 if scales is None else float(scales[i])
+            any_fp8 |= f.dtype == torch.float8_e4m3fn
+        a0, _, c0, d0 = patterns[0]
+        al, bl, _, dl = patterns[-1]
+        assert input.dim() == 2 and input.size(0 if bs_last else 1) == a0 * c0 * d0
+        batch = input.size(1 if bs_last else 0)
+        out_dtype = torch.float16 if any_fp8 else input.dtype
+        out_size = al * bl * dl
+        out = torch.empty((out_size, batch) if bs_last else (batch, out_size), dtype=out_dtype,
+                          device=input.device)
+        need = lib.ksmm_chain_workspace(descs, n, batch, dtype_code(out_dtype))
+        if need < 0:
+            _lib.check(int(need))
+        if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
+            workspace = torch.empty(need, dtype=torch.uint8, device=input.device)
+        ws_ptr = workspace.data_ptr() if need > 0 else None
+        ws_bytes = workspace.numel() * workspace.element_size() if need > 0 else 0
+        with torch.cuda.device(input.device):
+            rc = lib.ksmm_chain_forward(descs, n, input.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes,
+                                        batch, dtype_code(input.dtype), dtype_code(out_dtype),
+                                        int(bs_last), int(bool(fuse)), _stream_ptr(input))
+        _lib.check(rc)
+        return out
+
+
+def query_tile(batch, pattern, x_dtype, w_dtype=None, bs_last=True, algo=_lib.ALGO_AUTO):
+    """What the tile table picks for one factor (host only; no GPU needed)."""
+    lib = _lib.load()
+    w_dtype = x_dtype if w_dtype is None else w_dtype
+    y_dtype = torch.float16 if w_dtype == torch.float8_e4m3fn else x_dtype
+    t = _lib.KsmmTile()
+    a, b, c, d = pattern
+    _lib.check(lib.ksmm_query_tile(batch, a, b, c, d, dtype_code(x_dtype), dtype_code(w_dtype),
+                                   dtype_code(y_dtype), int(bool(bs_last)), int(algo),
+                                   ctypes.byref(t)))
+    return t.as_dict()

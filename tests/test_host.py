@@ -1,0 +1,192 @@
+"""CPU-only checks of the host side: the C ABI loads and exports every declared symbol, its
+argument validation returns the documented codes, and KSLinear's host logic mirrors the
+reference's error behaviour.  No GPU call is made."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import ks_oracle as O
+from tests.util import seeded_input, seeded_weights
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from ksmm_amd import _lib
+
+    header = open(os.path.join(ROOT, "include", "ksmm_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ksmm_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.ksmm_version() == 1
+
+
+def test_struct_layout_matches_header():
+    from ksmm_amd import _lib
+
+    assert ctypes.sizeof(_lib.KsmmTile) == 40
+    assert ctypes.sizeof(_lib.KsmmFactorDesc) == 32
+
+
+@pytest.mark.parametrize("args,code", [
+    ((25088, 1, 48, 48, 16, 0, 0, 0, 1), 0),
+    ((25088, 1, 48, 48, 16, 1, 1, 1, 0), 0),
+    ((25088, 1, 16, 16, 64, 2, 2, 1, 1), 0),
+    ((25088, 16, 16, 16, 4, 1, 2, 1, 1), 0),
+    ((25088, 0, 48, 48, 16, 0, 0, 0, 1), -2),
+    ((25088, 1, 48, -1, 16, 0, 0, 0, 1), -2),
+    ((0, 1, 48, 48, 16, 0, 0, 0, 1), -3),
+    ((25088, 1, 48, 48, 16, 0, 1, 0, 1), -4),      # f32 x with f16 w
+    ((25088, 1, 48, 48, 16, 2, 2, 2, 1), -4),      # fp8 output is not provided
+    ((25088, 1, 48, 48, 16, 7, 0, 0, 1), -4),
+    ((1 << 20, 1, 4096, 4096, 1, 0, 0, 0, 1), -5),
+    ((2, 1 << 15, 1 << 15, 1 << 15, 1 << 15, 0, 0, 0, 1), -5),
+])
+def test_validate_codes(lib, args, code):
+    assert lib.ksmm_validate(*args) == code
+    assert lib.ksmm_strerror(code)
+
+
+def test_strerror_distinct(lib):
+    msgs = {lib.ksmm_strerror(c) for c in range(0, -12, -1)}
+    assert len(msgs) == 12
+    assert lib.ksmm_strerror(-99) == b"unknown ksmm status"
+
+
+def test_query_tile_host_only(lib):
+    from ksmm_amd import query_tile
+
+    for prec in (torch.float32, torch.float16, torch.float8_e4m3fn):
+        for bs_last in (True, False):
+            for pattern in [(1, 48, 48, 16), (4, 192, 192, 1), (1, 17, 33, 2), (64, 16, 16, 1)]:
+                t = query_tile(25088, pattern, prec, bs_last=bs_last)
+                assert t["algo"] in (1, 2, 3) and t["threads"] > 0 and t["grid"] > 0
+                assert t["lds_bytes"] <= 160 * 1024
+    # the generic family takes anything
+    assert query_tile(3, (1, 17, 33, 2), torch.float32, algo=1)["algo"] == 1
+
+
+def test_forward_rejects_bad_arguments_without_gpu(lib):
+    # null pointers and aliasing are detected before any launch
+    f = lib.ksmm_factor_forward
+    assert f(None, None, None, 8, 1, 2, 2, 1, 0, 0, 0, 1, 1.0, None) == -1
+    assert f(4096, 8192, 4096, 8, 1, 2, 2, 1, 0, 0, 0, 1, 1.0, None) == -11
+    assert f(4096, 8192, 4096 + 32, 8, 1, 2, 2, 1, 0, 0, 0, 1, 1.0, None) == -11
+    assert lib.ksmm_factor_forward_algo(4096, 8192, 1 << 20, 8, 1, 2, 2, 1, 0, 0, 0, 1, 1.0, 99, -1,
+                                        None) == -6
+
+
+def test_chain_argument_checks(lib):
+    from ksmm_amd import _lib
+
+    d = (_lib.KsmmFactorDesc * 2)()
+    for i, p in enumerate([(2, 3, 5, 4), (3, 6, 4, 2)]):
+        d[i].w = 4096
+        d[i].a, d[i].b, d[i].c, d[i].d = p
+        d[i].w_dtype, d[i].scale = 0, 1.0
+    need = lib.ksmm_chain_workspace(d, 2, 100, 0)
+    assert need == 2 * ((24 * 100 * 4 + 255) // 256 * 256)
+    assert lib.ksmm_chain_workspace(d, 1, 100, 0) == 0
+    assert lib.ksmm_chain_workspace(d, 0, 100, 0) == -10
+    assert lib.ksmm_chain_forward(d, 2, 4096, 8192, None, 0, 100, 0, 0, 1, 1, None) == -9
+    d[1].c = 5  # 3*5*2 = 30 != 24
+    assert lib.ksmm_chain_forward(d, 2, 4096, 8192, 1 << 20, need, 100, 0, 0, 1, 1, None) == -8
+    assert lib.ksmm_chain_forward(d, 17, 4096, 8192, 1 << 20, need, 100, 0, 0, 1, 1, None) == -10
+
+
+def test_kslinear_constructor_contract():
+    from ksmm_amd import KSLinear
+
+    with pytest.raises(Exception, match="kernel expects device='cuda'"):
+        KSLinear([(1, 2, 2, 1)], algo="kernel", device="cpu")      # interface.py:163-164
+    with pytest.raises(AssertionError):
+        KSLinear([(1, 2, 2, 1)], algo="nope")                      # interface.py:141-148
+    with pytest.raises(AssertionError):
+        KSLinear([(1, 2, 2)], algo="dense")                        # interface.py:149-150
+    with pytest.raises(AssertionError):
+        KSLinear([(1, 2, 2, 1)], weights=[None, None], algo="dense")  # interface.py:170
+    k = KSLinear([(2, 3, 5, 4), (3, 6, 4, 2)], algo="bmm", dtype=torch.float32, bs_last=True)
+    assert (k.in_size, k.out_size, k.num_mat, k.algo, k.bs_last, k.vsize) == (40, 36, 2, "bmm", True, 4)
+    assert k.bias.shape == (36, 1)                                  # interface.py:186-189
+    assert KSLinear([(2, 3, 5, 4)], algo="dense", dtype=torch.float32).bias.shape == (24,)
+    assert [tuple(f.shape) for f in k.factors] == [(8, 3, 5), (6, 6, 4)]
+    assert "in_size=40, out_size=36, num_mat=2" in repr(k)
+
+
+@pytest.mark.parametrize("algo", ["dense", "bmm", "einsum"])
+@pytest.mark.parametrize("bs_last", [True, False])
+def test_kslinear_torch_algos_match_oracle(algo, bs_last):
+    from ksmm_amd import KSLinear
+
+    patterns = [(2, 3, 5, 4), (3, 6, 4, 2)]
+    ws = seeded_weights(patterns, seed=0)
+    x = seeded_input(40, 9, bs_last, seed=1)
+    k = KSLinear(patterns, weights=ws, bias=False, algo=algo, dtype=torch.float32, bs_last=bs_last)
+    y = k(x).detach().numpy()
+    z = O.chain_apply([w.double().numpy() for w in ws], x.double().numpy(), bs_last)
+    assert O.rel_fro_error(y, z) <= 1e-6
+    kd = k.get_dense_product().double().numpy()
+    assert abs(kd - O.chain_dense([w.double().numpy() for w in ws])).max() <= 1e-6
+
+
+def test_generate_factor_layouts_match_oracle():
+    from ksmm_amd import generate_factor
+
+    p = (2, 3, 5, 4)
+    (w4,) = seeded_weights([p], seed=2)
+    w = w4.numpy()
+    assert (generate_factor(*p, "kernel", w4, torch.float32).numpy() == O.pack_kernel_format(w)).all()
+    assert (generate_factor(*p, "bmm", w4, torch.float32).numpy() == O.pack_bmm_format(w)).all()
+    assert (generate_factor(*p, "dense", w4, torch.float32).numpy() == O.ks_dense(w)).all()
+    f = generate_factor(*p, "kernel", None, torch.float32)
+    assert f.shape == (40, 3) and f.abs().max() <= 1 / 5 ** 0.5
+
+
+def test_nd_input_and_bias_cpu():
+    from ksmm_amd import KSLinear
+
+    k = KSLinear([(2, 3, 5, 4)], algo="bmm", dtype=torch.float32, bs_last=False, bias=True)
+    x = torch.randn(4, 6, 40)
+    y = k(x)
+    assert y.shape == (4, 6, 24)
+    z = torch.nn.functional.linear(x, k.get_dense_product(), k.bias)
+    assert torch.allclose(y, z, atol=1e-5)
+    kl = KSLinear([(2, 3, 5, 4)], algo="einsum", dtype=torch.float32, bs_last=True, bias=True)
+    xl = torch.randn(40, 4, 6)
+    yl = kl(xl)
+    assert yl.shape == (24, 4, 6)
+    zl = (kl.get_dense_product() @ xl.reshape(40, -1) + kl.bias).reshape(24, 4, 6)
+    assert torch.allclose(yl, zl, atol=1e-5)
+
+
+def test_fp8_torch_algos_use_dequantised_operands():
+    from ksmm_amd import KSLinear, quantize_fp8
+
+    patterns = [(1, 16, 16, 4), (4, 16, 16, 1)]
+    ws = seeded_weights(patterns, seed=3, bound=0.25)
+    x = seeded_input(64, 11, True, seed=4)
+    k = KSLinear(patterns, weights=ws, bias=False, algo="dense", dtype=torch.float8_e4m3fn, bs_last=True)
+    y = k(x).detach().double().numpy()
+    wd = []
+    for w in ws:
+        q, s = O.fp8_quantize(w.numpy())
+        wd.append(O.fp8_dequantize(q, s).reshape(w.shape))
+    xq, xs = O.fp8_quantize(x.numpy())
+    z = O.chain_apply(wd, O.fp8_dequantize(xq, xs).reshape(x.shape), True)
+    assert O.rel_fro_error(y, z) <= 1e-6
+    q, s = quantize_fp8(x)
+    assert (q.view(torch.uint8).numpy() == xq).all() and abs(float(s) - float(xs)) < 1e-12
+
+
+def test_kernel_forward_host_checks():
+    from ksmm_amd import Kernel
+
+    x = torch.zeros(4, 8)
+    w = torch.zeros(8, 2)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):   # kernel.cpp:19
+        Kernel.forward(x, w, False, 1, 2, 8, 1)
