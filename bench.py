@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the KS hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all 0|1]
+
+A step is one forward pass of one KS factor over a batch of 25 088 columns.  The headline
+workload is BASELINE configuration 2: a single fp32 factor with pattern (1,48,48,16)
+(768 -> 768), batch-size-last.  The JSON line also carries every other configuration
+(µs per factor and per KSLinear, effective GB/s and TFLOP/s, fraction of the bounding
+roofline, parity error against the CPU oracle on sampled columns), the roofline record of
+the headline kernel and the CPU baseline (the reference's ``algo='bmm'`` algorithm restated
+with torch.bmm, timed on this host's cores).
+
+Inputs are synthetic (seeded), resident in HBM before the timed region.  To keep the 256 MB
+last-level cache from serving repeated launches, consecutive steps rotate through distinct
+input/output buffers whose total footprint exceeds 1 GB.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+BATCH = 25088
+SEED = 0
+FP8 = torch.float8_e4m3fn
+CONFIGS = [
+    # name, patterns, precision, bs_last, weight bound
+    ("C2_bs_last", [(1, 48, 48, 16)], "fp32", True, None),
+    ("C2_bs_first", [(1, 48, 48, 16)], "fp32", False, None),
+    ("C1_readme", [(6, 64, 64, 1), (1, 768, 192, 2)], "fp32", True, None),
+    ("C3_bs_last", [(4, 192, 192, 1)], "fp16", True, None),
+    ("C3_bs_first", [(4, 192, 192, 1)], "fp16", False, None),
+    ("C4_vit_b_up", [(12, 64, 64, 1), (1, 1536, 384, 2)], "fp16", False, None),
+    ("C5_butterfly", [(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], "fp8", True, 0.25),
+]
+DT = {"fp32": torch.float32, "fp16": torch.float16, "fp8": FP8}
+TOL = {"fp32": 1e-5, "fp16": 2e-3, "fp8": 5e-2}
+
+
+def make_weights(patterns, bound, gen):
+    out = []
+    for (a, b, c, d) in patterns:
+        s = bound if bound is not None else 1.0 / math.sqrt(c)
+        out.append((torch.rand(a, b, c, d, generator=gen) * 2 - 1) * s)
+    return out
+
+
+def time_launches(fn, n_sets, steps, warmup):
+    """Average seconds per call of fn(i) (i rotates over buffer sets).
+
+    The `steps` launches are captured once into a HIP graph on a side stream and replayed, so
+    that the timed region holds back-to-back kernels rather than Python launch overhead; HIP
+    events are recorded on the stream the graph (and hence every kernel) runs on, with a
+    device-wide synchronisation on both sides."""
+    for i in range(warmup):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(steps):
+                fn(i % n_sets)
+        graph.replay()  # untimed: first replay uploads the graph
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t0 = torch.cuda.Event(enable_timing=True)
+        t1 = torch.cuda.Event(enable_timing=True)
+        t0.record(stream)
+        graph.replay()
+        t1.record(stream)
+        stream.synchronize()
+    torch.cuda.synchronize()
+    return t0.elapsed_time(t1) / 1e3 / steps
+
+
+def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True):
+    """Per-factor and whole-chain timings of one configuration."""
+    from ksmm_amd import Kernel, generate_factor, quantize_fp8, query_tile
+    from ksmm_amd.roofline import factor_roofline, factor_work
+
+    gen = torch.Generator().manual_seed(SEED)
+    ws4 = make_weights(patterns, bound, gen)
+    in_size = patterns[0][0] * patterns[0][2] * patterns[0][3]
+    dt = DT[prec]
+    out_dt = torch.float16 if prec == "fp8" else dt
+    # enough rotating buffer sets to exceed the last-level cache several times over
+    widest = max([in_size] + [p[0] * p[1] * p[3] for p in patterns])
+    per_set = 2 * widest * BATCH * 4
+    n_sets = max(2, min(8, int(math.ceil(1.2e9 / per_set))))
+    xs, scales = [], []
+    for i in range(n_sets):
+        g = torch.Generator().manual_seed(SEED + 1 + i)
+        x = torch.randn(BATCH, in_size, generator=g)
+        x = x.t().contiguous() if bs_last else x
+        if prec == "fp8":
+            q, s = quantize_fp8(x)
+            xs.append(q.cuda())
+            scales.append(float(s))
+        else:
+            xs.append(x.to(dt).cuda())
+            scales.append(1.0)
+    facs, wscales = [], []
+    for p, w4 in zip(patterns, ws4):
+        if prec == "fp8":
+            q4, s = quantize_fp8(w4)
+            facs.append(generate_factor(*p, "kernel", q4.float(), FP8, "cuda"))
+            wscales.append(float(s))
+        else:
+            facs.append(generate_factor(*p, "kernel", w4, dt, "cuda"))
+            wscales.append(1.0)
+
+    result = {"name": name, "precision": prec, "bs_last": bs_last, "patterns": patterns, "factors": []}
+    # ---- per factor: input of factor i is the (precomputed) output of factor i-1 ----------
+    cur = xs
+    for i, p in enumerate(patterns):
+        a, b, c, d = p
+        out_size = a * b * d
+        shape = (out_size, BATCH) if bs_last else (BATCH, out_size)
+        outs = [torch.empty(shape, dtype=out_dt, device="cuda") for _ in range(n_sets)]
+        sc = [wscales[i] * (scales[j] if i == 0 else 1.0) for j in range(n_sets)]
+
+        def run(j, cur=cur, outs=outs, sc=sc, i=i, p=p):
+            Kernel.forward(cur[j], facs[i], bs_last, *p, scale=sc[j], out=outs[j])
+
+        sec = time_launches(run, n_sets, steps, warmup)
+        x_dt = cur[0].dtype
+        roof = factor_roofline(BATCH, p, x_dt, facs[i].dtype, out_dt, sec)
+        tile = query_tile(BATCH, p, x_dt, facs[i].dtype, bs_last)
+        result["factors"].append({
+            "pattern": p, "us": sec * 1e6, "gbs": roof["gbs"], "tflops": roof["tflops"],
+            "bound": roof["bound"], "roofline_frac": roof["frac"], "floor_us": roof["floor_us"],
+            "x_dtype": str(x_dt).replace("torch.", ""), "algo": tile["algo"], "variant": tile["variant"]})
+        cur = outs
+    # ---- whole KSLinear (chain launcher) ----------------------------------------------------
+    if len(patterns) > 1:
+        ws_bytes = torch.empty(2 * (widest * BATCH * 4 + 256), dtype=torch.uint8, device="cuda")
+
+        def run_chain(j):
+            sc = list(wscales)
+            sc[0] *= scales[j]
+            return Kernel.chain_forward(xs[j], facs, patterns, bs_last, scales=sc, workspace=ws_bytes)
+
+        sec = time_launches(run_chain, n_sets, max(3, steps // 2), max(1, warmup // 2))
+        result["kslinear_us"] = sec * 1e6
+        final = run_chain(0)
+    else:
+        result["kslinear_us"] = result["factors"][0]["us"]
+        final = cur[0]
+    # ---- parity on sampled batch columns ---------------------------------------------------
+    if check:
+        from oracle import ks_oracle as O
+        import numpy as np
+
+        cols = np.unique(np.concatenate([np.arange(0, BATCH, 197), np.arange(BATCH - 4, BATCH)]))
+        g = torch.Generator().manual_seed(SEED + 1)
+        x0 = torch.randn(BATCH, in_size, generator=g)
+        x0 = x0.t().contiguous() if bs_last else x0
+        if prec == "fp8":
+            xr = xs[0].cpu().to(torch.float32).double().numpy() * scales[0]
+            wr = [f.double().numpy() for f in
+                  [quantize_fp8(w)[0].to(torch.float32) * quantize_fp8(w)[1] for w in ws4]]
+        else:
+            xr = x0.to(dt).double().numpy()
+            wr = [w.to(dt).double().numpy() for w in ws4]
+        xsub = xr[:, cols] if bs_last else xr[cols, :]
+        z = O.chain_apply(wr, xsub, bs_last)
+        yh = final.float().cpu().numpy()
+        ysub = yh[:, cols] if bs_last else yh[cols, :]
+        result["rel_fro_error"] = O.rel_fro_error(ysub, z)
+        result["tolerance"] = TOL[prec]
+        result["parity_ok"] = bool(result["rel_fro_error"] <= TOL[prec])
+    return result
+
+
+def cpu_baseline(patterns, bs_last, budget_s=12.0):
+    """The reference's algo='bmm' CPU algorithm (restated in oracle/), fp32, on all host
+    cores; protocol of the reference's ksmm_time.py: blocked_autorange(min_run_time=0.25),
+    re-run with 11*max(mean, median) when fewer than 10 runs fit."""
+    import torch.utils.benchmark as tb
+    from oracle import ks_oracle as O
+
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count() or 1
+    cores = min(cores, os.cpu_count() or cores)
+    torch.set_num_threads(cores)
+    gen = torch.Generator().manual_seed(SEED)
+    ws4 = make_weights(patterns, None, gen)
+    wb = [torch.from_numpy(O.pack_bmm_format(w.numpy())) for w in ws4]
+    in_size = patterns[0][0] * patterns[0][2] * patterns[0][3]
+    x = torch.randn(BATCH, in_size, generator=gen)
+    x = x.t().contiguous() if bs_last else x
+    with torch.no_grad():
+        timer = tb.Timer(stmt="f(wb, x, patterns, bs_last)",
+                         globals={"f": O.torch_bmm_chain, "wb": wb, "x": x, "patterns": patterns,
+                                  "bs_last": bs_last}, num_threads=torch.get_num_threads())
+        m = timer.blocked_autorange(min_run_time=0.25)
+        if m.number_per_run <= 10:
+            m = timer.blocked_autorange(min_run_time=min(budget_s, 11 * max(m.mean, m.median)))
+    return {"value": m.median * 1e6, "unit": "us", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "full workload (B=%d, fp32, bs_last=%s, patterns=%s), %d timed calls of torch.bmm "
+                      "+ permute copies; median" % (BATCH, bs_last, patterns, len(m.times) * m.number_per_run),
+            "mean_us": m.mean * 1e6, "iqr_us": m.iqr * 1e6, "host_cpu_count": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--all", type=int, default=1, help="also time the other configurations")
+    ap.add_argument("--cpu", type=int, default=1, help="time the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build is single-GPU (the KS path shards on the batch axis without "
+              "communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from ksmm_amd import _lib
+    from ksmm_amd.roofline import factor_roofline
+
+    _lib.load()  # fails loudly if the HIP library is missing
+    t_start = time.time()
+    head = bench_config(*CONFIGS[0], steps=args.steps, warmup=args.warmup)
+    sec = head["factors"][0]["us"] / 1e6
+    roof = factor_roofline(BATCH, CONFIGS[0][1][0], torch.float32, torch.float32, torch.float32, sec)
+    others = []
+    if args.all:
+        for cfg in CONFIGS[1:]:
+            others.append(bench_config(*cfg, steps=max(20, args.steps // 2), warmup=max(5, args.warmup // 2)))
+    cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
+    line = {
+        "metric": "us_per_ks_factor", "value": head["factors"][0]["us"], "unit": "us",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seed %d): x~N(0,1), W~U(-1/sqrt(c),1/sqrt(c))" % SEED,
+        "config": {"workload": "single KS factor (1,48,48,16) 768->768, fp32, bs_last, B=25088",
+                   "batch": BATCH, "pattern": [1, 48, 48, 16], "layout": "bs_last"},
+        "roofline": {"bound": roof["bound"], "achieved": roof["achieved"], "peak": roof["peak"],
+                     "unit": roof["unit"], "frac": roof["frac"], "traffic": None},
+        "cpu_baseline": cpu,
+        "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),
+                   "ok": head.get("parity_ok")},
+        "configs": [head] + others,
+        "wall_s": time.time() - t_start,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
