@@ -178,7 +178,7 @@ def test_kernel_matches_dense_and_bmm_algos():
     for algo in ("kernel", "dense", "bmm", "einsum"):
         ksl = KSLinear(patterns, weights=ws4, bias=False, algo=algo, dtype=torch.float32,
                        bs_last=True, device="cuda")
-        ys[algo] = ksl(x).double().cpu().numpy()
+        ys[algo] = ksl(x).detach().double().cpu().numpy()
     for algo in ("dense", "bmm", "einsum"):
         assert O.rel_fro_error(ys["kernel"], ys[algo]) <= 1e-5, algo
 
