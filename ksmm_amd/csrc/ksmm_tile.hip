@@ -1,4 +1,409 @@
+// "Tile" family: LDS-staged MFMA kernel for b x c blocks that are real dense contractions.
+//
+// For one (a_i, d_i) block the factor is a GEMM  Y[b x B] = W[b x c] * X[c x B].  A workgroup
+// computes a TM (outputs) x TN (batch) tile, looping over c in slabs of TK that are staged in
+// LDS (double-buffered: the global loads of slab s+1 are in flight while slab s is multiplied).
+// 32x32 MFMA tiles with fp32 accumulation: v_mfma_f32_32x32x2_f32 for fp32,
+// v_mfma_f32_32x32x16_f16 for fp16 (e4m3fn operands are decoded to fp16 while they are
+// written to LDS, which is exact).
+//
+// Layout handling.  Both operands of a 16-bit MFMA want 8 consecutive k per lane.  The weight
+// is stored (c x b) with b contiguous and, batch-size-last, the input is (c x B) with B
+// contiguous: both "k-outer".  They are copied to LDS as they are and read back with
+// ds_read_b64_tr_b16, the gfx950 LDS transpose load (within 16 lanes, lane i receives
+// element i of each of the four 32-byte rows the group addresses).  Batch-size-first input
+// rows are already k-contiguous (d == 1) and are read with plain 16-byte LDS loads.  The
+// operand whose index runs along the contiguous output axis is the MFMA B operand, so that
+// the 32 lanes of a tile row store 32 consecutive elements:
+//   bs_last : A = W (rows = outputs), B = X (lanes = batch)    -> y[(.)*d*B + n]
+//   bs_first: A = X (rows = batch),   B = W (lanes = outputs)  -> y[n*out + (.)]
+//
+// Workgroup ids are remapped so that the workgroups that share an input tile (the TM-tiles of
+// one batch tile) run on the same XCD and hit the same L2.
+//
+// Reference counterpart: kernel_bs_{first,last}_{float,half2,half4}
+// (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-491,
+//  template_kernels_half.cuh:103-1092): same tiling idea (TILEX x TILEY output tile, TILEK
+// slabs, double-buffered shared memory) with scalar FMAs and fp16 accumulation for half.
 #include "ksmm_common.h"
+
 namespace ksmm {
-int tile_run(const Problem &, int, bool, ksmm_tile *) { return KSMM_ERR_BAD_ALGO; }
+
+namespace {
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+template <typename CT> struct compute;  // CT = element type held in LDS and fed to the MFMA
+template <> struct compute<float> {
+    static constexpr int KSTEP = 2;  // k per MFMA
+};
+template <> struct compute<half_t> {
+    static constexpr int KSTEP = 16;
+};
+
+// 16 bytes of global memory -> EPV elements of CT, written to LDS contiguously;
+// register-staged variant: load now, write to LDS later
+template <typename TS, typename CT> struct stage;
+template <> struct stage<float, float> {
+    static constexpr int EPV = 4;
+    uint4_t v;
+    __device__ __forceinline__ void load(const float *g) { v = *(const uint4_t *)g; }
+    __device__ __forceinline__ void store(float *l) const { *(uint4_t *)l = v; }
+};
+template <> struct stage<half_t, half_t> {
+    static constexpr int EPV = 8;
+    uint4_t v;
+    __device__ __forceinline__ void load(const half_t *g) { v = *(const uint4_t *)g; }
+    __device__ __forceinline__ void store(half_t *l) const { *(uint4_t *)l = v; }
+};
+template <> struct stage<fp8_t, half_t> {
+    static constexpr int EPV = 16;
+    uint4_t v;
+    __device__ __forceinline__ void load(const fp8_t *g) { v = *(const uint4_t *)g; }
+    __device__ __forceinline__ void store(half_t *l) const
+    {
+        uint4_t lo, hi;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            lo[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[i]));
+            lo[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[i] >> 16));
+            hi[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[2 + i]));
+            hi[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[2 + i] >> 16));
+        }
+        *(uint4_t *)l = lo;
+        *(uint4_t *)(l + 8) = hi;
+    }
+};
+
+// ---- MFMA fragment fetch from LDS ------------------------------------------------------------
+// K-outer storage S[k][idx] (row stride ld elements): lane (i = lane % 32, kq = lane / 32)
+template <typename CT> struct frag;
+template <> struct frag<float> {
+    typedef float type;
+    __device__ static __forceinline__ float k_outer(const float *s, int ld, int idx0, int k0, int lane)
+    {
+        return s[(k0 + (lane >> 5)) * ld + idx0 + (lane & 31)];
+    }
+    __device__ static __forceinline__ float k_inner(const float *s, int ld, int idx0, int k0, int lane)
+    {
+        return s[(idx0 + (lane & 31)) * ld + k0 + (lane >> 5)];
+    }
+    __device__ static __forceinline__ float16_t mfma(float a, float b, float16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct frag<half_t> {
+    typedef half8_t type;
+    __device__ static __forceinline__ half8_t k_outer(const half_t *s, int ld, int idx0, int k0, int lane)
+    {
+        // two transpose loads of 4 k each; a 16-lane group addresses 4 rows x 16 columns
+        const int kq = lane >> 5, i16 = lane & 15, half_sel = (lane >> 4) & 1;
+        const half_t *p = s + (k0 + 8 * kq + (i16 >> 2)) * ld + idx0 + 16 * half_sel + 4 * (i16 & 3);
+        typedef short4_t __attribute__((address_space(3))) * lds_ptr;
+        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * ld));
+        typedef short short8_t __attribute__((ext_vector_type(8)));
+        short8_t r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(half8_t, r);
+    }
+    __device__ static __forceinline__ half8_t k_inner(const half_t *s, int ld, int idx0, int k0, int lane)
+    {
+        return *(const half8_t *)(s + (idx0 + (lane & 31)) * ld + k0 + 8 * (lane >> 5));
+    }
+    __device__ static __forceinline__ float16_t mfma(half8_t a, half8_t b, float16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// LDS row paddings (elements): K-outer rows are read 32 consecutive elements at a time by
+// two or four row groups, K-inner rows by 16-byte pieces of 32 different rows.
+template <typename CT> struct pads;
+template <> struct pads<float> {
+    static constexpr int outer(int n) { return n + (((n % 64) == 32) ? 0 : ((96 - n % 64) % 64)); }
+    static constexpr int inner(int k) { return k + 4; }
+};
+template <> struct pads<half_t> {
+    static constexpr int outer(int n) { return n + ((((2 * n) % 128) == 32) ? 0 : (((160 - (2 * n) % 128) % 128) / 2)); }
+    static constexpr int inner(int k) { return k + 8; }
+};
+
+template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int TM, int TN, int TK,
+          int WM, int WN>
+struct TileCfg {
+    static constexpr int THREADS = 64 * WM * WN;
+    static constexpr int MT = TM / WM / 32, NT = TN / WN / 32;  // 32x32 MFMA tiles per wave
+    static constexpr int LDW = pads<CT>::outer(TM);
+    static constexpr int LDX = BS_LAST ? pads<CT>::outer(TN) : pads<CT>::inner(TK);
+    static constexpr int W_ELEMS = TK * LDW;
+    static constexpr int X_ELEMS = BS_LAST ? TK * LDX : TN * LDX;
+    static constexpr int LDS_BYTES = 2 * (W_ELEMS + X_ELEMS) * (int)sizeof(CT);
+    static constexpr int W_EPV = stage<TW, CT>::EPV, X_EPV = stage<TX, CT>::EPV;
+    static constexpr int W_VECS = TK * TM / W_EPV, X_VECS = TK * TN / X_EPV;
+    static constexpr int W_PER_T = (W_VECS + THREADS - 1) / THREADS, X_PER_T = (X_VECS + THREADS - 1) / THREADS;
+    static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0, "wave tiling");
+    static_assert(TK % compute<CT>::KSTEP == 0, "k slab");
+    static_assert(TM % W_EPV == 0 && (BS_LAST ? TN % X_EPV == 0 : TK % X_EPV == 0), "vector width");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int TM, int TN, int TK,
+          int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restrict__ x,
+                                                              const TW *__restrict__ w,
+                                                              TY *__restrict__ y, int batch, int a,
+                                                              int b, int c, int d, float scale,
+                                                              int m_tiles, int n_tiles, int blocks)
+{
+    typedef TileCfg<CT, TX, TW, TY, BS_LAST, TM, TN, TK, WM, WN> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    CT *const lds = (CT *)smem;
+    auto ws = [&](int buf) { return lds + buf * C::W_ELEMS; };
+    auto xs = [&](int buf) { return lds + 2 * C::W_ELEMS + buf * C::X_ELEMS; };
+
+    // XCD-aware id: hardware deals consecutive workgroup ids round-robin to the 8 XCDs; give
+    // each XCD a contiguous range of logical ids so that TM-tiles of one input tile share an L2.
+    const int per_xcd = (blocks + 7) / 8;
+    const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lid >= blocks) return;
+    const int mt_id = lid % m_tiles;
+    const int rest = lid / m_tiles;
+    const int nt_id = rest % n_tiles;
+    const int g = rest / n_tiles;  // a_i * d + d_i
+    const int a_i = g / d, d_i = g - a_i * d;
+    const int m0 = mt_id * TM, n0 = nt_id * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
+    const TW *wg = w + (size_t)g * c * b + m0;  // row k: + k * b
+    // x element (k, n): bs_last ((a_i*c + k)*d + d_i)*batch + n ; bs_first (d == 1) n*in + a_i*c + k
+    const TX *xg = BS_LAST ? x + ((size_t)a_i * c * d + d_i) * batch : x + (size_t)a_i * c;
+    const size_t x_kstride = BS_LAST ? (size_t)d * batch : 1;
+
+    stage<TW, CT> wreg[C::W_PER_T];
+    stage<TX, CT> xreg[C::X_PER_T];
+
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::W_VECS % C::THREADS == 0 || v < C::W_VECS) {
+                const int kk = v / (TM / C::W_EPV), mm = (v % (TM / C::W_EPV)) * C::W_EPV;
+                wreg[i].load(wg + (size_t)(k0 + kk) * b + mm);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                if (BS_LAST) {
+                    const int kk = v / (TN / C::X_EPV), nn = (v % (TN / C::X_EPV)) * C::X_EPV;
+                    // columns past the end are clamped to the last valid vector (never stored)
+                    const int col = min(n0 + nn, batch - C::X_EPV);
+                    xreg[i].load(xg + (size_t)(k0 + kk) * x_kstride + col);
+                } else {
+                    const int nn = v / (TK / C::X_EPV), kk = (v % (TK / C::X_EPV)) * C::X_EPV;
+                    const int row = min(n0 + nn, batch - 1);
+                    xreg[i].load(xg + (size_t)row * in_size + k0 + kk);
+                }
+            }
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::W_VECS % C::THREADS == 0 || v < C::W_VECS) {
+                const int kk = v / (TM / C::W_EPV), mm = (v % (TM / C::W_EPV)) * C::W_EPV;
+                wreg[i].store(ws(buf) + kk * C::LDW + mm);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                if (BS_LAST) {
+                    const int kk = v / (TN / C::X_EPV), nn = (v % (TN / C::X_EPV)) * C::X_EPV;
+                    xreg[i].store(xs(buf) + kk * C::LDX + nn);
+                } else {
+                    const int nn = v / (TK / C::X_EPV), kk = (v % (TK / C::X_EPV)) * C::X_EPV;
+                    xreg[i].store(xs(buf) + nn * C::LDX + kk);
+                }
+            }
+        }
+    };
+
+    float16_t acc[C::MT][C::NT];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const int steps = c / TK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int s = 0; s < steps; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < steps) gload((s + 1) * TK);
+        const CT *wb = ws(buf), *xb = xs(buf);
+#pragma unroll
+        for (int k0 = 0; k0 < TK; k0 += compute<CT>::KSTEP) {
+            typename frag<CT>::type fw[C::MT], fx[C::NT];
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+                fw[i] = frag<CT>::k_outer(wb, C::LDW, (wm * C::MT + i) * 32, k0, lane);
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+                fx[j] = BS_LAST ? frag<CT>::k_outer(xb, C::LDX, (wn * C::NT + j) * 32, k0, lane)
+                                : frag<CT>::k_inner(xb, C::LDX, (wn * C::NT + j) * 32, k0, lane);
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j)
+                    acc[i][j] = BS_LAST ? frag<CT>::mfma(fw[i], fx[j], acc[i][j])
+                                        : frag<CT>::mfma(fx[j], fw[i], acc[i][j]);
+        }
+        if (s + 1 < steps) lstore(buf ^ 1);
+        __syncthreads();
+    }
+
+    // D tile: lane holds column (lane % 32) of the B operand and rows 8*(e/4) + 4*(lane/32) + e%4
+    const int l32 = lane & 31, lq = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            const int mb = m0 + (wm * C::MT + i) * 32, nb = n0 + (wn * C::NT + j) * 32;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int rr = 8 * (e >> 2) + 4 * lq + (e & 3);
+                const float v = acc[i][j][e] * scale;
+                if (BS_LAST) {
+                    const int m = mb + rr, n = nb + l32;
+                    if (n < batch)
+                        elem<TY>::store(y + ((size_t)(a_i * b + m) * d + d_i) * batch + n, v);
+                } else {
+                    const int n = nb + rr, m = mb + l32;
+                    if (n < batch) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * b + m, v);
+                }
+            }
+        }
 }
+
+// ---- instance table -----------------------------------------------------------------------
+struct TileInst {
+    int combo, bs_last, tm, tn, tk, threads, lds;
+    const void *fn;
+};
+
+#define TILE_INST(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_)                          \
+    {COMBO_, BL_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                    \
+     TileCfg<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES,                           \
+     (const void *)ks_tile_kernel<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>}
+#define TILE_SET_F32(BL_)                                                                           \
+    TILE_INST(0, float, float, float, float, BL_, 128, 128, 16, 2, 2),                              \
+        TILE_INST(0, float, float, float, float, BL_, 64, 128, 16, 1, 4),                           \
+        TILE_INST(0, float, float, float, float, BL_, 32, 128, 16, 1, 4),                           \
+        TILE_INST(0, float, float, float, float, BL_, 64, 256, 16, 1, 4),                           \
+        TILE_INST(0, float, float, float, float, BL_, 128, 256, 16, 2, 2),                          \
+        TILE_INST(0, float, float, float, float, BL_, 96, 128, 16, 1, 4)
+#define TILE_SET_H(COMBO_, TX_, TW_, BL_)                                                           \
+    TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 128, 128, 32, 2, 2),                           \
+        TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 64, 128, 32, 1, 4),                        \
+        TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 32, 128, 32, 1, 4),                        \
+        TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 192, 128, 32, 2, 2),                       \
+        TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 128, 256, 32, 2, 2),                       \
+        TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 256, 256, 32, 2, 2),                       \
+        TILE_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 64, 256, 64, 1, 4)
+
+const TileInst tile_insts[] = {
+    TILE_SET_F32(true),
+    TILE_SET_F32(false),
+    TILE_SET_H(1, half_t, half_t, true),
+    TILE_SET_H(1, half_t, half_t, false),
+    TILE_SET_H(2, fp8_t, fp8_t, true),
+    TILE_SET_H(2, fp8_t, fp8_t, false),
+    TILE_SET_H(3, half_t, fp8_t, true),
+    TILE_SET_H(3, half_t, fp8_t, false),
+};
+constexpr int N_TILE_INSTS = sizeof(tile_insts) / sizeof(TileInst);
+
+bool tile_fits(const TileInst &t, const Problem &p, int combo)
+{
+    if (t.combo != combo || t.bs_last != p.bs_last) return false;
+    if (p.b % t.tm || p.c % t.tk) return false;
+    const int x_epv = 16 / (int)dtype_size(p.x_dtype), w_epv = 16 / (int)dtype_size(p.w_dtype);
+    // 16-byte global vectors: weight rows (b elements) and input rows must keep alignment
+    if (p.b % w_epv) return false;
+    if (p.bs_last) {
+        if (p.batch % x_epv || p.batch < x_epv) return false;
+    } else {
+        if (p.d != 1) return false;  // batch-size-first with d > 1 is not handled by this family
+        if (((int64_t)p.a * p.c) % x_epv || p.c % x_epv) return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
+{
+    const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
+    if (combo < 0) return KSMM_ERR_BAD_DTYPE;
+    int pick = -1;
+    if (variant >= 0) {
+        if (variant < N_TILE_INSTS && tile_fits(tile_insts[variant], p, combo)) pick = variant;
+    } else {
+        // heuristic: the largest TM that divides b (fewest re-reads of the input), then a batch
+        // tile that still leaves >= 2 workgroups per CU
+        int64_t best_score = -1;
+        for (int i = 0; i < N_TILE_INSTS; ++i) {
+            const TileInst &t = tile_insts[i];
+            if (!tile_fits(t, p, combo)) continue;
+            const int64_t wgs = (int64_t)p.a * p.d * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
+            int64_t score = (int64_t)t.tm * 1000 + t.tn;
+            if (wgs < 512) score -= 100000;
+            if (score > best_score) {
+                best_score = score;
+                pick = i;
+            }
+        }
+    }
+    if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    const TileInst &t = tile_insts[pick];
+    const int m_tiles = p.b / t.tm;
+    const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
+    const int64_t blocks = (int64_t)p.a * p.d * m_tiles * n_tiles;
+    const int64_t grid = (blocks + 7) / 8 * 8;
+    if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (tile) {
+        tile->algo = KSMM_ALGO_TILE;
+        tile->variant = pick;
+        tile->tile_m = t.tm;
+        tile->tile_n = t.tn;
+        tile->tile_k = t.tk;
+        tile->tile_d = 1;
+        tile->threads = t.threads;
+        tile->lds_bytes = t.lds;
+        tile->grid = grid;
+    }
+    if (!launch) return KSMM_OK;
+    if (t.lds > 64 * 1024) {
+        // opt in to more than 64 KB of dynamic LDS: a per-function attribute, set on every
+        // launch that needs it (idempotent, so there is no state to keep)
+        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
+            return KSMM_ERR_LAUNCH;
+    }
+    int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
+    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
+                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i};
+    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm

@@ -22,6 +22,8 @@
 // (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:297-491,
 //  template_kernels_half.cuh:629-826), which stage both operands in shared memory and use
 // scalar FMAs (and fp16 accumulation for half).
+#include <type_traits>
+
 #include "ksmm_common.h"
 
 namespace ksmm {
@@ -37,15 +39,13 @@ template <> struct hvec<8> { typedef half8_t type; };
 template <typename TX, int VEC> struct row_io;
 template <int VEC> struct row_io<half_t, VEC> {
     static constexpr int RAW = VEC / 2;  // dwords per row load
-    __device__ static __forceinline__ void load(const half_t *p, bool ok, uint32_t (&o)[RAW])
+    __device__ static __forceinline__ void load(const half_t *p, uint32_t (&o)[RAW])
     {
         if constexpr (VEC == 8) {
-            uint4_t v = {0, 0, 0, 0};
-            if (ok) v = *(const uint4_t *)p;
+            uint4_t v = *(const uint4_t *)p;
             o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
         } else {
-            uint2_t v = {0, 0};
-            if (ok) v = *(const uint2_t *)p;
+            uint2_t v = *(const uint2_t *)p;
             o[0] = v[0]; o[1] = v[1];
         }
     }
@@ -57,15 +57,13 @@ template <int VEC> struct row_io<half_t, VEC> {
 };
 template <int VEC> struct row_io<fp8_t, VEC> {
     static constexpr int RAW = VEC / 4;
-    __device__ static __forceinline__ void load(const fp8_t *p, bool ok, uint32_t (&o)[RAW])
+    __device__ static __forceinline__ void load(const fp8_t *p, uint32_t (&o)[RAW])
     {
         if constexpr (VEC == 16) {
-            uint4_t v = {0, 0, 0, 0};
-            if (ok) v = *(const uint4_t *)p;
+            uint4_t v = *(const uint4_t *)p;
             o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
         } else {
-            uint2_t v = {0, 0};
-            if (ok) v = *(const uint2_t *)p;
+            uint2_t v = *(const uint2_t *)p;
             o[0] = v[0]; o[1] = v[1];
         }
     }
@@ -104,8 +102,8 @@ template <> struct mfma16<8> {
 // fp32: v_mfma_f32_16x16x4_f32, VEC = 4 (16-byte loads and stores)
 // MT = b / 16, KS = c / 4.  Each wave iteration covers 64 batch columns.
 // ------------------------------------------------------------------------------------------
-template <int MT, int KS, bool PREFETCH>
-__global__ __launch_bounds__(256) void ks_wave_bl_f32(const float *__restrict__ x,
+template <int MT, int KS, int OCC>
+__global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restrict__ x,
                                                      const float *__restrict__ w,
                                                      float *__restrict__ y, int batch, int a, int b,
                                                      int c, int d, float scale, int n_slabs,
@@ -114,7 +112,7 @@ __global__ __launch_bounds__(256) void ks_wave_bl_f32(const float *__restrict__ 
     constexpr int VEC = 4, TN = 16 * VEC;
     const int lane = threadIdx.x & 63;
     const int q = lane >> 4, r = lane & 15;
-    const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     const int g = wave / n_slabs;  // block index a_i * d + d_i
     if (g >= a * d) return;
     const int slab = wave - g * n_slabs;
@@ -129,63 +127,80 @@ __global__ __launch_bounds__(256) void ks_wave_bl_f32(const float *__restrict__ 
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = wg[(4 * ks + q) * b + 16 * mt + r];
     }
-    const size_t row_stride = (size_t)d * batch;
-    const float *xg = x + ((size_t)a_i * c * d + d_i) * batch + (size_t)q * row_stride;
-    float *yg = y + ((size_t)a_i * b * d + d_i) * batch;
+    // Addressing: uniform (scalar) row base + one 32-bit per-lane byte offset, so that the
+    // loads and stores need no per-row vector address registers.  The host checks that the
+    // offsets fit in 32 bits.
+    const size_t row_stride = (size_t)d * batch;  // elements between consecutive c_i (or b_i)
+    const char *xg = (const char *)(x + ((size_t)a_i * c * d + d_i) * batch);
+    char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
+    const uint32_t x_lane = (uint32_t)(q * row_stride) * 4u;      // + column offset
+    const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 4u;  // + column offset
+    const int n_first = slab * iters * TN;                        // uniform
+    const int n_end = min(n_first + iters * TN, batch);           // uniform
+    const int last_vec = batch - VEC;
+    if (n_first >= n_end) return;
 
-    int n = slab * iters * TN + VEC * r;
-    float4_t xc[KS], xn[KS];
-    auto load_tile = [&](float4_t(&dst)[KS], int col) {
-        const bool ok = col < batch;
+    // Rolling register pipeline: xc[ks] holds input rows 4*ks + q of the current tile; as soon
+    // as the MFMAs of step ks are issued the same registers are refilled with the next tile's
+    // rows, so every load has a whole tile of matrix work to hide behind.  Columns past the
+    // end are clamped to the last valid vector (batch % VEC == 0) and never stored.
+    float4_t xc[KS];
+    auto col_off = [&](int n0) { return (uint32_t)min(n0 + VEC * r, last_vec) * 4u; };
+    {
+        const uint32_t off = x_lane + col_off(n_first);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (ok) v = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride + col);
-            dst[ks] = v;
-        }
-    };
-    load_tile(xc, n);
-    for (int it = 0; it < iters; ++it, n += TN) {
-        if (n - VEC * r >= batch) break;  // uniform across the wave
-        if (PREFETCH && it + 1 < iters) load_tile(xn, n + TN);
+        for (int ks = 0; ks < KS; ++ks)
+            xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + off);
+    }
+    // Everything issued so far (weights, first tile) is complete before the loop, so that the
+    // waits inside the loop only ever count that loop's own loads and stores.
+    __builtin_amdgcn_s_waitcnt(0);
+    const int n_last = n_first + ((n_end - n_first - 1) / TN) * TN;  // first column of the last tile
+    // FULL tiles store without a predicate, which keeps the loop body free of branches; a
+    // ragged last tile (batch not a multiple of the tile) runs once more with the predicate.
+    auto do_tile = [&](int n0, auto full) {
+        // the tile after the last one is the last one again (a cache hit that is not used)
+        const uint32_t next_off = x_lane + col_off(min(n0 + TN, n_last));
         float4_t acc[MT][VEC];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int v = 0; v < VEC; ++v) acc[mt][v] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+        for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     acc[mt][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[mt][ks], xc[ks][v],
                                                                       acc[mt][v], 0, 0, 0);
-        if (n < batch) {
+            xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + next_off);
+            __builtin_amdgcn_sched_barrier(0);  // keep the refill between the MFMA groups
+        }
+        const int col = n0 + VEC * r;
+        if (decltype(full)::value || col < batch) {
+            const uint32_t off = y_lane + (uint32_t)col * 4u;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float4_t o = {acc[mt][0][i] * scale, acc[mt][1][i] * scale,
                                   acc[mt][2][i] * scale, acc[mt][3][i] * scale};
-                    *(float4_t *)(yg + (size_t)(16 * mt + 4 * q + i) * row_stride + n) = o;
+                    *(float4_t *)(yg + (size_t)(16 * mt + i) * row_stride * 4 + off) = o;
                 }
         }
-        if (PREFETCH) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) xc[ks] = xn[ks];
-        } else if (it + 1 < iters) {
-            load_tile(xc, n + TN);
-        }
-    }
+    };
+    int n0 = n_first;
+    for (; n0 + TN <= n_end; n0 += TN) do_tile(n0, std::true_type{});
+    if (n0 < n_end) do_tile(n0, std::false_type{});
 }
 
 // ------------------------------------------------------------------------------------------
 // 16-bit MFMA path: x is fp16 or e4m3fn (decoded to fp16, exact), w is fp16 or e4m3fn,
 // y is fp16.  MT = b / 16, KS = c / (4 * KL).  Each wave iteration covers 16 * VEC columns.
 // ------------------------------------------------------------------------------------------
-template <typename TX, typename TW, int MT, int KS, int KL, int VEC, bool PREFETCH>
-__global__ __launch_bounds__(256) void ks_wave_bl_h(const TX *__restrict__ x,
+template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC>
+__global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ x,
                                                    const TW *__restrict__ w,
                                                    half_t *__restrict__ y, int batch, int a, int b,
                                                    int c, int d, float scale, int n_slabs, int iters)
@@ -194,7 +209,7 @@ __global__ __launch_bounds__(256) void ks_wave_bl_h(const TX *__restrict__ x,
     typedef typename hvec<KL>::type frag_t;
     const int lane = threadIdx.x & 63;
     const int q = lane >> 4, r = lane & 15;
-    const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     const int g = wave / n_slabs;
     if (g >= a * d) return;
     const int slab = wave - g * n_slabs;
@@ -212,53 +227,55 @@ __global__ __launch_bounds__(256) void ks_wave_bl_h(const TX *__restrict__ x,
                     areg[mt][ks][jj] =
                         (half_t)elem<TW>::load(wg + (KSTEP * ks + KL * q + jj) * b + 16 * mt + r);
     }
-    const size_t row_stride = (size_t)d * batch;
-    const TX *xg = x + ((size_t)a_i * c * d + d_i) * batch + (size_t)(KL * q) * row_stride;
-    half_t *yg = y + ((size_t)a_i * b * d + d_i) * batch;
-
     typedef row_io<TX, VEC> io;
-    struct raw_t {
-        uint32_t e[KS][KL][io::RAW];
-    };
-    struct tile_t {
-        uint32_t e[KS][KL][VEC / 2];  // fp16 pairs: columns (2i, 2i+1) of row (ks, jj)
-    };
-    int n = slab * iters * TN + VEC * r;
-    raw_t xn;
-    tile_t xc;
-    auto load_tile = [&](raw_t &dst, int col) {
-        const bool ok = col < batch;
+    const size_t row_stride = (size_t)d * batch;
+    const char *xg = (const char *)(x + ((size_t)a_i * c * d + d_i) * batch);
+    char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
+    const uint32_t x_lane = (uint32_t)(KL * q * row_stride) * (uint32_t)sizeof(TX);
+    const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 2u;
+    const int n_first = slab * iters * TN;
+    const int n_end = min(n_first + iters * TN, batch);
+    const int last_vec = batch - VEC;
+    if (n_first >= n_end) return;
+
+    // Rolling register pipeline as in the fp32 kernel: raw[ks][jj] holds VEC packed columns of
+    // input row KSTEP*ks + KL*q + jj; it is refilled for the next tile right after step ks.
+    uint32_t raw[KS][KL][io::RAW];
+    auto col_off = [&](int n0) { return (uint32_t)min(n0 + VEC * r, last_vec) * (uint32_t)sizeof(TX); };
+    {
+        const uint32_t off = x_lane + col_off(n_first);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
             for (int jj = 0; jj < KL; ++jj)
-                io::load(xg + (size_t)(KSTEP * ks + jj) * row_stride + col, ok, dst.e[ks][jj]);
-    };
-    auto unpack_tile = [&](const raw_t &src, tile_t &dst) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int jj = 0; jj < KL; ++jj) io::unpack(src.e[ks][jj], dst.e[ks][jj]);
-    };
-    load_tile(xn, n);
-    for (int it = 0; it < iters; ++it, n += TN) {
-        if (n - VEC * r >= batch) break;
-        unpack_tile(xn, xc);
-        if (PREFETCH && it + 1 < iters) load_tile(xn, n + TN);
+                io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + off),
+                         raw[ks][jj]);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    const int n_last = n_first + ((n_end - n_first - 1) / TN) * TN;
+    auto do_tile = [&](int n0, auto full) {
+        const uint32_t next_off = x_lane + col_off(min(n0 + TN, n_last));
         float4_t acc[MT][VEC];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int v = 0; v < VEC; ++v) acc[mt][v] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+        for (int ks = 0; ks < KS; ++ks) {
+            uint32_t xh[KL][VEC / 2];  // fp16 pairs: columns (2i, 2i+1) of row jj
+#pragma unroll
+            for (int jj = 0; jj < KL; ++jj) io::unpack(raw[ks][jj], xh[jj]);
+#pragma unroll
+            for (int jj = 0; jj < KL; ++jj)
+                io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + next_off),
+                         raw[ks][jj]);
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
                 // KL consecutive k of batch column VEC*r + v: in-register transpose
                 uint32_t bw[KL / 2];
 #pragma unroll
                 for (int pp = 0; pp < KL / 2; ++pp)
-                    bw[pp] = pick_pair(xc.e[ks][2 * pp][v / 2], xc.e[ks][2 * pp + 1][v / 2], v & 1);
+                    bw[pp] = pick_pair(xh[2 * pp][v / 2], xh[2 * pp + 1][v / 2], v & 1);
                 frag_t bf;
                 if constexpr (KL == 8)
                     bf = __builtin_bit_cast(frag_t, uint4_t{bw[0], bw[1], bw[2], bw[3]});
@@ -268,12 +285,16 @@ __global__ __launch_bounds__(256) void ks_wave_bl_h(const TX *__restrict__ x,
                 for (int mt = 0; mt < MT; ++mt)
                     acc[mt][v] = mfma16<KL>::run(areg[mt][ks], bf, acc[mt][v]);
             }
-        if (n < batch) {
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const int col = n0 + VEC * r;
+        if (decltype(full)::value || col < batch) {
+            const uint32_t off = y_lane + (uint32_t)col * 2u;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    half_t *dst = yg + (size_t)(16 * mt + 4 * q + i) * row_stride + n;
+                    half_t *dst = (half_t *)(yg + (size_t)(16 * mt + i) * row_stride * 2 + off);
                     constexpr int W = 8 < VEC ? 8 : VEC;  // halves per store (<= 16 bytes)
 #pragma unroll
                     for (int v0 = 0; v0 < VEC; v0 += W) {
@@ -284,13 +305,15 @@ __global__ __launch_bounds__(256) void ks_wave_bl_h(const TX *__restrict__ x,
                     }
                 }
         }
-        if (!PREFETCH && it + 1 < iters) load_tile(xn, n + TN);
-    }
+    };
+    int n0 = n_first;
+    for (; n0 + TN <= n_end; n0 += TN) do_tile(n0, std::true_type{});
+    if (n0 < n_end) do_tile(n0, std::false_type{});
 }
 
 // ---- instance table ---------------------------------------------------------------------
 struct WaveInst {
-    int b, c, vec, kl, prefetch;
+    int b, c, vec, kl, occ;
     const void *fn;
 };
 
@@ -298,35 +321,30 @@ typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int
 template <typename TX, typename TW>
 using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int, float, int, int);
 
-#define F32_INST(B_, C_, PF_) \
-    {B_, C_, 4, 1, PF_, (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, PF_>}
+// OCC_ = minimum waves per SIMD the register allocation must allow
+#define F32_INST(B_, C_, OCC_) \
+    {B_, C_, 4, 1, OCC_, (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_>}
 const WaveInst f32_insts[] = {
-    F32_INST(48, 48, true),  F32_INST(48, 48, false), F32_INST(64, 64, true), F32_INST(64, 64, false),
-    F32_INST(16, 16, true),  F32_INST(32, 32, true),
+    F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
+    F32_INST(16, 16, 4), F32_INST(32, 32, 3),
 };
 
-#define H_INST(TX_, TW_, B_, C_, KL_, VEC_, PF_)                            \
-    {B_, C_, VEC_, KL_, PF_,                                                \
-     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, PF_>}
-const WaveInst h_insts[] = {
-    H_INST(half_t, half_t, 64, 64, 8, 4, true),  H_INST(half_t, half_t, 64, 64, 8, 8, true),
-    H_INST(half_t, half_t, 64, 64, 8, 4, false), H_INST(half_t, half_t, 48, 48, 4, 4, true),
-    H_INST(half_t, half_t, 48, 48, 4, 8, true),  H_INST(half_t, half_t, 16, 16, 4, 8, true),
-    H_INST(half_t, half_t, 16, 16, 4, 4, true),  H_INST(half_t, half_t, 32, 32, 8, 8, true),
-    H_INST(half_t, half_t, 96, 96, 8, 4, false),
-};
-const WaveInst hq_insts[] = {
-    H_INST(half_t, fp8_t, 64, 64, 8, 4, true),  H_INST(half_t, fp8_t, 64, 64, 8, 8, true),
-    H_INST(half_t, fp8_t, 64, 64, 8, 4, false), H_INST(half_t, fp8_t, 48, 48, 4, 4, true),
-    H_INST(half_t, fp8_t, 48, 48, 4, 8, true),  H_INST(half_t, fp8_t, 16, 16, 4, 8, true),
-    H_INST(half_t, fp8_t, 16, 16, 4, 4, true),  H_INST(half_t, fp8_t, 32, 32, 8, 8, true),
-    H_INST(half_t, fp8_t, 96, 96, 8, 4, false),
-};
+#define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_)                           \
+    {B_, C_, VEC_, KL_, OCC_,                                               \
+     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_>}
+#define H_SET(TX_, TW_)                                                                      \
+    H_INST(TX_, TW_, 64, 64, 8, 4, 2), H_INST(TX_, TW_, 64, 64, 8, 8, 2),                    \
+        H_INST(TX_, TW_, 64, 64, 8, 8, 1), H_INST(TX_, TW_, 48, 48, 4, 4, 3),                \
+        H_INST(TX_, TW_, 48, 48, 4, 8, 2), H_INST(TX_, TW_, 16, 16, 4, 8, 4),                \
+        H_INST(TX_, TW_, 16, 16, 4, 4, 4), H_INST(TX_, TW_, 32, 32, 8, 8, 3),                \
+        H_INST(TX_, TW_, 96, 96, 8, 4, 1)
+const WaveInst h_insts[] = {H_SET(half_t, half_t)};
+const WaveInst hq_insts[] = {H_SET(half_t, fp8_t)};
 const WaveInst q_insts[] = {
-    H_INST(fp8_t, fp8_t, 64, 64, 8, 8, true),  H_INST(fp8_t, fp8_t, 64, 64, 8, 8, false),
-    H_INST(fp8_t, fp8_t, 48, 48, 4, 8, true),  H_INST(fp8_t, fp8_t, 16, 16, 4, 16, true),
-    H_INST(fp8_t, fp8_t, 16, 16, 4, 8, true),  H_INST(fp8_t, fp8_t, 32, 32, 8, 16, true),
-    H_INST(fp8_t, fp8_t, 32, 32, 8, 8, true),
+    H_INST(fp8_t, fp8_t, 64, 64, 8, 8, 2),  H_INST(fp8_t, fp8_t, 64, 64, 8, 8, 1),
+    H_INST(fp8_t, fp8_t, 48, 48, 4, 8, 2),  H_INST(fp8_t, fp8_t, 16, 16, 4, 16, 3),
+    H_INST(fp8_t, fp8_t, 16, 16, 4, 8, 4),  H_INST(fp8_t, fp8_t, 32, 32, 8, 16, 2),
+    H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),
 };
 
 }  // namespace
@@ -359,6 +377,8 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
     const WaveInst &in = insts[pick];
+    // per-lane byte offsets (up to 4*KL rows of d*batch elements plus one row) must fit in 32 bits
+    if ((int64_t)(4 * in.kl + 1) * p.d * p.batch * 4 >= 0xffffffffLL) return KSMM_ERR_BAD_ALGO;
     const int tn = 16 * in.vec;
     const int64_t n_tiles = (p.batch + tn - 1) / tn;
     // columns per wave: enough wave-iterations to amortise the weight load, while keeping
