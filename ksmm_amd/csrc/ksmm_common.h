@@ -91,5 +91,6 @@ static inline int combo_of(int xd, int wd, int yd)
 int generic_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
+int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 
 }  // namespace ksmm

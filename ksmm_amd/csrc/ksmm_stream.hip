@@ -1,0 +1,378 @@
+// "Stream" kernels of the tile family: the bandwidth-bound path for mid-sized b x c blocks.
+//
+// A persistent workgroup owns one (a_i, d_i) block and an equal share of the batch columns.
+// The b x c weight block is staged through LDS once and then lives in registers as MFMA
+// operands.  Input tiles (the whole c extent x TN batch columns) are brought in with
+// direct-to-LDS loads (global_load_lds_dwordx4: no staging registers), ST tiles deep, so that
+// a CU keeps ~100 KB of HBM reads in flight: enough to cover the memory latency at 8 TB/s
+// with one workgroup per CU.  The output tile is transposed through LDS and written with
+// 16-byte stores along the contiguous axis.
+//
+// Direct-to-LDS loads write 64 consecutive 16-byte chunks per wave instruction, so tiles are
+// stored without row padding; bank conflicts are avoided with an XOR swizzle of the chunk
+// index by the row index instead (the swizzle is applied to the *global* address each lane
+// fetches, and again by the MFMA operand reads).
+//
+// The loads are issued from inline assembly and tracked by hand: the kernel waits with
+// s_waitcnt vmcnt(N) where N is the number of vector-memory instructions issued after the
+// loads of the tile it is about to read (the counter retires in order).  The loop issues the
+// same number of loads (L) and stores (S) per iteration in every wave, which makes N a
+// compile-time constant.
+//
+// MFMA roles: the axis that is contiguous in the output runs along the MFMA *rows*, so that a
+// lane holds 4 consecutive output elements and the LDS transpose takes 8/16-byte writes:
+//   bs_last : A = X (rows = batch),   B = W (lanes = outputs)
+//   bs_first: A = W (rows = outputs), B = X (lanes = batch)      (d == 1)
+//
+// Reference counterpart: kernel_bs_{first,last}_{float,half2,half4}
+// (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-491,
+//  template_kernels_half.cuh:103-1092).
+#include "ksmm_mfma.h"
+
+namespace ksmm {
+
+namespace {
+
+// s_waitcnt immediate for gfx9-family encodings: vmcnt in bits [3:0] and [15:14], expcnt and
+// lgkmcnt left at their maxima (no wait)
+constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | (((n >> 4) & 3) << 14); }
+
+// one direct-to-LDS load: lane i of the wave writes its 16 bytes to lds_addr + 16 * i
+__device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+template <typename CT, typename TW, bool BS_LAST, int BB, int CC, int TN, int WM, int WN, int ST>
+struct StreamCfg {
+    static constexpr int THREADS = 64 * WM * WN;
+    static constexpr int ES = (int)sizeof(CT);
+    static constexpr int EPC = 16 / ES;  // elements per 16-byte chunk
+    static constexpr int KSTEP = compute<CT>::KSTEP;
+    static constexpr int MT = BB / WM / 32, NT = TN / WN / 32, KS = CC / KSTEP;
+    // input stage: bs_last CC rows of TN elements (k-outer); bs_first TN rows of CC (k-inner)
+    static constexpr int X_ROWS = BS_LAST ? CC : TN, X_COLS = BS_LAST ? TN : CC;
+    static constexpr int X_CPR = X_COLS / EPC;
+    static constexpr int X_CHUNKS = X_ROWS * X_CPR, L = X_CHUNKS / THREADS;
+    static constexpr int X_STAGE_BYTES = X_CHUNKS * 16;
+    // output tile: bs_last BB rows of TN; bs_first TN rows of BB; rows padded by one chunk
+    static constexpr int O_ROWS = BS_LAST ? BB : TN, O_COLS = BS_LAST ? TN : BB;
+    static constexpr int O_CPR = O_COLS / EPC, O_LD = O_COLS + EPC;
+    static constexpr int O_CHUNKS = O_ROWS * O_CPR, S = O_CHUNKS / THREADS;
+    static constexpr int O_BYTES = O_ROWS * O_LD * ES;
+    static constexpr int LDW = pads<CT>::outer(BB);
+    static constexpr int W_BYTES = CC * LDW * ES;
+    static constexpr int W_EPV = stage<TW, CT>::EPV, W_VECS = CC * BB / W_EPV;
+    static constexpr int PIPE_BYTES = ST * X_STAGE_BYTES + O_BYTES;
+    static constexpr int LDS_BYTES = W_BYTES > PIPE_BYTES ? W_BYTES : PIPE_BYTES;
+    // vector-memory instructions issued after the loads of the tile being waited for
+    static constexpr int N_SAFE = (ST - 1) * L;             // while fewer than ST-1 tiles were stored
+    static constexpr int N_FULL = (ST - 1) * (L + S);       // steady state
+    static_assert(BB % (32 * WM) == 0 && TN % (32 * WN) == 0 && CC % KSTEP == 0, "wave tiling");
+    static_assert(X_CHUNKS % THREADS == 0 && O_CHUNKS % THREADS == 0, "every wave issues L loads and S stores");
+    static_assert(X_CPR % (ES == 2 ? 8 : (BS_LAST ? 16 : 8)) == 0, "swizzle group");
+    static_assert(N_FULL <= 63, "vmcnt range");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+    static_assert(BB % W_EPV == 0, "weight vectors");
+};
+
+// swizzle of the 16-byte chunk index inside a row of the input stage
+template <typename CT, bool BS_LAST> __device__ __forceinline__ int swz(int row)
+{
+    if (BS_LAST) return sizeof(CT) == 2 ? 2 * (row & 3) : 8 * (row & 1);
+    return row & 7;
+}
+
+// MFMA operand of the input from a swizzled stage
+template <typename CT, bool BS_LAST, int X_COLS> struct xfrag;
+template <int X_COLS> struct xfrag<half_t, true, X_COLS> {  // k-outer, transpose loads
+    __device__ static __forceinline__ half8_t get(const half_t *s, int idx0, int k0, int lane)
+    {
+        const int kq = lane >> 5, i16 = lane & 15, hs = (lane >> 4) & 1;
+        const int row = k0 + 8 * kq + (i16 >> 2);  // + 4 for the second load: same row & 3
+        const int chunk = (idx0 >> 3) + 2 * hs + ((i16 & 3) >> 1);
+        const int off = ((chunk ^ (2 * ((i16 >> 2) & 3))) << 3) + 4 * (i16 & 1);
+        typedef short4_t __attribute__((address_space(3))) * lds_ptr;
+        const half_t *p = s + row * X_COLS + off;
+        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * X_COLS));
+        typedef short short8_t __attribute__((ext_vector_type(8)));
+        short8_t r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(half8_t, r);
+    }
+};
+template <int X_COLS> struct xfrag<half_t, false, X_COLS> {  // k-inner, 16-byte loads
+    __device__ static __forceinline__ half8_t get(const half_t *s, int idx0, int k0, int lane)
+    {
+        const int row = idx0 + (lane & 31);
+        const int chunk = (k0 >> 3) + (lane >> 5);
+        return *(const half8_t *)(s + row * X_COLS + ((chunk ^ (row & 7)) << 3));
+    }
+};
+template <int X_COLS> struct xfrag<float, true, X_COLS> {  // k-outer, 4-byte loads
+    __device__ static __forceinline__ float get(const float *s, int idx0, int k0, int lane)
+    {
+        const int row = k0 + (lane >> 5), col = idx0 + (lane & 31);
+        return s[row * X_COLS + ((((col >> 2) ^ (8 * (row & 1))) << 2) | (col & 3))];
+    }
+};
+
+template <typename CT, typename TW, typename TY, bool BS_LAST, int BB, int CC, int TN, int WM, int WN,
+          int ST>
+__global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__restrict__ x,
+                                                                const TW *__restrict__ w,
+                                                                TY *__restrict__ y, int batch, int a,
+                                                                int d, float scale, int wgs_per_group,
+                                                                int share)
+{
+    typedef StreamCfg<CT, TW, BS_LAST, BB, CC, TN, WM, WN, ST> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int g = blockIdx.x / wgs_per_group;  // a_i * d + d_i
+    const int s = blockIdx.x - g * wgs_per_group;
+    const int c_begin = s * share, c_end = min(batch, c_begin + share);  // this workgroup's columns
+    if (c_begin >= c_end) return;
+    const int a_i = g / d, d_i = g - a_i * d;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
+
+    // ---- weights: global -> LDS (as stored, c x b, padded rows) -> registers ---------------
+    {
+        CT *wl = (CT *)smem;
+        const TW *wg = w + (size_t)g * CC * BB;
+        for (int v = tid; v < C::W_VECS; v += C::THREADS) {
+            const int kk = v / (BB / C::W_EPV), mm = (v % (BB / C::W_EPV)) * C::W_EPV;
+            stage<TW, CT> r;
+            r.load(wg + (size_t)kk * BB + mm);
+            r.store(wl + kk * C::LDW + mm);
+        }
+        __syncthreads();
+    }
+    typename frag<CT>::type wreg[C::MT][C::KS];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+            wreg[i][ks] = frag<CT>::k_outer((const CT *)smem, C::LDW, (wm * C::MT + i) * 32, ks * C::KSTEP, lane);
+    __syncthreads();  // LDS is reused for the input stages and the output tile from here on
+
+    // ---- direct-to-LDS loads of one input tile ---------------------------------------------
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const CT *xg = BS_LAST ? x + ((size_t)a_i * CC * d + d_i) * batch : x + (size_t)a_i * CC;
+    const size_t x_kstride = (size_t)d * batch;
+    // per-lane part of the global address of load i: fixed over tiles except for the column/row base
+    size_t goff[C::L];  // element offset relative to (xg + tile base)
+    int gcol[C::L];     // bs_last: column inside the tile; bs_first: row inside the tile
+#pragma unroll
+    for (int i = 0; i < C::L; ++i) {
+        const int q = tid + i * C::THREADS;
+        const int row = q / C::X_CPR, pc = q % C::X_CPR;
+        const int col = (pc ^ swz<CT, BS_LAST>(row)) * C::EPC;  // logical column of this chunk
+        if (BS_LAST) {
+            goff[i] = (size_t)row * x_kstride;
+            gcol[i] = col;
+        } else {
+            goff[i] = (size_t)col;
+            gcol[i] = row;
+        }
+    }
+    auto issue = [&](int n0, int stg) {
+        const uint32_t dst = lds_base + stg * C::X_STAGE_BYTES + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < C::L; ++i) {
+            const CT *p;
+            if (BS_LAST)
+                p = xg + goff[i] + min(n0 + gcol[i], c_end - C::EPC);  // clamped: never past the share
+            else
+                p = xg + (size_t)min(n0 + gcol[i], c_end - 1) * in_size + goff[i];
+            dma16(p, dst + i * (C::THREADS * 16));
+        }
+    };
+
+    CT *const out = (CT *)(smem + ST * C::X_STAGE_BYTES);
+    const int l32 = lane & 31, lq = lane >> 5;
+    const int n_iters = (c_end - c_begin + TN - 1) / TN;
+    // prologue: ST-1 tiles in flight (tiles past the end repeat the last one; never read)
+#pragma unroll
+    for (int p = 0; p < ST - 1; ++p) issue(c_begin + min(p, n_iters - 1) * TN, p);
+
+    for (int it = 0; it < n_iters; ++it) {
+        const int n0 = c_begin + it * TN;
+        issue(c_begin + min(it + ST - 1, n_iters - 1) * TN, (it + ST - 1) % ST);
+        if (it >= ST - 1)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_FULL));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_SAFE));
+        __syncthreads();  // tile `it` has landed for every wave
+
+        const CT *xb = (const CT *)(smem + (it % ST) * C::X_STAGE_BYTES);
+        float16_t acc[C::MT][C::NT];
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks) {
+            typename frag<CT>::type fx[C::NT];
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+                fx[j] = xfrag<CT, BS_LAST, C::X_COLS>::get(xb, (wn * C::NT + j) * 32, ks * C::KSTEP, lane);
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j)
+                    acc[i][j] = BS_LAST ? frag<CT>::mfma(fx[j], wreg[i][ks], acc[i][j])
+                                        : frag<CT>::mfma(wreg[i][ks], fx[j], acc[i][j]);
+        }
+        // ---- accumulators -> LDS output tile: out[lane index][4 consecutive row indices] ----
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j) {
+                const int mb = (wm * C::MT + i) * 32, nb = (wn * C::NT + j) * 32;
+                // bs_last: rows = batch, lanes = outputs -> out[m][n..n+3]
+                // bs_first: rows = outputs, lanes = batch -> out[n][m..m+3]
+                const int orow = (BS_LAST ? mb : nb) + l32;
+                const int ocol0 = (BS_LAST ? nb : mb) + 4 * lq;
+#pragma unroll
+                for (int eg = 0; eg < 4; ++eg) {
+                    CT *dst = out + orow * C::O_LD + ocol0 + 8 * eg;
+                    if constexpr (sizeof(CT) == 2) {
+                        half4_t hv = {(half_t)(acc[i][j][4 * eg] * scale), (half_t)(acc[i][j][4 * eg + 1] * scale),
+                                      (half_t)(acc[i][j][4 * eg + 2] * scale), (half_t)(acc[i][j][4 * eg + 3] * scale)};
+                        *(half4_t *)dst = hv;
+                    } else {
+                        float4_t fv = {acc[i][j][4 * eg] * scale, acc[i][j][4 * eg + 1] * scale,
+                                       acc[i][j][4 * eg + 2] * scale, acc[i][j][4 * eg + 3] * scale};
+                        *(float4_t *)dst = fv;
+                    }
+                }
+            }
+        __syncthreads();
+        // ---- LDS output tile -> global, 16 bytes per lane along the contiguous axis --------
+#pragma unroll
+        for (int i = 0; i < C::S; ++i) {
+            const int q = tid + i * C::THREADS;
+            const int orow = q / C::O_CPR, oc = (q % C::O_CPR) * C::EPC;
+            const uint4_t v = *(const uint4_t *)(out + orow * C::O_LD + oc);
+            // the store is issued by every wave in every iteration (vmcnt bookkeeping); lanes
+            // outside the share are masked off
+            if (BS_LAST) {
+                const int n = n0 + oc;
+                TY *dst = y + ((size_t)(a_i * BB + orow) * d + d_i) * batch + min(n, c_end - C::EPC);
+                if (n < c_end) *(uint4_t *)dst = v;
+            } else {
+                const int n = n0 + orow;
+                TY *dst = y + (size_t)min(n, c_end - 1) * out_size + (size_t)a_i * BB + oc;
+                if (n < c_end) *(uint4_t *)dst = v;
+            }
+        }
+    }
+    // direct-to-LDS loads of the repeated last tile may still be in flight: they must land
+    // before this workgroup's LDS is handed to another one
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+}
+
+struct StreamInst {
+    int combo, bs_last, bb, cc, tn, threads, lds, epc;
+    const void *fn;
+};
+#define STREAM_INST(COMBO_, CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_)                              \
+    {COMBO_, BL_, BB_, CC_, TN_, 64 * WM_ * WN_,                                                     \
+     StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::LDS_BYTES,                               \
+     StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::EPC,                                     \
+     (const void *)ks_stream_kernel<CT_, TW_, CT_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>}
+#define STREAM_SET_H(COMBO_, TW_)                                                                     \
+    STREAM_INST(COMBO_, half_t, TW_, true, 192, 192, 64, 2, 2, 4),                                   \
+        STREAM_INST(COMBO_, half_t, TW_, false, 192, 192, 64, 2, 2, 4),                              \
+        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 128, 1, 4, 5),                                \
+        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 128, 1, 4, 5),                               \
+        STREAM_INST(COMBO_, half_t, TW_, true, 128, 128, 64, 2, 2, 4),                               \
+        STREAM_INST(COMBO_, half_t, TW_, false, 128, 128, 64, 2, 2, 4),                              \
+        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 64, 1, 2, 6),                                 \
+        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 64, 1, 2, 6)
+const StreamInst stream_insts[] = {
+    STREAM_SET_H(1, half_t),
+    STREAM_SET_H(3, fp8_t),
+    STREAM_INST(0, float, float, true, 64, 64, 64, 1, 2, 4),
+    STREAM_INST(0, float, float, true, 64, 64, 128, 1, 4, 3),
+    STREAM_INST(0, float, float, true, 128, 128, 64, 2, 2, 3),
+};
+constexpr int N_STREAM_INSTS = sizeof(stream_insts) / sizeof(StreamInst);
+
+bool stream_fits(const StreamInst &t, const Problem &p, int combo)
+{
+    if (t.combo != combo || t.bs_last != p.bs_last) return false;
+    if (p.b != t.bb || p.c != t.cc) return false;
+    // every global access is a 16-byte vector along the contiguous axis
+    if (p.bs_last) {
+        if (p.batch % t.epc) return false;
+    } else {
+        if (p.d != 1) return false;
+        if (((int64_t)p.a * p.c) % t.epc || ((int64_t)p.a * p.b) % t.epc) return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+// variant: bits 0-6 instance (0x7f: first that fits), bits 7.. workgroups per group (0: heuristic)
+int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
+{
+    const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
+    const int want = variant < 0 ? 0x7f : (variant & 0x7f);
+    int64_t wgs = variant < 0 ? 0 : (variant >> 7);
+    int pick = -1;
+    for (int i = 0; i < N_STREAM_INSTS; ++i) {
+        if (want != 0x7f && want != i) continue;
+        if (stream_fits(stream_insts[i], p, combo)) {
+            pick = i;
+            break;
+        }
+    }
+    if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    const StreamInst &t = stream_insts[pick];
+    const int64_t groups = (int64_t)p.a * p.d;
+    // bs_last shares are column ranges (multiples of the 16-byte vector), bs_first shares are rows
+    const int unit = p.bs_last ? t.epc : 1;
+    const int64_t units = p.batch / unit;
+    if (wgs <= 0) {
+        const int per_cu = t.lds * 2 <= 160 * 1024 ? 2 : 1;
+        wgs = (256 * per_cu + groups - 1) / groups;
+    }
+    if (wgs > units) wgs = units;
+    if (wgs < 1) wgs = 1;
+    const int64_t share = (units + wgs - 1) / wgs * unit;
+    wgs = (p.batch + share - 1) / share;
+    const int64_t grid = groups * wgs;
+    if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (tile) {
+        tile->algo = KSMM_ALGO_TILE;
+        tile->variant = 2000 + pick;
+        tile->tile_m = t.bb;
+        tile->tile_n = t.tn;
+        tile->tile_k = t.cc;
+        tile->tile_d = 1;
+        tile->threads = t.threads;
+        tile->lds_bytes = t.lds;
+        tile->grid = grid;
+    }
+    if (!launch) return KSMM_OK;
+    if (t.lds > 64 * 1024) {
+        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
+            return KSMM_ERR_LAUNCH;
+    }
+    int batch_i = (int)p.batch, wgs_i = (int)wgs, share_i = (int)share;
+    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
+                    (void *)&p.scale, &wgs_i, &share_i};
+    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm

@@ -25,109 +25,11 @@
 // (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-491,
 //  template_kernels_half.cuh:103-1092): same tiling idea (TILEX x TILEY output tile, TILEK
 // slabs, double-buffered shared memory) with scalar FMAs and fp16 accumulation for half.
-#include "ksmm_common.h"
+#include "ksmm_mfma.h"
 
 namespace ksmm {
 
 namespace {
-
-typedef short short4_t __attribute__((ext_vector_type(4)));
-
-template <typename CT> struct compute;  // CT = element type held in LDS and fed to the MFMA
-template <> struct compute<float> {
-    static constexpr int KSTEP = 2;  // k per MFMA
-};
-template <> struct compute<half_t> {
-    static constexpr int KSTEP = 16;
-};
-
-// 16 bytes of global memory -> EPV elements of CT, written to LDS contiguously;
-// register-staged variant: load now, write to LDS later
-template <typename TS, typename CT> struct stage;
-template <> struct stage<float, float> {
-    static constexpr int EPV = 4;
-    uint4_t v;
-    __device__ __forceinline__ void load(const float *g) { v = *(const uint4_t *)g; }
-    __device__ __forceinline__ void store(float *l) const { *(uint4_t *)l = v; }
-};
-template <> struct stage<half_t, half_t> {
-    static constexpr int EPV = 8;
-    uint4_t v;
-    __device__ __forceinline__ void load(const half_t *g) { v = *(const uint4_t *)g; }
-    __device__ __forceinline__ void store(half_t *l) const { *(uint4_t *)l = v; }
-};
-template <> struct stage<fp8_t, half_t> {
-    static constexpr int EPV = 16;
-    uint4_t v;
-    __device__ __forceinline__ void load(const fp8_t *g) { v = *(const uint4_t *)g; }
-    __device__ __forceinline__ void store(half_t *l) const
-    {
-        uint4_t lo, hi;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            lo[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[i]));
-            lo[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[i] >> 16));
-            hi[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[2 + i]));
-            hi[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[2 + i] >> 16));
-        }
-        *(uint4_t *)l = lo;
-        *(uint4_t *)(l + 8) = hi;
-    }
-};
-
-// ---- MFMA fragment fetch from LDS ------------------------------------------------------------
-// K-outer storage S[k][idx] (row stride ld elements): lane (i = lane % 32, kq = lane / 32)
-template <typename CT> struct frag;
-template <> struct frag<float> {
-    typedef float type;
-    __device__ static __forceinline__ float k_outer(const float *s, int ld, int idx0, int k0, int lane)
-    {
-        return s[(k0 + (lane >> 5)) * ld + idx0 + (lane & 31)];
-    }
-    __device__ static __forceinline__ float k_inner(const float *s, int ld, int idx0, int k0, int lane)
-    {
-        return s[(idx0 + (lane & 31)) * ld + k0 + (lane >> 5)];
-    }
-    __device__ static __forceinline__ float16_t mfma(float a, float b, float16_t c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct frag<half_t> {
-    typedef half8_t type;
-    __device__ static __forceinline__ half8_t k_outer(const half_t *s, int ld, int idx0, int k0, int lane)
-    {
-        // two transpose loads of 4 k each; a 16-lane group addresses 4 rows x 16 columns
-        const int kq = lane >> 5, i16 = lane & 15, half_sel = (lane >> 4) & 1;
-        const half_t *p = s + (k0 + 8 * kq + (i16 >> 2)) * ld + idx0 + 16 * half_sel + 4 * (i16 & 3);
-        typedef short4_t __attribute__((address_space(3))) * lds_ptr;
-        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
-        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * ld));
-        typedef short short8_t __attribute__((ext_vector_type(8)));
-        short8_t r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        return __builtin_bit_cast(half8_t, r);
-    }
-    __device__ static __forceinline__ half8_t k_inner(const half_t *s, int ld, int idx0, int k0, int lane)
-    {
-        return *(const half8_t *)(s + (idx0 + (lane & 31)) * ld + k0 + 8 * (lane >> 5));
-    }
-    __device__ static __forceinline__ float16_t mfma(half8_t a, half8_t b, float16_t c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
-
-// LDS row paddings (elements): K-outer rows are read 32 consecutive elements at a time by
-// two or four row groups, K-inner rows by 16-byte pieces of 32 different rows.
-template <typename CT> struct pads;
-template <> struct pads<float> {
-    static constexpr int outer(int n) { return n + (((n % 64) == 32) ? 0 : ((96 - n % 64) % 64)); }
-    static constexpr int inner(int k) { return k + 4; }
-};
-template <> struct pads<half_t> {
-    static constexpr int outer(int n) { return n + ((((2 * n) % 128) == 32) ? 0 : (((160 - (2 * n) % 128) % 128) / 2)); }
-    static constexpr int inner(int k) { return k + 8; }
-};
 
 template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int TM, int TN, int TK,
           int WM, int WN>
@@ -295,6 +197,260 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
         }
 }
 
+// ------------------------------------------------------------------------------------------
+// Weight-stationary variant for mid-sized blocks (b*c elements fit the register file of one
+// workgroup): a persistent workgroup owns one (a_i, d_i) block and a contiguous range of batch
+// tiles.  The b x c weight block is staged through LDS once and kept in registers as MFMA
+// operands (split over WM waves); after that LDS only holds input tiles with the whole c
+// extent, double-buffered across batch tiles, so that the HBM loads of tile t+1 are in flight
+// while tile t is multiplied and stored.  This is the bandwidth-bound regime: per tile the
+// matrix cores need a fraction of the time HBM needs.
+// ------------------------------------------------------------------------------------------
+template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int BB, int CC, int TN,
+          int WM, int WN>
+struct WsCfg {
+    static constexpr int THREADS = 64 * WM * WN;
+    static constexpr int KSTEP = compute<CT>::KSTEP;
+    static constexpr int MT = BB / WM / 32, NT = TN / WN / 32, KS = CC / KSTEP;
+    static constexpr int LDW = pads<CT>::outer(BB);
+    static constexpr int LDX = BS_LAST ? pads<CT>::outer(TN) : pads<CT>::inner(CC);
+    static constexpr int W_ELEMS = CC * LDW;
+    static constexpr int X_ELEMS = BS_LAST ? CC * LDX : TN * LDX;
+    static constexpr int LDS_ELEMS = (2 * X_ELEMS > W_ELEMS) ? 2 * X_ELEMS : W_ELEMS;
+    static constexpr int LDS_BYTES = LDS_ELEMS * (int)sizeof(CT);
+    static constexpr int W_EPV = stage<TW, CT>::EPV, X_EPV = stage<TX, CT>::EPV;
+    static constexpr int W_VECS = CC * BB / W_EPV, X_VECS = CC * TN / X_EPV;
+    static constexpr int X_PER_T = (X_VECS + THREADS - 1) / THREADS;
+    static_assert(BB % (32 * WM) == 0 && TN % (32 * WN) == 0, "wave tiling");
+    static_assert(CC % KSTEP == 0 && BB % W_EPV == 0, "block shape");
+    static_assert(BS_LAST ? TN % X_EPV == 0 : CC % X_EPV == 0, "vector width");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int BB, int CC, int TN,
+          int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void ks_ws_kernel(const TX *__restrict__ x,
+                                                            const TW *__restrict__ w,
+                                                            TY *__restrict__ y, int batch, int a,
+                                                            int d, float scale, int wgs_per_group,
+                                                            int n_tiles)
+{
+    typedef WsCfg<CT, TX, TW, TY, BS_LAST, BB, CC, TN, WM, WN> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    CT *const lds = (CT *)smem;
+    const int g = blockIdx.x / wgs_per_group;  // a_i * d + d_i
+    const int s = blockIdx.x - g * wgs_per_group;
+    const int per = (n_tiles + wgs_per_group - 1) / wgs_per_group;
+    const int t_begin = s * per, t_end = min(n_tiles, t_begin + per);
+    if (t_begin >= t_end) return;
+    const int a_i = g / d, d_i = g - a_i * d;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
+
+    // ---- weights: global -> LDS (as stored, c x b) -> registers (MFMA operand layout) ----
+    {
+        const TW *wg = w + (size_t)g * CC * BB;
+        for (int v = tid; v < C::W_VECS; v += C::THREADS) {
+            const int kk = v / (BB / C::W_EPV), mm = (v % (BB / C::W_EPV)) * C::W_EPV;
+            stage<TW, CT> r;
+            r.load(wg + (size_t)kk * BB + mm);
+            r.store(lds + kk * C::LDW + mm);
+        }
+    }
+    __syncthreads();
+    typename frag<CT>::type wreg[C::MT][C::KS];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+            wreg[i][ks] = frag<CT>::k_outer(lds, C::LDW, (wm * C::MT + i) * 32, ks * C::KSTEP, lane);
+    __syncthreads();  // LDS is reused for the input tiles from here on
+
+    const TX *xg = BS_LAST ? x + ((size_t)a_i * CC * d + d_i) * batch : x + (size_t)a_i * CC;
+    const size_t x_kstride = BS_LAST ? (size_t)d * batch : 1;
+    stage<TX, CT> xreg[C::X_PER_T];
+    auto gload = [&](int t) {
+        const int n0 = t * TN;
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                if (BS_LAST) {
+                    const int kk = v / (TN / C::X_EPV), nn = (v % (TN / C::X_EPV)) * C::X_EPV;
+                    const int col = min(n0 + nn, batch - C::X_EPV);
+                    xreg[i].load(xg + (size_t)kk * x_kstride + col);
+                } else {
+                    const int nn = v / (CC / C::X_EPV), kk = (v % (CC / C::X_EPV)) * C::X_EPV;
+                    const int row = min(n0 + nn, batch - 1);
+                    xreg[i].load(xg + (size_t)row * in_size + kk);
+                }
+            }
+        }
+    };
+    auto lstore = [&](int buf) {
+        CT *xb = lds + buf * C::X_ELEMS;
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                if (BS_LAST) {
+                    const int kk = v / (TN / C::X_EPV), nn = (v % (TN / C::X_EPV)) * C::X_EPV;
+                    xreg[i].store(xb + kk * C::LDX + nn);
+                } else {
+                    const int nn = v / (CC / C::X_EPV), kk = (v % (CC / C::X_EPV)) * C::X_EPV;
+                    xreg[i].store(xb + nn * C::LDX + kk);
+                }
+            }
+        }
+    };
+
+    const int l32 = lane & 31, lq = lane >> 5;
+    gload(t_begin);
+    lstore(0);
+    __syncthreads();
+    for (int t = t_begin; t < t_end; ++t) {
+        const int buf = (t - t_begin) & 1;
+        if (t + 1 < t_end) gload(t + 1);
+        const CT *xb = lds + buf * C::X_ELEMS;
+        float16_t acc[C::MT][C::NT];
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks) {
+            typename frag<CT>::type fx[C::NT];
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+                fx[j] = BS_LAST ? frag<CT>::k_outer(xb, C::LDX, (wn * C::NT + j) * 32, ks * C::KSTEP, lane)
+                                : frag<CT>::k_inner(xb, C::LDX, (wn * C::NT + j) * 32, ks * C::KSTEP, lane);
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j)
+                    acc[i][j] = BS_LAST ? frag<CT>::mfma(wreg[i][ks], fx[j], acc[i][j])
+                                        : frag<CT>::mfma(fx[j], wreg[i][ks], acc[i][j]);
+        }
+        const int n0 = t * TN;
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j) {
+                const int mb = (wm * C::MT + i) * 32, nb = n0 + (wn * C::NT + j) * 32;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int rr = 8 * (e >> 2) + 4 * lq + (e & 3);
+                    const float v = acc[i][j][e] * scale;
+                    if (BS_LAST) {
+                        const int m = mb + rr, n = nb + l32;
+                        if (n < batch)
+                            elem<TY>::store(y + ((size_t)(a_i * BB + m) * d + d_i) * batch + n, v);
+                    } else {
+                        const int n = nb + rr, m = mb + l32;
+                        if (n < batch) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * BB + m, v);
+                    }
+                }
+            }
+        if (t + 1 < t_end) lstore(buf ^ 1);
+        __syncthreads();
+    }
+}
+
+struct WsInst {
+    int combo, bs_last, bb, cc, tn, threads, lds;
+    const void *fn;
+};
+#define WS_INST(COMBO_, CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_)                            \
+    {COMBO_, BL_, BB_, CC_, TN_, 64 * WM_ * WN_,                                                    \
+     WsCfg<CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_>::LDS_BYTES,                             \
+     (const void *)ks_ws_kernel<CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_>}
+#define WS_SET_H(COMBO_, TX_, TW_, BL_)                                                             \
+    WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 192, 192, 64, 2, 2),                             \
+        WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 192, 192, 128, 2, 2),                        \
+        WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 128, 128, 64, 2, 2),                         \
+        WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 128, 128, 128, 2, 2),                        \
+        WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 96, 96, 128, 1, 4),                          \
+        WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 64, 64, 128, 1, 4),                          \
+        WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 64, 64, 64, 2, 2)
+#define WS_SET_F32(BL_)                                                                             \
+    WS_INST(0, float, float, float, float, BL_, 128, 128, 64, 2, 2),                                \
+        WS_INST(0, float, float, float, float, BL_, 96, 96, 128, 1, 4),                             \
+        WS_INST(0, float, float, float, float, BL_, 64, 64, 128, 1, 4),                             \
+        WS_INST(0, float, float, float, float, BL_, 64, 64, 64, 2, 2)
+const WsInst ws_insts[] = {
+    WS_SET_F32(true),
+    WS_SET_F32(false),
+    WS_SET_H(1, half_t, half_t, true),
+    WS_SET_H(1, half_t, half_t, false),
+    WS_SET_H(2, fp8_t, fp8_t, true),
+    WS_SET_H(2, fp8_t, fp8_t, false),
+    WS_SET_H(3, half_t, fp8_t, true),
+    WS_SET_H(3, half_t, fp8_t, false),
+};
+constexpr int N_WS_INSTS = sizeof(ws_insts) / sizeof(WsInst);
+constexpr int WS_VARIANT_BASE = 1000;
+
+bool ws_fits(const WsInst &t, const Problem &p, int combo)
+{
+    if (t.combo != combo || t.bs_last != p.bs_last) return false;
+    if (p.b != t.bb || p.c != t.cc) return false;
+    const int x_epv = 16 / (int)dtype_size(p.x_dtype);
+    if (p.bs_last) {
+        if (p.batch % x_epv || p.batch < x_epv) return false;
+    } else {
+        if (p.d != 1) return false;
+    }
+    return true;
+}
+
+int ws_run(const Problem &p, int variant, int wgs_hint, bool launch, ksmm_tile *tile)
+{
+    const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
+    int pick = -1;
+    for (int i = 0; i < N_WS_INSTS; ++i) {
+        if (variant >= 0 && variant != i) continue;
+        if (ws_fits(ws_insts[i], p, combo)) {
+            pick = i;
+            break;
+        }
+    }
+    if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    const WsInst &t = ws_insts[pick];
+    const int64_t groups = (int64_t)p.a * p.d;
+    const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
+    // persistent workgroups: about `target` per CU over all groups, never more than tiles
+    const int per_cu = t.lds * 2 <= 160 * 1024 ? 2 : 1;
+    int64_t wgs = wgs_hint > 0 ? wgs_hint : (256 * per_cu + groups - 1) / groups;
+    if (wgs > n_tiles) wgs = n_tiles;
+    if (wgs < 1) wgs = 1;
+    const int64_t grid = groups * wgs;
+    if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (tile) {
+        tile->algo = KSMM_ALGO_TILE;
+        tile->variant = WS_VARIANT_BASE + pick;
+        tile->tile_m = t.bb;
+        tile->tile_n = t.tn;
+        tile->tile_k = t.cc;
+        tile->tile_d = 1;
+        tile->threads = t.threads;
+        tile->lds_bytes = t.lds;
+        tile->grid = grid;
+    }
+    if (!launch) return KSMM_OK;
+    if (t.lds > 64 * 1024) {
+        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
+            return KSMM_ERR_LAUNCH;
+    }
+    int batch_i = (int)p.batch, wgs_i = (int)wgs, n_tiles_i = (int)n_tiles;
+    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
+                    (void *)&p.scale, &wgs_i, &n_tiles_i};
+    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
 // ---- instance table -----------------------------------------------------------------------
 struct TileInst {
     int combo, bs_last, tm, tn, tk, threads, lds;
@@ -355,6 +511,19 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     if (combo < 0) return KSMM_ERR_BAD_DTYPE;
+    // variants >= 1000: weight-stationary kernels (bits: 1000 + instance + 100 * workgroups/group hint)
+    // variants >= 2000: stream kernels (direct-to-LDS pipeline), see ksmm_stream.hip
+    if (variant >= 2000) return stream_run(p, variant - 2000, launch, tile);
+    if (variant >= WS_VARIANT_BASE) {
+        const int v = variant - WS_VARIANT_BASE;
+        return ws_run(p, v % 100, v / 100, launch, tile);
+    }
+    if (variant < 0) {
+        int rc = stream_run(p, -1, launch, tile);
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        rc = ws_run(p, -1, 0, launch, tile);
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
+    }
     int pick = -1;
     if (variant >= 0) {
         if (variant < N_TILE_INSTS && tile_fits(tile_insts[variant], p, combo)) pick = variant;
