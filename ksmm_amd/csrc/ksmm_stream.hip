@@ -29,6 +29,18 @@
 //  template_kernels_half.cuh:103-1092).
 #include "ksmm_mfma.h"
 
+#ifdef KSMM_PROFILE
+// Phase timestamps of wave 0 of every workgroup (standalone profiling builds only).
+__device__ unsigned long long ksmm_prof[512][64];
+#define KS_STAMP(slot)                                                                         \
+    do {                                                                                       \
+        if (threadIdx.x == 0 && blockIdx.x < 512 && (slot) < 64)                               \
+            ksmm_prof[blockIdx.x][(slot)] = __builtin_amdgcn_s_memtime();                      \
+    } while (0)
+#else
+#define KS_STAMP(slot) do { } while (0)
+#endif
+
 namespace ksmm {
 
 namespace {
@@ -66,8 +78,11 @@ struct StreamCfg {
     static constexpr int LDW = pads<CT>::outer(BB);
     static constexpr int W_BYTES = CC * LDW * ES;
     static constexpr int W_EPV = stage<TW, CT>::EPV, W_VECS = CC * BB / W_EPV;
-    static constexpr int PIPE_BYTES = ST * X_STAGE_BYTES + O_BYTES;
-    static constexpr int LDS_BYTES = W_BYTES > PIPE_BYTES ? W_BYTES : PIPE_BYTES;
+    // LDS map: [weight staging, later the output tile][ST input stages]; the stages do not
+    // overlap the weight staging area, so the first input tiles are requested before the
+    // weights are staged
+    static constexpr int HEAD_BYTES = ((W_BYTES > O_BYTES ? W_BYTES : O_BYTES) + 1023) / 1024 * 1024;
+    static constexpr int LDS_BYTES = HEAD_BYTES + ST * X_STAGE_BYTES;
     // vector-memory instructions issued after the loads of the tile being waited for
     static constexpr int N_SAFE = (ST - 1) * L;             // while fewer than ST-1 tiles were stored
     static constexpr int N_FULL = (ST - 1) * (L + S);       // steady state
@@ -139,26 +154,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
-
-    // ---- weights: global -> LDS (as stored, c x b, padded rows) -> registers ---------------
-    {
-        CT *wl = (CT *)smem;
-        const TW *wg = w + (size_t)g * CC * BB;
-        for (int v = tid; v < C::W_VECS; v += C::THREADS) {
-            const int kk = v / (BB / C::W_EPV), mm = (v % (BB / C::W_EPV)) * C::W_EPV;
-            stage<TW, CT> r;
-            r.load(wg + (size_t)kk * BB + mm);
-            r.store(wl + kk * C::LDW + mm);
-        }
-        __syncthreads();
-    }
-    typename frag<CT>::type wreg[C::MT][C::KS];
-#pragma unroll
-    for (int i = 0; i < C::MT; ++i)
-#pragma unroll
-        for (int ks = 0; ks < C::KS; ++ks)
-            wreg[i][ks] = frag<CT>::k_outer((const CT *)smem, C::LDW, (wm * C::MT + i) * 32, ks * C::KSTEP, lane);
-    __syncthreads();  // LDS is reused for the input stages and the output tile from here on
+    KS_STAMP(0);
 
     // ---- direct-to-LDS loads of one input tile ---------------------------------------------
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -181,7 +177,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
         }
     }
     auto issue = [&](int n0, int stg) {
-        const uint32_t dst = lds_base + stg * C::X_STAGE_BYTES + wave * 1024;
+        const uint32_t dst = lds_base + C::HEAD_BYTES + stg * C::X_STAGE_BYTES + wave * 1024;
 #pragma unroll
         for (int i = 0; i < C::L; ++i) {
             const CT *p;
@@ -193,12 +189,42 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
         }
     };
 
-    CT *const out = (CT *)(smem + ST * C::X_STAGE_BYTES);
+    CT *const out = (CT *)smem;
     const int l32 = lane & 31, lq = lane >> 5;
     const int n_iters = (c_end - c_begin + TN - 1) / TN;
     // prologue: ST-1 tiles in flight (tiles past the end repeat the last one; never read)
 #pragma unroll
     for (int p = 0; p < ST - 1; ++p) issue(c_begin + min(p, n_iters - 1) * TN, p);
+    KS_STAMP(1);
+
+    // ---- weights: global -> LDS (as stored, c x b, padded rows) -> registers ---------------
+    {
+        CT *wl = (CT *)smem;
+        const TW *wg = w + (size_t)g * CC * BB;
+        // all loads first, then all LDS writes: one memory latency instead of one per vector
+        constexpr int W_PER_T = (C::W_VECS + C::THREADS - 1) / C::THREADS;
+        stage<TW, CT> r[W_PER_T];
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) {
+            const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
+            r[i].load(wg + (size_t)(v / (BB / C::W_EPV)) * BB + (v % (BB / C::W_EPV)) * C::W_EPV);
+        }
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) {
+            const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
+            r[i].store(wl + (v / (BB / C::W_EPV)) * C::LDW + (v % (BB / C::W_EPV)) * C::W_EPV);
+        }
+        __syncthreads();
+    }
+    typename frag<CT>::type wreg[C::MT][C::KS];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+            wreg[i][ks] = frag<CT>::k_outer((const CT *)smem, C::LDW, (wm * C::MT + i) * 32, ks * C::KSTEP, lane);
+    __syncthreads();  // the staging area becomes the output tile from here on
+    KS_STAMP(2);
+
 
     for (int it = 0; it < n_iters; ++it) {
         const int n0 = c_begin + it * TN;
@@ -208,8 +234,9 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
         else
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_SAFE));
         __syncthreads();  // tile `it` has landed for every wave
+        KS_STAMP(4 + 4 * it);
 
-        const CT *xb = (const CT *)(smem + (it % ST) * C::X_STAGE_BYTES);
+        const CT *xb = (const CT *)(smem + C::HEAD_BYTES + (it % ST) * C::X_STAGE_BYTES);
         float16_t acc[C::MT][C::NT];
 #pragma unroll
         for (int i = 0; i < C::MT; ++i)
@@ -217,19 +244,23 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
             for (int j = 0; j < C::NT; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        // all operand reads of the tile are issued before the first MFMA: with one wave per
+        // SIMD nothing else would hide the LDS latency
+        typename frag<CT>::type fx[C::KS][C::NT];
 #pragma unroll
-        for (int ks = 0; ks < C::KS; ++ks) {
-            typename frag<CT>::type fx[C::NT];
+        for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
             for (int j = 0; j < C::NT; ++j)
-                fx[j] = xfrag<CT, BS_LAST, C::X_COLS>::get(xb, (wn * C::NT + j) * 32, ks * C::KSTEP, lane);
+                fx[ks][j] = xfrag<CT, BS_LAST, C::X_COLS>::get(xb, (wn * C::NT + j) * 32, ks * C::KSTEP, lane);
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
             for (int i = 0; i < C::MT; ++i)
 #pragma unroll
                 for (int j = 0; j < C::NT; ++j)
-                    acc[i][j] = BS_LAST ? frag<CT>::mfma(fx[j], wreg[i][ks], acc[i][j])
-                                        : frag<CT>::mfma(wreg[i][ks], fx[j], acc[i][j]);
-        }
+                    acc[i][j] = BS_LAST ? frag<CT>::mfma(fx[ks][j], wreg[i][ks], acc[i][j])
+                                        : frag<CT>::mfma(wreg[i][ks], fx[ks][j], acc[i][j]);
+        KS_STAMP(5 + 4 * it);
         // ---- accumulators -> LDS output tile: out[lane index][4 consecutive row indices] ----
 #pragma unroll
         for (int i = 0; i < C::MT; ++i)
@@ -255,6 +286,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
                 }
             }
         __syncthreads();
+        KS_STAMP(6 + 4 * it);
         // ---- LDS output tile -> global, 16 bytes per lane along the contiguous axis --------
 #pragma unroll
         for (int i = 0; i < C::S; ++i) {
@@ -273,7 +305,9 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
                 if (n < c_end) *(uint4_t *)dst = v;
             }
         }
+        KS_STAMP(7 + 4 * it);
     }
+    KS_STAMP(3);
     // direct-to-LDS loads of the repeated last tile may still be in flight: they must land
     // before this workgroup's LDS is handed to another one
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -289,8 +323,8 @@ struct StreamInst {
      StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::EPC,                                     \
      (const void *)ks_stream_kernel<CT_, TW_, CT_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>}
 #define STREAM_SET_H(COMBO_, TW_)                                                                     \
-    STREAM_INST(COMBO_, half_t, TW_, true, 192, 192, 64, 2, 2, 4),                                   \
-        STREAM_INST(COMBO_, half_t, TW_, false, 192, 192, 64, 2, 2, 4),                              \
+    STREAM_INST(COMBO_, half_t, TW_, true, 192, 192, 64, 2, 2, 3),                                   \
+        STREAM_INST(COMBO_, half_t, TW_, false, 192, 192, 64, 2, 2, 3),                              \
         STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 128, 1, 4, 5),                                \
         STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 128, 1, 4, 5),                               \
         STREAM_INST(COMBO_, half_t, TW_, true, 128, 128, 64, 2, 2, 4),                               \
@@ -302,7 +336,7 @@ const StreamInst stream_insts[] = {
     STREAM_SET_H(3, fp8_t),
     STREAM_INST(0, float, float, true, 64, 64, 64, 1, 2, 4),
     STREAM_INST(0, float, float, true, 64, 64, 128, 1, 4, 3),
-    STREAM_INST(0, float, float, true, 128, 128, 64, 2, 2, 3),
+    STREAM_INST(0, float, float, true, 128, 128, 64, 2, 2, 2),
 };
 constexpr int N_STREAM_INSTS = sizeof(stream_insts) / sizeof(StreamInst);
 

@@ -251,11 +251,18 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_ws_kernel(const TX *__restric
     // ---- weights: global -> LDS (as stored, c x b) -> registers (MFMA operand layout) ----
     {
         const TW *wg = w + (size_t)g * CC * BB;
-        for (int v = tid; v < C::W_VECS; v += C::THREADS) {
-            const int kk = v / (BB / C::W_EPV), mm = (v % (BB / C::W_EPV)) * C::W_EPV;
-            stage<TW, CT> r;
-            r.load(wg + (size_t)kk * BB + mm);
-            r.store(lds + kk * C::LDW + mm);
+        // all loads first, then all LDS writes: one memory latency instead of one per vector
+        constexpr int W_PER_T = (C::W_VECS + C::THREADS - 1) / C::THREADS;
+        stage<TW, CT> r[W_PER_T];
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) {
+            const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
+            r[i].load(wg + (size_t)(v / (BB / C::W_EPV)) * BB + (v % (BB / C::W_EPV)) * C::W_EPV);
+        }
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) {
+            const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
+            r[i].store(lds + (v / (BB / C::W_EPV)) * C::LDW + (v % (BB / C::W_EPV)) * C::W_EPV);
         }
     }
     __syncthreads();
@@ -512,6 +519,9 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     if (combo < 0) return KSMM_ERR_BAD_DTYPE;
     // variants >= 1000: weight-stationary kernels (bits: 1000 + instance + 100 * workgroups/group hint)
+    // variants >= 3000: batch-size-first kernels for small d > 1, see ksmm_tile_bf.hip
+    if (variant >= 3000) return tile_bf_run(p, variant - 3000, launch, tile);
+    if (variant < 0 && !p.bs_last && p.d > 1) return tile_bf_run(p, -1, launch, tile);
     // variants >= 2000: stream kernels (direct-to-LDS pipeline), see ksmm_stream.hip
     if (variant >= 2000) return stream_run(p, variant - 2000, launch, tile);
     if (variant >= WS_VARIANT_BASE) {

@@ -1,0 +1,276 @@
+// Tile kernel for the batch-size-first layout with a small d > 1.
+//
+// Batch-size-first rows hold the features as (a_i, c_i, d_i) with d_i fastest, so for d > 1
+// the c inputs of one (a_i, d_i) block are strided by d.  A workgroup therefore takes all d
+// blocks of one a_i at once: it reads the contiguous run x[n][(a_i*c + k0)*d .. (a_i*c + k0 +
+// TK)*d) with 16-byte loads, splits it by d_i while writing it to LDS (one k-contiguous plane
+// per d_i), runs d independent TM x TN x TK MFMA products against the d weight blocks, and
+// interleaves the d results again in registers, so that a lane stores d consecutive output
+// features and a tile row is one contiguous run of y.
+//
+// MFMA roles as in the batch-size-first case of the plain tile kernel: A = X (rows = batch),
+// B = W (lanes = outputs), fp32 accumulation, 32x32 tiles.
+//
+// Reference counterpart: kernel_bs_first_float / kernel_bs_first_half2
+// (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-286,
+//  template_kernels_half.cuh:103-299), which gather the strided inputs with scalar loads.
+#include "ksmm_mfma.h"
+
+namespace ksmm {
+
+namespace {
+
+template <typename CT, int N> struct alignas(N * sizeof(CT)) pack_t {
+    CT e[N];
+};
+
+template <typename CT, typename TW, int DD, int TM, int TN, int TK, int WM, int WN> struct BfCfg {
+    static constexpr int THREADS = 64 * WM * WN;
+    static constexpr int KSTEP = compute<CT>::KSTEP;
+    static constexpr int MT = TM / WM / 32, NT = TN / WN / 32;
+    static constexpr int EPV = 16 / (int)sizeof(CT);  // elements per 16-byte input vector
+    static constexpr int KPV = EPV / DD;              // consecutive k per input vector
+    static constexpr int LDW = pads<CT>::outer(TM);
+    static constexpr int LDK = pads<CT>::inner(TK);
+    static constexpr int W_ELEMS = DD * TK * LDW, X_ELEMS = DD * TN * LDK;
+    static constexpr int LDS_BYTES = 2 * (W_ELEMS + X_ELEMS) * (int)sizeof(CT);
+    static constexpr int W_EPV = stage<TW, CT>::EPV;
+    static constexpr int W_VECS = DD * TK * TM / W_EPV, X_VECS = TN * TK * DD / EPV;
+    static constexpr int W_PER_T = (W_VECS + THREADS - 1) / THREADS, X_PER_T = (X_VECS + THREADS - 1) / THREADS;
+    static_assert(EPV % DD == 0 && KPV >= 1, "d must divide the 16-byte vector");
+    static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0 && TK % KSTEP == 0, "wave tiling");
+    static_assert(TM % W_EPV == 0 && TK % KPV == 0, "vector width");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+template <typename CT, typename TW, typename TY, int DD, int TM, int TN, int TK, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__restrict__ x,
+                                                                 const TW *__restrict__ w,
+                                                                 TY *__restrict__ y, int batch, int a,
+                                                                 int b, int c, float scale,
+                                                                 int m_tiles, int n_tiles, int blocks)
+{
+    typedef BfCfg<CT, TW, DD, TM, TN, TK, WM, WN> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    CT *const lds = (CT *)smem;
+    auto ws = [&](int buf, int dd) { return lds + buf * C::W_ELEMS + dd * TK * C::LDW; };
+    auto xs = [&](int buf, int dd) { return lds + 2 * C::W_ELEMS + buf * C::X_ELEMS + dd * TN * C::LDK; };
+
+    // workgroups that share an input tile (the TM-tiles of one batch tile) get consecutive
+    // logical ids on one XCD
+    const int per_xcd = (blocks + 7) / 8;
+    const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lid >= blocks) return;
+    const int mt_id = lid % m_tiles;
+    const int rest = lid / m_tiles;
+    const int nt_id = rest % n_tiles;
+    const int a_i = rest / n_tiles;
+    const int m0 = mt_id * TM, n0 = nt_id * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const size_t in_size = (size_t)a * c * DD, out_size = (size_t)a * b * DD;
+    const CT *xg = x + (size_t)a_i * c * DD;  // + n * in_size + k * DD + dd
+
+    stage<TW, CT> wreg[C::W_PER_T];
+    uint4_t xreg[C::X_PER_T];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::W_VECS % C::THREADS == 0 || v < C::W_VECS) {
+                const int per_dd = TK * TM / C::W_EPV;
+                const int dd = v / per_dd, r = v % per_dd;
+                const int kk = r / (TM / C::W_EPV), mm = (r % (TM / C::W_EPV)) * C::W_EPV;
+                wreg[i].load(w + ((size_t)(a_i * DD + dd) * c + k0 + kk) * b + m0 + mm);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                const int vpr = TK * DD / C::EPV;  // vectors per row
+                const int nn = v / vpr, e0 = (v % vpr) * C::EPV;
+                const int row = min(n0 + nn, batch - 1);
+                xreg[i] = *(const uint4_t *)(xg + (size_t)row * in_size + (size_t)k0 * DD + e0);
+            }
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < C::W_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::W_VECS % C::THREADS == 0 || v < C::W_VECS) {
+                const int per_dd = TK * TM / C::W_EPV;
+                const int dd = v / per_dd, r = v % per_dd;
+                const int kk = r / (TM / C::W_EPV), mm = (r % (TM / C::W_EPV)) * C::W_EPV;
+                wreg[i].store(ws(buf, dd) + kk * C::LDW + mm);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                const int vpr = TK * DD / C::EPV;
+                const int nn = v / vpr, kk = (v % vpr) * C::KPV;
+                // split the vector by d_i: element e is (k = kk + e / DD, d_i = e % DD)
+                pack_t<CT, C::EPV> all = __builtin_bit_cast(pack_t<CT, C::EPV>, xreg[i]);
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd) {
+                    pack_t<CT, C::KPV> part;
+#pragma unroll
+                    for (int q = 0; q < C::KPV; ++q) part.e[q] = all.e[q * DD + dd];
+                    *(pack_t<CT, C::KPV> *)(xs(buf, dd) + nn * C::LDK + kk) = part;
+                }
+            }
+        }
+    };
+
+    float16_t acc[DD][C::MT][C::NT];
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = 0.f;
+
+    const int steps = c / TK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int s = 0; s < steps; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < steps) gload((s + 1) * TK);
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) {
+            const CT *wb = ws(buf, dd), *xb = xs(buf, dd);
+#pragma unroll
+            for (int k0 = 0; k0 < TK; k0 += C::KSTEP) {
+                typename frag<CT>::type fw[C::MT], fx[C::NT];
+#pragma unroll
+                for (int i = 0; i < C::MT; ++i)
+                    fw[i] = frag<CT>::k_outer(wb, C::LDW, (wm * C::MT + i) * 32, k0, lane);
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j)
+                    fx[j] = frag<CT>::k_inner(xb, C::LDK, (wn * C::NT + j) * 32, k0, lane);
+#pragma unroll
+                for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::NT; ++j)
+                        acc[dd][i][j] = frag<CT>::mfma(fx[j], fw[i], acc[dd][i][j]);
+            }
+        }
+        if (s + 1 < steps) lstore(buf ^ 1);
+        __syncthreads();
+    }
+
+    // D tile: lane holds output column m = lane % 32, batch rows 8*(e/4) + 4*(lane/32) + e%4;
+    // the DD results of one (n, m) are adjacent in y
+    const int l32 = lane & 31, lq = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            const int m = m0 + (wm * C::MT + i) * 32 + l32;
+            const int nb = n0 + (wn * C::NT + j) * 32;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int n = nb + 8 * (e >> 2) + 4 * lq + (e & 3);
+                pack_t<TY, DD> o;
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd) o.e[dd] = (TY)(acc[dd][i][j][e] * scale);
+                if (n < batch)
+                    *(pack_t<TY, DD> *)(y + (size_t)n * out_size + ((size_t)a_i * b + m) * DD) = o;
+            }
+        }
+}
+
+struct BfInst {
+    int combo, dd, tm, tn, tk, threads, lds;
+    const void *fn;
+};
+#define BF_INST(COMBO_, CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_)                                  \
+    {COMBO_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, BfCfg<CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, \
+     (const void *)ks_tile_bf_kernel<CT_, TW_, CT_, DD_, TM_, TN_, TK_, WM_, WN_>}
+#define BF_SET_H(COMBO_, TW_)                                                                    \
+    BF_INST(COMBO_, half_t, TW_, 2, 128, 128, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 2, 256, 128, 32, 2, 2), \
+        BF_INST(COMBO_, half_t, TW_, 2, 128, 256, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 2, 64, 128, 32, 1, 4), \
+        BF_INST(COMBO_, half_t, TW_, 2, 32, 128, 32, 1, 4), BF_INST(COMBO_, half_t, TW_, 4, 64, 128, 32, 1, 4), \
+        BF_INST(COMBO_, half_t, TW_, 4, 32, 128, 32, 1, 4)
+const BfInst bf_insts[] = {
+    BF_SET_H(1, half_t),
+    BF_SET_H(3, fp8_t),
+    BF_INST(0, float, float, 2, 128, 128, 16, 2, 2),
+    BF_INST(0, float, float, 2, 64, 128, 16, 1, 4),
+    BF_INST(0, float, float, 2, 32, 128, 16, 1, 4),
+    BF_INST(0, float, float, 4, 64, 128, 16, 1, 4),
+    BF_INST(0, float, float, 4, 32, 128, 16, 1, 4),
+};
+constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
+
+bool bf_fits(const BfInst &t, const Problem &p, int combo)
+{
+    if (t.combo != combo || p.bs_last || p.d != t.dd) return false;
+    if (p.b % t.tm || p.c % t.tk) return false;
+    const int x_epv = 16 / (int)dtype_size(p.x_dtype), w_epv = 16 / (int)dtype_size(p.w_dtype);
+    if (p.b % w_epv) return false;
+    // rows of x start at multiples of in_size, slabs at multiples of TK * d: keep 16-byte alignment
+    if (((int64_t)p.a * p.c * p.d) % x_epv || ((int64_t)p.c * p.d) % x_epv) return false;
+    return true;
+}
+
+}  // namespace
+
+// variant: index into the instance table (-1: heuristic)
+int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
+{
+    const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
+    int pick = -1;
+    if (variant >= 0) {
+        if (variant < N_BF_INSTS && bf_fits(bf_insts[variant], p, combo)) pick = variant;
+    } else {
+        int64_t best = -1;
+        for (int i = 0; i < N_BF_INSTS; ++i) {
+            const BfInst &t = bf_insts[i];
+            if (!bf_fits(t, p, combo)) continue;
+            const int64_t wgs = (int64_t)p.a * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
+            int64_t score = (int64_t)t.tm * 1000 + t.tn;
+            if (wgs < 512) score -= 100000;
+            if (score > best) {
+                best = score;
+                pick = i;
+            }
+        }
+    }
+    if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    const BfInst &t = bf_insts[pick];
+    const int m_tiles = p.b / t.tm;
+    const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
+    const int64_t blocks = (int64_t)p.a * m_tiles * n_tiles;
+    const int64_t grid = (blocks + 7) / 8 * 8;
+    if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (tile) {
+        tile->algo = KSMM_ALGO_TILE;
+        tile->variant = 3000 + pick;
+        tile->tile_m = t.tm;
+        tile->tile_n = t.tn;
+        tile->tile_k = t.tk;
+        tile->tile_d = t.dd;
+        tile->threads = t.threads;
+        tile->lds_bytes = t.lds;
+        tile->grid = grid;
+    }
+    if (!launch) return KSMM_OK;
+    if (t.lds > 64 * 1024) {
+        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
+            return KSMM_ERR_LAUNCH;
+    }
+    int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
+    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
+                    (void *)&p.c, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i};
+    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm
