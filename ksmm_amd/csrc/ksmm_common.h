@@ -92,6 +92,7 @@ int generic_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
+int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the wave family
 int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 
 }  // namespace ksmm

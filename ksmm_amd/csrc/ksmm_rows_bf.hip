@@ -1,0 +1,200 @@
+// "Row" kernel: batch-size-first layout, d > 1, small b x c blocks, fp32.
+//
+// In this layout a batch row holds, for one a_i, the c*d inputs of all d blocks interleaved
+// (d_i fastest).  A workgroup owns one a_i and a range of batch rows; it has one wavefront per
+// d_i, and each wavefront keeps the b x c weight block of its d_i in registers as MFMA
+// operands (v_mfma_f32_16x16x4_f32, fp32 accumulation).  Whole row segments (c*d contiguous
+// floats) are copied to LDS with 16-byte loads, every wave picks the inputs of its own d_i
+// out of LDS (stride d), the d result blocks are interleaved again in an LDS output tile, and
+// the b*d outputs of each row are written back as one contiguous run.  HBM sees only full,
+// coalesced rows; the stride-d gather the layout forces happens in LDS.
+//
+// Input tiles are double-buffered in LDS across batch tiles (the loads of tile t+1 are in
+// flight while tile t is multiplied and stored).
+//
+// Reference counterpart: kernel_bs_first_float
+// (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-286), whose strided scalar
+// gathers from global memory (:156-161) make this the slowest layout of the reference
+// (0.86 ms for (1,48,48,16) in kernel_bs_first_float.best:9).
+#include "ksmm_common.h"
+
+namespace ksmm {
+
+namespace {
+
+template <int BB, int CC, int DD, int TN> struct RowCfg {
+    static constexpr int NW = DD, THREADS = 64 * NW;
+    static constexpr int MT = BB / 16, KS = CC / 4, NT = TN / 16;
+    static constexpr int XROW = CC * DD, OROW = BB * DD;  // floats per row segment
+    static constexpr int LDX = XROW + 4, LDO = OROW + 4;
+    static constexpr int X_VECS = TN * XROW / 4, O_VECS = TN * OROW / 4;
+    static constexpr int X_PER_T = (X_VECS + THREADS - 1) / THREADS, O_PER_T = (O_VECS + THREADS - 1) / THREADS;
+    static constexpr int LDS_BYTES = (2 * TN * LDX + TN * LDO) * 4;
+    static_assert(BB % 16 == 0 && CC % 4 == 0 && TN % 16 == 0, "MFMA tiling");
+    static_assert(NW <= 16 && XROW % 4 == 0 && OROW % 4 == 0, "shape");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+template <int BB, int CC, int DD, int TN>
+__global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__restrict__ x,
+                                                            const float *__restrict__ w,
+                                                            float *__restrict__ y, int batch, int a,
+                                                            float scale, int wgs_per_a, int n_tiles)
+{
+    typedef RowCfg<BB, CC, DD, TN> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float *const xs = (float *)smem;                // [2][TN][LDX]
+    float *const os = xs + 2 * TN * C::LDX;         // [TN][LDO]
+    const int a_i = blockIdx.x / wgs_per_a;
+    const int s = blockIdx.x - a_i * wgs_per_a;
+    const int per = (n_tiles + wgs_per_a - 1) / wgs_per_a;
+    const int t_begin = s * per, t_end = min(n_tiles, t_begin + per);
+    if (t_begin >= t_end) return;
+    const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
+    const int dd = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's d_i
+    const size_t in_size = (size_t)a * C::XROW, out_size = (size_t)a * C::OROW;
+
+    // weights of block (a_i, dd): element (k, m) at ((a_i*d + dd)*c + k)*b + m -> A operands
+    float wreg[C::MT][C::KS];
+    {
+        const float *wg = w + (size_t)(a_i * DD + dd) * CC * BB;
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < C::MT; ++mt) wreg[mt][ks] = wg[(4 * ks + q) * BB + 16 * mt + r];
+    }
+
+    const float *xg = x + (size_t)a_i * C::XROW;
+    float *yg = y + (size_t)a_i * C::OROW;
+    float4_t xreg[C::X_PER_T];
+    auto gload = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                const int nn = v / (C::XROW / 4), e0 = (v % (C::XROW / 4)) * 4;
+                const int row = min(t * TN + nn, batch - 1);
+                xreg[i] = *(const float4_t *)(xg + (size_t)row * in_size + e0);
+            }
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                const int nn = v / (C::XROW / 4), e0 = (v % (C::XROW / 4)) * 4;
+                *(float4_t *)(xs + (buf * TN + nn) * C::LDX + e0) = xreg[i];
+            }
+        }
+    };
+
+    gload(t_begin);
+    lstore(0);
+    __syncthreads();
+    for (int t = t_begin; t < t_end; ++t) {
+        const int buf = (t - t_begin) & 1;
+        if (t + 1 < t_end) gload(t + 1);
+        const float *xb = xs + buf * TN * C::LDX;
+        float4_t acc[C::MT][C::NT];
+#pragma unroll
+        for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt) acc[mt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+        // B operand: lane (r, q) = input (k = 4*ks + q) of batch row 16*nt + r, for this d_i
+        float xf[C::KS][C::NT];
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt) xf[ks][nt] = xb[(16 * nt + r) * C::LDX + (4 * ks + q) * DD + dd];
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < C::MT; ++mt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[mt][ks], xf[ks][nt], acc[mt][nt], 0, 0, 0);
+        // D: lane (r, q) holds batch row 16*nt + r, outputs m = 16*mt + 4*q + i
+#pragma unroll
+        for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = acc[mt][nt][i] * scale;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < C::O_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::O_VECS % C::THREADS == 0 || v < C::O_VECS) {
+                const int nn = v / (C::OROW / 4), e0 = (v % (C::OROW / 4)) * 4;
+                const int row = t * TN + nn;
+                if (row < batch)
+                    __builtin_nontemporal_store(*(const float4_t *)(os + nn * C::LDO + e0),
+                                                (float4_t *)(yg + (size_t)row * out_size + e0));
+            }
+        }
+        if (t + 1 < t_end) lstore(buf ^ 1);
+        __syncthreads();
+    }
+}
+
+struct RowInst {
+    int bb, cc, dd, tn, lds;
+    const void *fn;
+};
+#define ROW_INST(BB_, CC_, DD_, TN_) \
+    {BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_>}
+const RowInst row_insts[] = {
+    ROW_INST(48, 48, 16, 16), ROW_INST(48, 48, 8, 32), ROW_INST(48, 48, 4, 64), ROW_INST(64, 64, 8, 16),
+    ROW_INST(64, 64, 4, 32),  ROW_INST(16, 16, 16, 32), ROW_INST(16, 16, 4, 128), ROW_INST(32, 32, 8, 32),
+};
+constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
+
+}  // namespace
+
+// variant: bits 0-6 instance (0x7f: first that fits), bits 7.. workgroups per a_i (0: heuristic)
+int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
+{
+    if (p.bs_last || combo_of(p.x_dtype, p.w_dtype, p.y_dtype) != 0) return KSMM_ERR_BAD_ALGO;
+    const int want = variant < 0 ? 0x7f : (variant & 0x7f);
+    int64_t wgs = variant < 0 ? 0 : (variant >> 7);
+    int pick = -1;
+    for (int i = 0; i < N_ROW_INSTS; ++i) {
+        if (want != 0x7f && want != i) continue;
+        if (row_insts[i].bb == p.b && row_insts[i].cc == p.c && row_insts[i].dd == p.d) {
+            pick = i;
+            break;
+        }
+    }
+    if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    const RowInst &t = row_insts[pick];
+    const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
+    if (wgs <= 0) wgs = (256 + p.a - 1) / p.a;
+    if (wgs > n_tiles) wgs = n_tiles;
+    const int64_t grid = (int64_t)p.a * wgs;
+    if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (tile) {
+        tile->algo = KSMM_ALGO_WAVE;
+        tile->variant = 1000 + pick;
+        tile->tile_m = t.bb;
+        tile->tile_n = t.tn;
+        tile->tile_k = t.cc;
+        tile->tile_d = t.dd;
+        tile->threads = 64 * t.dd;
+        tile->lds_bytes = t.lds;
+        tile->grid = grid;
+    }
+    if (!launch) return KSMM_OK;
+    if (t.lds > 64 * 1024) {
+        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
+            return KSMM_ERR_LAUNCH;
+    }
+    int batch_i = (int)p.batch, wgs_i = (int)wgs, n_tiles_i = (int)n_tiles;
+    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.scale,
+                    &wgs_i, &n_tiles_i};
+    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(64 * t.dd), args, t.lds, p.stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm

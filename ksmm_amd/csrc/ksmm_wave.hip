@@ -351,7 +351,9 @@ const WaveInst q_insts[] = {
 
 int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
-    if (!p.bs_last) return KSMM_ERR_BAD_ALGO;
+    // batch-size-first: the register-stationary row kernel (variants >= 1000), d > 1 only
+    if (!p.bs_last) return rows_bf_run(p, variant >= 1000 ? variant - 1000 : -1, launch, tile);
+    if (variant >= 1000) return KSMM_ERR_BAD_ALGO;
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     const WaveInst *insts;
     int n_insts;

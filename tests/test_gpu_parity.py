@@ -18,7 +18,7 @@ SMALL_PATTERNS = [
     (1, 16, 16, 1), (2, 16, 16, 3), (1, 48, 48, 16), (6, 64, 64, 1), (1, 16, 16, 64),
     (16, 16, 16, 4), (64, 16, 16, 1), (2, 32, 64, 2), (1, 64, 32, 4), (3, 48, 16, 2),
     (1, 96, 96, 2), (1, 128, 128, 1), (2, 192, 192, 1), (1, 256, 64, 2), (1, 80, 48, 1),
-    (1, 17, 33, 2), (2, 64, 32, 2), (1, 128, 64, 4), (3, 32, 32, 8), (1, 256, 128, 2),
+    (1, 17, 33, 2), (2, 16, 16, 16), (1, 64, 64, 4), (2, 48, 48, 8), (2, 64, 32, 2), (1, 128, 64, 4), (3, 32, 32, 8), (1, 256, 128, 2),
 ]
 BATCHES = [1, 7, 64, 200, 1024]
 
