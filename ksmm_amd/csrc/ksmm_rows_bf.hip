@@ -35,7 +35,7 @@ template <int BB, int CC, int DD, int TN> struct RowCfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-template <int BB, int CC, int DD, int TN>
+template <int BB, int CC, int DD, int TN, bool NT_STORE>
 __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a,
@@ -129,9 +129,13 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
             if (C::O_VECS % C::THREADS == 0 || v < C::O_VECS) {
                 const int nn = v / (C::OROW / 4), e0 = (v % (C::OROW / 4)) * 4;
                 const int row = t * TN + nn;
-                if (row < batch)
-                    __builtin_nontemporal_store(*(const float4_t *)(os + nn * C::LDO + e0),
-                                                (float4_t *)(yg + (size_t)row * out_size + e0));
+                if (row < batch) {
+                    const float4_t o = *(const float4_t *)(os + nn * C::LDO + e0);
+                    if (NT_STORE)
+                        __builtin_nontemporal_store(o, (float4_t *)(yg + (size_t)row * out_size + e0));
+                    else
+                        *(float4_t *)(yg + (size_t)row * out_size + e0) = o;
+                }
             }
         }
         if (t + 1 < t_end) lstore(buf ^ 1);
@@ -143,11 +147,12 @@ struct RowInst {
     int bb, cc, dd, tn, lds;
     const void *fn;
 };
-#define ROW_INST(BB_, CC_, DD_, TN_) \
-    {BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_>}
+#define ROW_INST(BB_, CC_, DD_, TN_, NT_) \
+    {BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
 const RowInst row_insts[] = {
-    ROW_INST(48, 48, 16, 16), ROW_INST(48, 48, 8, 32), ROW_INST(48, 48, 4, 64), ROW_INST(64, 64, 8, 16),
-    ROW_INST(64, 64, 4, 32),  ROW_INST(16, 16, 16, 32), ROW_INST(16, 16, 4, 128), ROW_INST(32, 32, 8, 32),
+    ROW_INST(48, 48, 16, 16, true), ROW_INST(48, 48, 8, 32, true), ROW_INST(48, 48, 4, 64, true),
+    ROW_INST(64, 64, 8, 16, true),  ROW_INST(64, 64, 4, 32, true), ROW_INST(16, 16, 16, 32, true),
+    ROW_INST(16, 16, 4, 128, true), ROW_INST(32, 32, 8, 32, true), ROW_INST(48, 48, 16, 16, false),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 

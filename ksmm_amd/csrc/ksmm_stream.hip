@@ -35,7 +35,7 @@ __device__ unsigned long long ksmm_prof[512][64];
 #define KS_STAMP(slot)                                                                         \
     do {                                                                                       \
         if (threadIdx.x == 0 && blockIdx.x < 512 && (slot) < 64)                               \
-            ksmm_prof[blockIdx.x][(slot)] = __builtin_amdgcn_s_memtime();                      \
+            ksmm_prof[blockIdx.x][(slot)] = ((slot) == 0 || (slot) == 3) ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); \
     } while (0)
 #else
 #define KS_STAMP(slot) do { } while (0)
@@ -298,11 +298,12 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
             if (BS_LAST) {
                 const int n = n0 + oc;
                 TY *dst = y + ((size_t)(a_i * BB + orow) * d + d_i) * batch + min(n, c_end - C::EPC);
-                if (n < c_end) *(uint4_t *)dst = v;
+                if (n < c_end) *(uint4_t *)dst = v;  // 128/256-byte row pieces: plain stores measured faster
             } else {
                 const int n = n0 + orow;
                 TY *dst = y + (size_t)min(n, c_end - 1) * out_size + (size_t)a_i * BB + oc;
-                if (n < c_end) *(uint4_t *)dst = v;
+                // whole rows of b outputs: streaming (nontemporal) stores measured faster
+                if (n < c_end) __builtin_nontemporal_store(v, (uint4_t *)dst);
             }
         }
         KS_STAMP(7 + 4 * it);
@@ -315,28 +316,36 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
 
 struct StreamInst {
     int combo, bs_last, bb, cc, tn, threads, lds, epc;
+    int per_cu;  // persistent workgroups per CU the heuristic launches; 0: only when forced
     const void *fn;
 };
-#define STREAM_INST(COMBO_, CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_)                              \
+#define STREAM_INST(COMBO_, CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_, PER_CU_)                     \
     {COMBO_, BL_, BB_, CC_, TN_, 64 * WM_ * WN_,                                                     \
      StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::LDS_BYTES,                               \
-     StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::EPC,                                     \
+     StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::EPC, PER_CU_,                            \
      (const void *)ks_stream_kernel<CT_, TW_, CT_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>}
+// The first instance that fits a problem is the default; the order and the workgroups-per-CU
+// column come from sweeps at batch 25088 on MI355X.
 #define STREAM_SET_H(COMBO_, TW_)                                                                     \
-    STREAM_INST(COMBO_, half_t, TW_, true, 192, 192, 64, 2, 2, 3),                                   \
-        STREAM_INST(COMBO_, half_t, TW_, false, 192, 192, 64, 2, 2, 3),                              \
-        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 128, 1, 4, 5),                                \
-        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 128, 1, 4, 5),                               \
-        STREAM_INST(COMBO_, half_t, TW_, true, 128, 128, 64, 2, 2, 4),                               \
-        STREAM_INST(COMBO_, half_t, TW_, false, 128, 128, 64, 2, 2, 4),                              \
-        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 64, 1, 2, 6),                                 \
-        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 64, 1, 2, 6)
+    STREAM_INST(COMBO_, half_t, TW_, true, 192, 192, 64, 2, 2, 3, 1),                                \
+        STREAM_INST(COMBO_, half_t, TW_, false, 192, 192, 64, 2, 2, 3, 1),                           \
+        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 128, 1, 4, 3, 1),                             \
+        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 64, 1, 2, 3, 3),                             \
+        STREAM_INST(COMBO_, half_t, TW_, true, 128, 128, 64, 2, 2, 4, 1),                            \
+        STREAM_INST(COMBO_, half_t, TW_, false, 128, 128, 64, 2, 2, 4, 1),                           \
+        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 128, 1, 4, 5, 1),                             \
+        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 128, 1, 4, 5, 1),                            \
+        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 64, 1, 2, 6, 2),                              \
+        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 64, 1, 2, 6, 2),                             \
+        STREAM_INST(COMBO_, half_t, TW_, false, 64, 64, 128, 1, 4, 3, 2),                            \
+        STREAM_INST(COMBO_, half_t, TW_, true, 64, 64, 64, 1, 2, 3, 3)
 const StreamInst stream_insts[] = {
     STREAM_SET_H(1, half_t),
     STREAM_SET_H(3, fp8_t),
-    STREAM_INST(0, float, float, true, 64, 64, 64, 1, 2, 4),
-    STREAM_INST(0, float, float, true, 64, 64, 128, 1, 4, 3),
-    STREAM_INST(0, float, float, true, 128, 128, 64, 2, 2, 2),
+    // fp32: slower than the wave family on every block shape measured so far; forced use only
+    STREAM_INST(0, float, float, true, 64, 64, 64, 1, 2, 4, 0),
+    STREAM_INST(0, float, float, true, 64, 64, 128, 1, 4, 3, 0),
+    STREAM_INST(0, float, float, true, 128, 128, 64, 2, 2, 2, 0),
 };
 constexpr int N_STREAM_INSTS = sizeof(stream_insts) / sizeof(StreamInst);
 
@@ -365,6 +374,7 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int pick = -1;
     for (int i = 0; i < N_STREAM_INSTS; ++i) {
         if (want != 0x7f && want != i) continue;
+        if (want == 0x7f && stream_insts[i].per_cu == 0) continue;
         if (stream_fits(stream_insts[i], p, combo)) {
             pick = i;
             break;
@@ -377,7 +387,7 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int unit = p.bs_last ? t.epc : 1;
     const int64_t units = p.batch / unit;
     if (wgs <= 0) {
-        const int per_cu = t.lds * 2 <= 160 * 1024 ? 2 : 1;
+        const int per_cu = t.per_cu > 0 ? t.per_cu : 1;
         wgs = (256 * per_cu + groups - 1) / groups;
     }
     if (wgs > units) wgs = units;
@@ -388,7 +398,7 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_TILE;
-        tile->variant = 2000 + pick;
+        tile->variant = (2 << 24) | pick;
         tile->tile_m = t.bb;
         tile->tile_n = t.tn;
         tile->tile_k = t.cc;

@@ -398,7 +398,6 @@ const WsInst ws_insts[] = {
     WS_SET_H(3, half_t, fp8_t, false),
 };
 constexpr int N_WS_INSTS = sizeof(ws_insts) / sizeof(WsInst);
-constexpr int WS_VARIANT_BASE = 1000;
 
 bool ws_fits(const WsInst &t, const Problem &p, int combo)
 {
@@ -437,7 +436,7 @@ int ws_run(const Problem &p, int variant, int wgs_hint, bool launch, ksmm_tile *
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_TILE;
-        tile->variant = WS_VARIANT_BASE + pick;
+        tile->variant = (1 << 24) | pick;
         tile->tile_m = t.bb;
         tile->tile_n = t.tn;
         tile->tile_k = t.cc;
@@ -518,17 +517,17 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     if (combo < 0) return KSMM_ERR_BAD_DTYPE;
-    // variants >= 1000: weight-stationary kernels (bits: 1000 + instance + 100 * workgroups/group hint)
-    // variants >= 3000: batch-size-first kernels for small d > 1, see ksmm_tile_bf.hip
-    if (variant >= 3000) return tile_bf_run(p, variant - 3000, launch, tile);
-    if (variant < 0 && !p.bs_last && p.d > 1) return tile_bf_run(p, -1, launch, tile);
-    // variants >= 2000: stream kernels (direct-to-LDS pipeline), see ksmm_stream.hip
-    if (variant >= 2000) return stream_run(p, variant - 2000, launch, tile);
-    if (variant >= WS_VARIANT_BASE) {
-        const int v = variant - WS_VARIANT_BASE;
-        return ws_run(p, v % 100, v / 100, launch, tile);
-    }
-    if (variant < 0) {
+    // variant layout: bits 24-27 sub-family (0 k-loop tiles, 1 weight-stationary, 2 stream,
+    // 3 batch-size-first with d > 1), bits 0-7 instance (0xff: first that fits), bits 8-23 a
+    // sub-family parameter (persistent workgroups per block); -1: everything automatic
+    if (variant >= 0) {
+        const int sub = (variant >> 24) & 15, inst = variant & 0xff, par = (variant >> 8) & 0xffff;
+        if (sub == 3) return tile_bf_run(p, inst == 0xff ? -1 : inst, launch, tile);
+        if (sub == 2) return stream_run(p, (inst == 0xff ? 0x7f : inst) | (par << 7), launch, tile);
+        if (sub == 1) return ws_run(p, inst == 0xff ? -1 : inst, par, launch, tile);
+        variant = inst == 0xff ? -2 : inst;  // -2: heuristic among the k-loop tiles only
+    } else {
+        if (!p.bs_last && p.d > 1) return tile_bf_run(p, -1, launch, tile);
         int rc = stream_run(p, -1, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
         rc = ws_run(p, -1, 0, launch, tile);
@@ -537,7 +536,7 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int pick = -1;
     if (variant >= 0) {
         if (variant < N_TILE_INSTS && tile_fits(tile_insts[variant], p, combo)) pick = variant;
-    } else {
+    } else {  // -1 or -2
         // heuristic: the largest TM that divides b (fewest re-reads of the input), then a batch
         // tile that still leaves >= 2 workgroups per CU
         int64_t best_score = -1;

@@ -252,7 +252,7 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_TILE;
-        tile->variant = 3000 + pick;
+        tile->variant = (3 << 24) | pick;
         tile->tile_m = t.tm;
         tile->tile_n = t.tn;
         tile->tile_k = t.tk;

@@ -383,12 +383,13 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if ((int64_t)(4 * in.kl + 1) * p.d * p.batch * 4 >= 0xffffffffLL) return KSMM_ERR_BAD_ALGO;
     const int tn = 16 * in.vec;
     const int64_t n_tiles = (p.batch + tn - 1) / tn;
-    // columns per wave: enough wave-iterations to amortise the weight load, while keeping
-    // several waves per SIMD busy on all 256 CUs
+    // Columns per wave: about one wave per SIMD (256 CUs x 4) over the whole problem, so that
+    // every wave amortises its weight load and runs its register pipeline over several tiles;
+    // measured best on (1,48,48,16) fp32 and flat elsewhere.  At most 8 tiles per wave.
     const int64_t groups = (int64_t)p.a * p.d;
     if (iters == 0) {
-        iters = 4;
-        while (iters > 1 && groups * ((n_tiles + iters - 1) / iters) < 256 * 4 * 4) iters >>= 1;
+        int64_t it = groups * n_tiles / 1024;
+        iters = (int)(it < 1 ? 1 : (it > 8 ? 8 : it));
     }
     const int64_t n_slabs = (n_tiles + iters - 1) / iters;
     const int64_t waves = groups * n_slabs;
