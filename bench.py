@@ -180,6 +180,23 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
     return result
 
 
+def copy_reference(steps, warmup):
+    """Plain elementwise stream (y = x + 1) over the headline workload's bytes (77 MB in, 77 MB out) with
+    the same buffer rotation and timing: what this particular GPU sustains for the simplest
+    read+write stream, next to the 8 TB/s datasheet figure."""
+    n_sets = 4
+    src = [torch.randn(768, BATCH, device="cuda") for _ in range(n_sets)]
+    dst = [torch.empty_like(t) for t in src]
+
+    def run(j):
+        torch.add(src[j], 1.0, out=dst[j])  # one elementwise kernel: 1 read + 1 write stream
+
+    sec = time_launches(run, n_sets, steps, warmup)
+    nbytes = 2 * src[0].numel() * 4
+    return {"us": sec * 1e6, "gbs": nbytes / sec / 1e9, "frac_of_8tbs": nbytes / sec / 8e12,
+            "bytes": nbytes, "kernel": "torch.add(x, 1, out=y) elementwise kernel"}
+
+
 def cpu_baseline(patterns, bs_last, budget_s=12.0):
     """The reference's algo='bmm' CPU algorithm (restated in oracle/), fp32, on all host
     cores; protocol of the reference's ksmm_time.py: blocked_autorange(min_run_time=0.25),
@@ -216,6 +233,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--all", type=int, default=1, help="also time the other configurations")
     ap.add_argument("--cpu", type=int, default=1, help="time the CPU baseline")
+    ap.add_argument("--copy-calib", type=int, default=0,
+                    help="also run N plain device copies of 77 MB (counter calibration for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU (the KS path shards on the batch axis without "
@@ -229,6 +248,14 @@ def main():
 
     _lib.load()  # fails loudly if the HIP library is missing
     t_start = time.time()
+    if args.copy_calib:
+        # a copy kernel of known size (read 77 070 336 B, write 77 070 336 B) so that HBM byte
+        # counters of a profiling run can be scaled
+        src = torch.randn(768, BATCH, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.copy_calib):
+            torch.add(src, 1.0, out=dst)  # one elementwise kernel per call: 1 read + 1 write stream
+        torch.cuda.synchronize()
     head = bench_config(*CONFIGS[0], steps=args.steps, warmup=args.warmup)
     sec = head["factors"][0]["us"] / 1e6
     roof = factor_roofline(BATCH, CONFIGS[0][1][0], torch.float32, torch.float32, torch.float32, sec)
@@ -236,6 +263,7 @@ def main():
     if args.all:
         for cfg in CONFIGS[1:]:
             others.append(bench_config(*cfg, steps=max(20, args.steps // 2), warmup=max(5, args.warmup // 2)))
+    copy_ref = copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
     line = {
         "metric": "us_per_ks_factor", "value": head["factors"][0]["us"], "unit": "us",
@@ -247,6 +275,7 @@ def main():
         "roofline": {"bound": roof["bound"], "achieved": roof["achieved"], "peak": roof["peak"],
                      "unit": roof["unit"], "frac": roof["frac"], "traffic": None},
         "cpu_baseline": cpu,
+        "copy_reference": copy_ref,
         "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),
                    "ok": head.get("parity_ok")},
         "configs": [head] + others,
