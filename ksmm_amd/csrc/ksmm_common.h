@@ -93,6 +93,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);
 int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the wave family
+int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 
 }  // namespace ksmm

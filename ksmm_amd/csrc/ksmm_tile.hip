@@ -518,17 +518,20 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     if (combo < 0) return KSMM_ERR_BAD_DTYPE;
     // variant layout: bits 24-27 sub-family (0 k-loop tiles, 1 weight-stationary, 2 stream,
-    // 3 batch-size-first with d > 1), bits 0-7 instance (0xff: first that fits), bits 8-23 a
+    // 3 batch-size-first with d > 1, 4 direct-to-LDS GEMM), bits 0-7 instance (0xff: first that fits), bits 8-23 a
     // sub-family parameter (persistent workgroups per block); -1: everything automatic
     if (variant >= 0) {
         const int sub = (variant >> 24) & 15, inst = variant & 0xff, par = (variant >> 8) & 0xffff;
+        if (sub == 4) return gemm_run(p, inst == 0xff ? -1 : inst, launch, tile);
         if (sub == 3) return tile_bf_run(p, inst == 0xff ? -1 : inst, launch, tile);
         if (sub == 2) return stream_run(p, (inst == 0xff ? 0x7f : inst) | (par << 7), launch, tile);
         if (sub == 1) return ws_run(p, inst == 0xff ? -1 : inst, par, launch, tile);
         variant = inst == 0xff ? -2 : inst;  // -2: heuristic among the k-loop tiles only
     } else {
+        int rc = gemm_run(p, -1, launch, tile);  // large blocks: matrix-core-bound
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
         if (!p.bs_last && p.d > 1) return tile_bf_run(p, -1, launch, tile);
-        int rc = stream_run(p, -1, launch, tile);
+        rc = stream_run(p, -1, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
         rc = ws_run(p, -1, 0, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;

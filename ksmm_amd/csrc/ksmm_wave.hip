@@ -26,6 +26,19 @@
 
 #include "ksmm_common.h"
 
+#ifdef KSMM_PROFILE
+// Phase timestamps of wave 0 of every workgroup (standalone profiling builds only).
+__device__ unsigned long long ksmm_wprof[2048][40];
+#define KW_STAMP(slot)                                                                           \
+    do {                                                                                         \
+        if (threadIdx.x == 0 && blockIdx.x < 2048 && (slot) < 40)                                \
+            ksmm_wprof[blockIdx.x][(slot)] = ((slot) < 2) ? __builtin_amdgcn_s_memrealtime()     \
+                                                          : __builtin_amdgcn_s_memtime();        \
+    } while (0)
+#else
+#define KW_STAMP(slot) do { } while (0)
+#endif
+
 namespace ksmm {
 
 namespace {
@@ -117,6 +130,8 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     if (g >= a * d) return;
     const int slab = wave - g * n_slabs;
     const int a_i = g / d, d_i = g - a_i * d;
+    KW_STAMP(0);
+    KW_STAMP(2);
 
     // weights -> A operands, once per wave
     float areg[MT][KS];
@@ -126,6 +141,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = wg[(4 * ks + q) * b + 16 * mt + r];
+#ifdef KSMM_ABL_NOW
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = (float)(ks + mt + lane);
+#endif
     }
     // Addressing: uniform (scalar) row base + one 32-bit per-lane byte offset, so that the
     // loads and stores need no per-row vector address registers.  The host checks that the
@@ -155,6 +176,8 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     // Everything issued so far (weights, first tile) is complete before the loop, so that the
     // waits inside the loop only ever count that loop's own loads and stores.
     __builtin_amdgcn_s_waitcnt(0);
+    KW_STAMP(3);
+    int kw_slot = 4;
     const int n_last = n_first + ((n_end - n_first - 1) / TN) * TN;  // first column of the last tile
     // FULL tiles store without a predicate, which keeps the loop body free of branches; a
     // ragged last tile (batch not a multiple of the tile) runs once more with the predicate.
@@ -168,15 +191,23 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
             for (int v = 0; v < VEC; ++v) acc[mt][v] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
+#ifdef KSMM_ABL_NOMFMA
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][v][ks & 3] += areg[mt][ks] + xc[ks][v];
+#else
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     acc[mt][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[mt][ks], xc[ks][v],
                                                                       acc[mt][v], 0, 0, 0);
+#endif
             xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + next_off);
             __builtin_amdgcn_sched_barrier(0);  // keep the refill between the MFMA groups
         }
+        KW_STAMP(kw_slot);
         const int col = n0 + VEC * r;
         if (decltype(full)::value || col < batch) {
             const uint32_t off = y_lane + (uint32_t)col * 4u;
@@ -189,10 +220,15 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
                     *(float4_t *)(yg + (size_t)(16 * mt + i) * row_stride * 4 + off) = o;
                 }
         }
+        KW_STAMP(kw_slot + 1);
+#ifdef KSMM_PROFILE
+        kw_slot += 2;
+#endif
     };
     int n0 = n_first;
     for (; n0 + TN <= n_end; n0 += TN) do_tile(n0, std::true_type{});
     if (n0 < n_end) do_tile(n0, std::false_type{});
+    KW_STAMP(1);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -72,6 +72,34 @@ def test_factor_small(prec, bs_last, algo):
         pytest.skip("family %s takes none of the small problems for %s" % (algo, prec))
 
 
+def test_gemm_kernels_forced():
+    """Every instance of the direct-to-LDS GEMM sub-family (tile variant 4<<24 | i), forced on
+    shapes with batch tails, several blocks per factor and d > 1."""
+    from ksmm_amd import Kernel, generate_factor, _lib
+
+    cases = [("fp16", True, (2, 256, 64, 3)), ("fp16", False, (2, 256, 64, 1)), ("fp16", False, (2, 256, 64, 2)),
+             ("fp16", False, (1, 128, 128, 2)), ("fp32", True, (1, 256, 64, 2)), ("fp32", True, (2, 128, 32, 1))]
+    ran = 0
+    for prec, bs_last, pattern in cases:
+        a, b, c, d = pattern
+        for batch in (1000, 264):
+            (w4,) = seeded_weights([pattern], seed=21)
+            x = seeded_input(a * c * d, batch, bs_last, seed=22)
+            dt = TORCH_DTYPE[prec]
+            fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+            z = O.ks_apply_einsum(round_to(w4, prec)[0], round_to(x, prec)[0], bs_last)
+            for inst in range(32):
+                try:
+                    y = Kernel.forward(x.to(dt).cuda(), fac, bs_last, a, b, c, d, algo=3, variant=(4 << 24) | inst)
+                except _lib.KsmmError as e:
+                    assert e.status == -6
+                    continue
+                ran += 1
+                err = O.rel_fro_error(y.float().cpu().numpy(), z)
+                assert err <= TOL[prec], (prec, bs_last, pattern, batch, inst, err)
+    assert ran >= 12
+
+
 def test_fp16_input_fp8_weight_factor():
     """Chain intermediate type: fp16 activations times e4m3fn weights."""
     from ksmm_amd import Kernel, generate_factor, quantize_fp8
