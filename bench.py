@@ -143,13 +143,16 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
     if len(patterns) > 1:
         ws_bytes = torch.empty(2 * (widest * BATCH * 4 + 256), dtype=torch.uint8, device="cuda")
 
-        def run_chain(j):
+        def run_chain(j, fuse=True):
             sc = list(wscales)
             sc[0] *= scales[j]
-            return Kernel.chain_forward(xs[j], facs, patterns, bs_last, scales=sc, workspace=ws_bytes)
+            return Kernel.chain_forward(xs[j], facs, patterns, bs_last, scales=sc, fuse=fuse,
+                                        workspace=ws_bytes)
 
         sec = time_launches(run_chain, n_sets, max(3, steps // 2), max(1, warmup // 2))
         result["kslinear_us"] = sec * 1e6
+        sec = time_launches(lambda j: run_chain(j, False), n_sets, max(3, steps // 2), max(1, warmup // 2))
+        result["kslinear_unfused_us"] = sec * 1e6
         final = run_chain(0)
     else:
         result["kslinear_us"] = result["factors"][0]["us"]

@@ -168,7 +168,12 @@ int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const voi
     if (!x || !y) return KSMM_ERR_NULL_POINTER;
     for (int i = 0; i < n_factors; ++i)
         if (!factors[i].w) return KSMM_ERR_NULL_POINTER;
-    (void)fuse;
+    if (fuse) {
+        // chains whose intermediates fit LDS run as one kernel (no workspace traffic)
+        rc = chain16_run(factors, n_factors, x, y, batch, x_dtype, y_dtype, bs_last ? 1 : 0, true,
+                         (hipStream_t)stream);
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
+    }
     const int64_t need = ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
     if (n_factors > 1 && (!workspace || workspace_bytes < need)) return KSMM_ERR_WORKSPACE;
     char *buf[2] = {(char *)workspace, (char *)workspace + need / 2};

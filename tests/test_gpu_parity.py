@@ -164,6 +164,38 @@ def test_config_full_batch(name):
             assert O.rel_fro_error(y2.float().cpu().numpy(), 2 * yh) <= 2e-3
 
 
+@pytest.mark.parametrize("prec", ["fp8", "fp16"])
+def test_fused_radix16_chain_matches_unfused_and_oracle(prec):
+    """The LDS-resident fused chain (all factors b = c = 16) against the factor-by-factor launch
+    and the oracle, on 2-, 3- and 4-factor chains and ragged batch sizes."""
+    from ksmm_amd import KSLinear
+
+    chains = [[(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)],
+              [(4, 16, 16, 4), (16, 16, 16, 1)],
+              [(1, 16, 16, 32), (2, 16, 16, 16), (8, 16, 16, 4), (32, 16, 16, 1)],
+              [(64, 16, 16, 1), (1, 16, 16, 64)]]
+    for patterns in chains:
+        n_feat = patterns[0][0] * 16 * patterns[0][3]
+        for batch in (16, 80, 1000 if prec == "fp16" else 1008, 4096 + 48):
+            ws4 = seeded_weights(patterns, seed=31, bound=0.25)
+            x = seeded_input(n_feat, batch, True, seed=32)
+            outs = {}
+            for fuse in (True, False):
+                ksl = KSLinear(patterns, weights=ws4, bias=False, algo="kernel", dtype=TORCH_DTYPE[prec],
+                               bs_last=True, device="cuda", fuse=fuse)
+                if prec == "fp8":
+                    xr, xq, xs = round_to(x, prec)
+                    outs[fuse] = ksl(xq.cuda(), x_scale=xs).float().cpu().numpy()
+                else:
+                    xr = round_to(x, prec)[0]
+                    outs[fuse] = ksl(x.half().cuda()).float().cpu().numpy()
+            wr = [round_to(w, prec)[0] for w in ws4]
+            z = oracle_chain(wr, xr, True)
+            assert O.rel_fro_error(outs[True], z) <= TOL[prec], (patterns, batch, "fused")
+            assert O.rel_fro_error(outs[False], z) <= TOL[prec], (patterns, batch, "unfused")
+            assert O.rel_fro_error(outs[True], outs[False]) <= 2e-3, (patterns, batch)
+
+
 def test_layouts_agree_full_batch():
     """bs_last result == transposed bs_first result (same weights, fp32, C2 at full batch)."""
     from ksmm_amd import KSLinear
