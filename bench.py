@@ -229,6 +229,17 @@ def cpu_baseline(patterns, bs_last, budget_s=12.0):
             "mean_us": m.mean * 1e6, "iqr_us": m.iqr * 1e6, "host_cpu_count": os.cpu_count()}
 
 
+# HBM bytes per launch of the headline kernel, ks_wave_bl_f32<3,12,2> on (1,48,48,16) fp32 bs_last
+# at B = 25088, from two counter passes over this script
+#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 20 --warmup 5 --cpu 0 --copy-calib 10
+#   rocprofv3 --pmc WRITE_SIZE -- python3 bench.py --steps 20 --warmup 5 --cpu 0 --copy-calib 10
+# FETCH_SIZE 39152.9 KiB and WRITE_SIZE 75264.0 KiB per dispatch, each divided by what the same
+# counter reads for the torch.add calibration kernel per KiB it moves (0.5002 and 1.0000).
+# Counters cannot be collected from inside a timed run, so the figure is carried here; it
+# belongs to that kernel and workload only and is dropped if another kernel is dispatched.
+MEASURED_TRAFFIC = {"algo": 2, "variant": 0, "bytes": int((39152.9 / 0.5002 + 75264.0 / 1.0) * 1024)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -262,6 +273,9 @@ def main():
     head = bench_config(*CONFIGS[0], steps=args.steps, warmup=args.warmup)
     sec = head["factors"][0]["us"] / 1e6
     roof = factor_roofline(BATCH, CONFIGS[0][1][0], torch.float32, torch.float32, torch.float32, sec)
+    hf = head["factors"][0]
+    traffic = (MEASURED_TRAFFIC["bytes"]
+               if (hf["algo"], hf["variant"]) == (MEASURED_TRAFFIC["algo"], MEASURED_TRAFFIC["variant"]) else None)
     others = []
     if args.all:
         for cfg in CONFIGS[1:]:
@@ -276,7 +290,7 @@ def main():
         "config": {"workload": "single KS factor (1,48,48,16) 768->768, fp32, bs_last, B=25088",
                    "batch": BATCH, "pattern": [1, 48, 48, 16], "layout": "bs_last"},
         "roofline": {"bound": roof["bound"], "achieved": roof["achieved"], "peak": roof["peak"],
-                     "unit": roof["unit"], "frac": roof["frac"], "traffic": None},
+                     "unit": roof["unit"], "frac": roof["frac"], "traffic": traffic},
         "cpu_baseline": cpu,
         "copy_reference": copy_ref,
         "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),
