@@ -115,7 +115,7 @@ template <> struct mfma16<8> {
 // fp32: v_mfma_f32_16x16x4_f32, VEC = 4 (16-byte loads and stores)
 // MT = b / 16, KS = c / 4.  Each wave iteration covers 64 batch columns.
 // ------------------------------------------------------------------------------------------
-template <int MT, int KS, int OCC>
+template <int MT, int KS, int OCC, bool ROLL>
 __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restrict__ x,
                                                      const float *__restrict__ w,
                                                      float *__restrict__ y, int batch, int a, int b,
@@ -204,8 +204,10 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
                     acc[mt][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[mt][ks], xc[ks][v],
                                                                       acc[mt][v], 0, 0, 0);
 #endif
-            xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + next_off);
-            __builtin_amdgcn_sched_barrier(0);  // keep the refill between the MFMA groups
+            if constexpr (ROLL) {
+                xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + next_off);
+                __builtin_amdgcn_sched_barrier(0);  // keep the refill between the MFMA groups
+            }
         }
         KW_STAMP(kw_slot);
         const int col = n0 + VEC * r;
@@ -235,7 +237,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
 // 16-bit MFMA path: x is fp16 or e4m3fn (decoded to fp16, exact), w is fp16 or e4m3fn,
 // y is fp16.  MT = b / 16, KS = c / (4 * KL).  Each wave iteration covers 16 * VEC columns.
 // ------------------------------------------------------------------------------------------
-template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC>
+template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC, bool ROLL>
 __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ x,
                                                    const TW *__restrict__ w,
                                                    half_t *__restrict__ y, int batch, int a, int b,
@@ -301,10 +303,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
             uint32_t xh[KL][VEC / 2];  // fp16 pairs: columns (2i, 2i+1) of row jj
 #pragma unroll
             for (int jj = 0; jj < KL; ++jj) io::unpack(raw[ks][jj], xh[jj]);
+            if constexpr (ROLL) {
 #pragma unroll
-            for (int jj = 0; jj < KL; ++jj)
-                io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + next_off),
-                         raw[ks][jj]);
+                for (int jj = 0; jj < KL; ++jj)
+                    io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + next_off),
+                             raw[ks][jj]);
+            }
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
                 // KL consecutive k of batch column VEC*r + v: in-register transpose
@@ -321,7 +325,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
                 for (int mt = 0; mt < MT; ++mt)
                     acc[mt][v] = mfma16<KL>::run(areg[mt][ks], bf, acc[mt][v]);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (ROLL) __builtin_amdgcn_sched_barrier(0);
         }
         const int col = n0 + VEC * r;
         if (decltype(full)::value || col < batch) {
@@ -350,7 +354,8 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
 // ---- instance table ---------------------------------------------------------------------
 struct WaveInst {
     int b, c, vec, kl, occ;
-    const void *fn;
+    const void *fn;       // several tiles per wave, rolling register pipeline
+    const void *fn_once;  // one tile per wave: nothing is reloaded
 };
 
 typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, float, int, int);
@@ -359,7 +364,8 @@ using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int,
 
 // OCC_ = minimum waves per SIMD the register allocation must allow
 #define F32_INST(B_, C_, OCC_) \
-    {B_, C_, 4, 1, OCC_, (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_>}
+    {B_, C_, 4, 1, OCC_, (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_, true>, \
+     (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_, false>}
 const WaveInst f32_insts[] = {
     F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
     F32_INST(16, 16, 4), F32_INST(32, 32, 3),
@@ -367,7 +373,8 @@ const WaveInst f32_insts[] = {
 
 #define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_)                           \
     {B_, C_, VEC_, KL_, OCC_,                                               \
-     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_>}
+     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, true>, \
+     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, false>}
 #define H_SET(TX_, TW_)                                                                      \
     H_INST(TX_, TW_, 64, 64, 8, 4, 2), H_INST(TX_, TW_, 64, 64, 8, 8, 2),                    \
         H_INST(TX_, TW_, 64, 64, 8, 8, 1), H_INST(TX_, TW_, 48, 48, 4, 4, 3),                \
@@ -378,8 +385,8 @@ const WaveInst h_insts[] = {H_SET(half_t, half_t)};
 const WaveInst hq_insts[] = {H_SET(half_t, fp8_t)};
 const WaveInst q_insts[] = {
     H_INST(fp8_t, fp8_t, 64, 64, 8, 8, 2),  H_INST(fp8_t, fp8_t, 64, 64, 8, 8, 1),
-    H_INST(fp8_t, fp8_t, 48, 48, 4, 8, 2),  H_INST(fp8_t, fp8_t, 16, 16, 4, 16, 3),
-    H_INST(fp8_t, fp8_t, 16, 16, 4, 8, 4),  H_INST(fp8_t, fp8_t, 32, 32, 8, 16, 2),
+    H_INST(fp8_t, fp8_t, 48, 48, 4, 8, 2),  H_INST(fp8_t, fp8_t, 16, 16, 4, 8, 4),
+    H_INST(fp8_t, fp8_t, 16, 16, 4, 16, 3), H_INST(fp8_t, fp8_t, 32, 32, 8, 16, 2),
     H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),
 };
 
@@ -389,7 +396,6 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     // batch-size-first: the register-stationary row kernel (variants >= 1000), d > 1 only
     if (!p.bs_last) return rows_bf_run(p, variant >= 1000 ? variant - 1000 : -1, launch, tile);
-    if (variant >= 1000) return KSMM_ERR_BAD_ALGO;
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     const WaveInst *insts;
     int n_insts;
@@ -419,17 +425,21 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if ((int64_t)(4 * in.kl + 1) * p.d * p.batch * 4 >= 0xffffffffLL) return KSMM_ERR_BAD_ALGO;
     const int tn = 16 * in.vec;
     const int64_t n_tiles = (p.batch + tn - 1) / tn;
-    // Columns per wave: about one wave per SIMD (256 CUs x 4) over the whole problem, so that
-    // every wave amortises its weight load and runs its register pipeline over several tiles;
-    // measured best on (1,48,48,16) fp32 and flat elsewhere.  At most 8 tiles per wave.
+    // Tiles per wave.  Small blocks (16x16, 32x32) have little matrix work per byte: one tile
+    // per wave and many waves in flight measured best.  Larger blocks keep a SIMD's matrix pipe
+    // busy for microseconds per tile; there a single round of workgroups (at most one per CU,
+    // 4 waves each) with the rolling pipeline over several tiles is best, and a few workgroups
+    // beyond 256 double the run time (two share a CU while the others have finished): take the
+    // smallest count that fits one round.
     const int64_t groups = (int64_t)p.a * p.d;
+    const int wpb = 4;
     if (iters == 0) {
-        int64_t it = groups * n_tiles / 1024;
-        iters = (int)(it < 1 ? 1 : (it > 8 ? 8 : it));
+        iters = 1;
+        if (p.b * p.c > 1024)
+            while (iters < 255 && (groups * ((n_tiles + iters - 1) / iters) + wpb - 1) / wpb > 256) ++iters;
     }
     const int64_t n_slabs = (n_tiles + iters - 1) / iters;
     const int64_t waves = groups * n_slabs;
-    const int wpb = 4;
     const int64_t blocks = (waves + wpb - 1) / wpb;
     if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
@@ -450,7 +460,8 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     args[3] = &batch_i;
     args[9] = &n_slabs_i;
     args[10] = &iters;
-    hipError_t e = hipLaunchKernel(in.fn, dim3((unsigned)blocks), dim3(64 * wpb), args, 0, p.stream);
+    const void *fn = iters == 1 ? in.fn_once : in.fn;
+    hipError_t e = hipLaunchKernel(fn, dim3((unsigned)blocks), dim3(64 * wpb), args, 0, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
