@@ -1,6 +1,6 @@
 // "Stream" kernels of the tile family: the bandwidth-bound path for mid-sized b x c blocks.
 //
-// A persistent workgroup owns one (a_i, d_i) block and an equal share of the batch columns.
+// A persistent workgroup owns one (a_i, d_i) block and every wgs-th tile of batch columns.
 // The b x c weight block is staged through LDS once and then lives in registers as MFMA
 // operands.  Input tiles (the whole c extent x TN batch columns) are brought in with
 // direct-to-LDS loads (global_load_lds_dwordx4: no staging registers), ST tiles deep, so that
@@ -140,15 +140,18 @@ template <typename CT, typename TW, typename TY, bool BS_LAST, int BB, int CC, i
 __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__restrict__ x,
                                                                 const TW *__restrict__ w,
                                                                 TY *__restrict__ y, int batch, int a,
-                                                                int d, float scale, int wgs_per_group,
-                                                                int share)
+                                                                int d, float scale, int wgs_per_group)
 {
     typedef StreamCfg<CT, TW, BS_LAST, BB, CC, TN, WM, WN, ST> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int g = blockIdx.x / wgs_per_group;  // a_i * d + d_i
     const int s = blockIdx.x - g * wgs_per_group;
-    const int c_begin = s * share, c_end = min(batch, c_begin + share);  // this workgroup's columns
-    if (c_begin >= c_end) return;
+    // Tiles of TN batch columns (rows for bs_first), dealt round-robin over the workgroups of
+    // the block: at any time the workgroups of a block work on neighbouring tiles, so the row
+    // pieces in flight are contiguous in memory (and TN-aligned).
+    const int n_tiles = (batch + TN - 1) / TN;
+    if (s >= n_tiles) return;
+    const int c_begin = s * TN, c_end = batch, step = wgs_per_group * TN;
     const int a_i = g / d, d_i = g - a_i * d;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -191,13 +194,11 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
 
     CT *const out = (CT *)smem;
     const int l32 = lane & 31, lq = lane >> 5;
-    const int n_iters = (c_end - c_begin + TN - 1) / TN;
-    // prologue: ST-1 tiles in flight (tiles past the end repeat the last one; never read)
-#pragma unroll
-    for (int p = 0; p < ST - 1; ++p) issue(c_begin + min(p, n_iters - 1) * TN, p);
-    KS_STAMP(1);
-
+    const int n_iters = (n_tiles - s + wgs_per_group - 1) / wgs_per_group;
     // ---- weights: global -> LDS (as stored, c x b, padded rows) -> registers ---------------
+    // Their loads go out before the input tiles' so that they are not queued behind them; the
+    // prologue tiles (ST-1 in flight; tiles past the end repeat the last one and are never
+    // read) follow at once, and staging the weights overlaps with their flight.
     {
         CT *wl = (CT *)smem;
         const TW *wg = w + (size_t)g * CC * BB;
@@ -209,6 +210,9 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
             const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
             r[i].load(wg + (size_t)(v / (BB / C::W_EPV)) * BB + (v % (BB / C::W_EPV)) * C::W_EPV);
         }
+#pragma unroll
+        for (int p = 0; p < ST - 1; ++p) issue(c_begin + min(p, n_iters - 1) * step, p);
+        KS_STAMP(1);
 #pragma unroll
         for (int i = 0; i < W_PER_T; ++i) {
             const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
@@ -227,8 +231,9 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
 
 
     for (int it = 0; it < n_iters; ++it) {
-        const int n0 = c_begin + it * TN;
-        issue(c_begin + min(it + ST - 1, n_iters - 1) * TN, (it + ST - 1) % ST);
+        const int n0 = c_begin + it * step;
+        const int n_stop = min(n0 + TN, c_end);  // columns (rows) this tile stores
+        issue(c_begin + min(it + ST - 1, n_iters - 1) * step, (it + ST - 1) % ST);
         if (it >= ST - 1)
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_FULL));
         else
@@ -298,12 +303,12 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
             if (BS_LAST) {
                 const int n = n0 + oc;
                 TY *dst = y + ((size_t)(a_i * BB + orow) * d + d_i) * batch + min(n, c_end - C::EPC);
-                if (n < c_end) *(uint4_t *)dst = v;  // 128/256-byte row pieces: plain stores measured faster
+                if (n < n_stop) *(uint4_t *)dst = v;  // 128/256-byte row pieces: plain stores measured faster
             } else {
                 const int n = n0 + orow;
                 TY *dst = y + (size_t)min(n, c_end - 1) * out_size + (size_t)a_i * BB + oc;
                 // whole rows of b outputs: streaming (nontemporal) stores measured faster
-                if (n < c_end) __builtin_nontemporal_store(v, (uint4_t *)dst);
+                if (n < n_stop) __builtin_nontemporal_store(v, (uint4_t *)dst);
             }
         }
         KS_STAMP(7 + 4 * it);
@@ -384,16 +389,13 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const StreamInst &t = stream_insts[pick];
     const int64_t groups = (int64_t)p.a * p.d;
     // bs_last shares are column ranges (multiples of the 16-byte vector), bs_first shares are rows
-    const int unit = p.bs_last ? t.epc : 1;
-    const int64_t units = p.batch / unit;
     if (wgs <= 0) {
         const int per_cu = t.per_cu > 0 ? t.per_cu : 1;
         wgs = (256 * per_cu + groups - 1) / groups;
     }
-    if (wgs > units) wgs = units;
     if (wgs < 1) wgs = 1;
-    const int64_t share = (units + wgs - 1) / wgs * unit;
-    wgs = (p.batch + share - 1) / share;
+    const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
+    if (wgs > n_tiles) wgs = n_tiles;
     const int64_t grid = groups * wgs;
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
@@ -412,9 +414,9 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
             return KSMM_ERR_LAUNCH;
     }
-    int batch_i = (int)p.batch, wgs_i = (int)wgs, share_i = (int)share;
+    int batch_i = (int)p.batch, wgs_i = (int)wgs;
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
-                    (void *)&p.scale, &wgs_i, &share_i};
+                    (void *)&p.scale, &wgs_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
