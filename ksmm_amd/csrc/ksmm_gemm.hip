@@ -47,9 +47,29 @@ constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | (((n >
 
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr)
 {
+#ifdef KSMM_GABL_NODMA
+    if (lds_addr != 0xffffffffu) return;
+#endif
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(gptr), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+#ifdef KSMM_GABL_NOMFMA
+__device__ __forceinline__ float abl_first(float v) { return v; }
+__device__ __forceinline__ float abl_first(half8_t v) { return (float)v[0] + (float)v[7]; }
+#endif
+
+// the same with a uniform 64-bit base (SGPR pair) and a 32-bit per-lane byte offset
+__device__ __forceinline__ void dma16s(const void *sbase, uint32_t voff, uint32_t lds_addr)
+{
+#ifdef KSMM_GABL_NODMA
+    if (lds_addr != 0xffffffffu) return;
+#endif
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_addr)
                  : "memory", "m0");
 }
 
@@ -72,38 +92,63 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
     static_assert(ES == 2 || BS_LAST, "fp32 batch-size-first uses the plain tile kernel");
     static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0 && TK % KSTEP == 0, "wave tiling");
     static_assert(W_CHUNKS % THREADS == 0 && X_CHUNKS % THREADS == 0, "every wave issues L loads per slab");
-    static_assert(W_CPR % (ES == 2 ? 8 : 16) == 0, "weight swizzle group");
-    static_assert(BS_LAST ? X_CPR % (ES == 2 ? 8 : 16) == 0 : (X_CPR == 4 || X_CPR % 8 == 0), "input swizzle group");
+    static_assert(ES == 2 ? (W_CPR == 8 || W_CPR % 16 == 0) : W_CPR % 16 == 0, "weight swizzle group");
+    static_assert(BS_LAST ? (ES == 2 ? (X_CPR == 8 || X_CPR % 16 == 0) : X_CPR % 16 == 0) : (X_CPR == 4 || X_CPR == 8 || X_CPR % 16 == 0), "input swizzle group");
     static_assert(ST >= 2 && N_WAIT <= 63 && LDS_BYTES <= 160 * 1024, "ring");
     static_assert(DD * MT * NT * 16 <= 256, "accumulators");
 };
 
 // chunk swizzles (applied to the global address a lane fetches and by the operand reads)
-template <typename CT> __device__ __forceinline__ int swz_outer(int row) { return sizeof(CT) == 2 ? 2 * (row & 3) : 8 * (row & 1); }
-template <int CPR> __device__ __forceinline__ int swz_inner(int row) { return CPR == 4 ? ((row >> 2) & 3) : (row & 7); }
+// LDS has 64 banks of 4 bytes: a ds_read_b64 is served 32 lanes per clock and a ds_read_b128
+// 16 lanes per clock, conflict-free when those lanes cover 256 bytes of distinct banks.
+//  k-outer fp16 rows (CPR chunks of 16 bytes): the 32 lanes of a transpose load read 4 rows x
+//  64 bytes -> XOR the 64-byte group index with row & 3 (32-byte groups when a row has only 8).
+//  k-outer fp32: 2 rows x 128 bytes per ds_read_b32 wave -> XOR the 128-byte half with row & 1.
+//  k-inner rows: 16 lanes read one chunk of 16 consecutive rows -> XOR the chunk so that the
+//  rows sharing a 256-byte bank line differ (rows of 64, 128, >= 256 bytes).
+template <typename CT, int CPR> __device__ __forceinline__ int swz_outer(int row)
+{
+    return sizeof(CT) == 2 ? (CPR >= 16 ? 4 : 2) * (row & 3) : 8 * (row & 1);
+}
+template <int CPR> __device__ __forceinline__ int swz_inner(int row)
+{
+    return CPR == 4 ? ((row >> 2) & 3) : CPR == 8 ? ((row >> 1) & 7) : (row & 15);
+}
 
-// k-outer operand (weights always, input for bs_last): S[k][idx], row of COLS elements
+// k-outer operand (weights always, input for bs_last): S[k][idx], row of COLS elements.
+// The address of a fragment is (per-lane byte offset, fixed for the kernel) + (stage base,
+// uniform) + (k0 * row bytes, a compile-time constant that goes into the instruction's offset
+// field): outer_off gives the first, outer_read takes the sum of the first two.
+typedef __attribute__((address_space(3))) unsigned char *lds_bytes_t;
 template <typename CT, int COLS> struct outer_frag;
 template <int COLS> struct outer_frag<half_t, COLS> {
-    __device__ static __forceinline__ half8_t get(const half_t *s, int idx0, int k0, int lane)
+    __device__ static __forceinline__ uint32_t off(int idx0, int lane)
     {
         const int kq = lane >> 5, i16 = lane & 15, hs = (lane >> 4) & 1;
-        const int row = k0 + 8 * kq + (i16 >> 2);
+        const int row = 8 * kq + (i16 >> 2);  // + k0 (a multiple of 16): same row & 3
         const int chunk = (idx0 >> 3) + 2 * hs + ((i16 & 3) >> 1);
-        const half_t *p = s + row * COLS + ((chunk ^ (2 * ((i16 >> 2) & 3))) << 3) + 4 * (i16 & 1);
+        return (uint32_t)(row * COLS * 2 + ((chunk ^ swz_outer<half_t, COLS / 8>(row)) << 4) + 8 * (i16 & 1));
+    }
+    __device__ static __forceinline__ half8_t read(uint32_t addr, int k0)
+    {
         typedef short4_t __attribute__((address_space(3))) * lds_ptr;
-        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
-        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * COLS));
+        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(lds_bytes_t)(uintptr_t)(addr + k0 * COLS * 2));
+        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(lds_bytes_t)(uintptr_t)(addr + (k0 + 4) * COLS * 2));
         typedef short short8_t __attribute__((ext_vector_type(8)));
         short8_t r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return __builtin_bit_cast(half8_t, r);
     }
 };
 template <int COLS> struct outer_frag<float, COLS> {
-    __device__ static __forceinline__ float get(const float *s, int idx0, int k0, int lane)
+    __device__ static __forceinline__ uint32_t off(int idx0, int lane)
     {
-        const int row = k0 + (lane >> 5), col = idx0 + (lane & 31);
-        return s[row * COLS + ((((col >> 2) ^ (8 * (row & 1))) << 2) | (col & 3))];
+        const int row = lane >> 5, col = idx0 + (lane & 31);  // + k0 (even): same row & 1
+        return (uint32_t)((row * COLS + ((((col >> 2) ^ (8 * (row & 1))) << 2) | (col & 3))) * 4);
+    }
+    __device__ static __forceinline__ float read(uint32_t addr, int k0)
+    {
+        typedef __attribute__((address_space(3))) float *lds_ptr;
+        return *(lds_ptr)(lds_bytes_t)(uintptr_t)(addr + k0 * COLS * 4);
     }
 };
 
@@ -131,41 +176,60 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     const int wm = wave / WN, wn = wave % WN;
     const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
 
-    // ---- per-lane global addresses of the loads of one slab (k0 = 0) ----------------------
-    const CT *wptr[C::LW];
-    const CT *xptr[C::LX];
+    // ---- global addresses of the loads of one slab: uniform base + 32-bit per-lane offset ----
+    // (the host checks that the offsets fit)
+    const char *const wbase = (const char *)(w + ((size_t)(DD == 1 ? g : a_i * DD) * c) * b + m0);
+    const char *const xbase = BS_LAST ? (const char *)(x + ((size_t)a_i * c * d + d_i) * batch + n0)
+                                      : (const char *)(x + (size_t)n0 * in_size + (size_t)a_i * c * DD);
+    uint32_t wvoff[C::LW], xvoff[C::LX];
 #pragma unroll
     for (int i = 0; i < C::LW; ++i) {
         const int q = tid + i * C::THREADS;
         const int dd = q / (TK * C::W_CPR), r = q % (TK * C::W_CPR);
         const int row = r / C::W_CPR, pc = r % C::W_CPR;
-        const int col = (pc ^ swz_outer<CT>(row)) * C::EPC;
-        const int blk = DD == 1 ? g : a_i * DD + dd;
-        wptr[i] = w + ((size_t)blk * c + row) * b + m0 + col;
+        const int col = (pc ^ swz_outer<CT, C::W_CPR>(row)) * C::EPC;
+        wvoff[i] = (uint32_t)((((size_t)dd * c + row) * b + col) * C::ES);
     }
 #pragma unroll
     for (int i = 0; i < C::LX; ++i) {
         const int q = tid + i * C::THREADS;
         const int row = q / C::X_CPR, pc = q % C::X_CPR;
         if (BS_LAST) {
-            const int col = (pc ^ swz_outer<CT>(row)) * C::EPC;
-            xptr[i] = x + ((size_t)(a_i * c + row) * d + d_i) * batch + min(n0 + col, batch - C::EPC);
+            const int col = (pc ^ swz_outer<CT, C::X_CPR>(row)) * C::EPC;
+            xvoff[i] = (uint32_t)(((size_t)row * d * batch + min(col, batch - C::EPC - n0)) * C::ES);
         } else {
             const int col = (pc ^ swz_inner<C::X_CPR>(row)) * C::EPC;
-            xptr[i] = x + (size_t)min(n0 + row, batch - 1) * in_size + (size_t)a_i * c * DD + col;
+            xvoff[i] = (uint32_t)(((size_t)min(row, batch - 1 - n0) * in_size + col) * C::ES);
         }
     }
-    const size_t w_step = (size_t)TK * b;                                   // elements per slab
-    const size_t x_step = BS_LAST ? (size_t)TK * d * batch : (size_t)TK * DD;
+    const size_t w_step = (size_t)TK * b * C::ES;                                   // bytes per slab
+    const size_t x_step = (BS_LAST ? (size_t)TK * d * batch : (size_t)TK * DD) * C::ES;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     auto issue = [&](int step, int stg) {
         const uint32_t dst = lds_base + stg * C::STAGE_BYTES + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < C::LW; ++i) dma16(wptr[i] + step * w_step, dst + i * (C::THREADS * 16));
+        for (int i = 0; i < C::LW; ++i) dma16s(wbase + step * w_step, wvoff[i], dst + i * (C::THREADS * 16));
 #pragma unroll
         for (int i = 0; i < C::LX; ++i)
-            dma16(xptr[i] + step * x_step, dst + C::W_BYTES + i * (C::THREADS * 16));
+            dma16s(xbase + step * x_step, xvoff[i], dst + C::W_BYTES + i * (C::THREADS * 16));
     };
+
+    // ---- per-lane byte offsets of the MFMA operands inside a stage (sub-step 0) --------------
+    uint32_t woff[C::MT], xoff[C::NT];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i) woff[i] = outer_frag<CT, TM>::off((wm * C::MT + i) * 32, lane);
+#pragma unroll
+    for (int j = 0; j < C::NT; ++j) {
+        const int idx0 = (wn * C::NT + j) * 32;
+        if constexpr (BS_LAST) {
+            xoff[j] = C::W_BYTES + outer_frag<CT, TN>::off(idx0, lane);
+        } else {
+            // k-inner rows of TK*DD elements; chunk (k0/8 + lane/32) (x 2 for the d_i pairs),
+            // swizzled: the k0 part is XORed in when the operand is read
+            const int row = idx0 + (lane & 31), lq = lane >> 5;
+            xoff[j] = C::W_BYTES + row * (TK * DD * 2) + (((DD == 2 ? 2 * lq : lq) ^ swz_inner<C::X_CPR>(row)) << 4);
+        }
+    }
 
     float16_t acc[DD][C::MT][C::NT];
 #pragma unroll
@@ -183,28 +247,31 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     for (int p = 0; p < ST - 1; ++p) issue(min(p, steps - 1), p);
     KG_STAMP(1);
 
-    // MFMA operands of sub-step k0 of the current slab
+    // MFMA operands of sub-step k0 of the slab whose operand addresses are wa[] / xa[]
     typedef typename frag<CT>::type frag_t;
-    auto load_frags = [&](const CT *wb, const CT *xb, int k0, frag_t(&fw)[DD][C::MT], frag_t(&fx)[DD][C::NT]) {
+    auto load_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[DD][C::MT],
+                          frag_t(&fx)[DD][C::NT]) {
+#ifdef KSMM_GABL_NOFRAG
+        if (batch != -12345) return;
+#endif
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
             for (int i = 0; i < C::MT; ++i)
-                fw[dd][i] = outer_frag<CT, TM>::get(wb + dd * TK * TM, (wm * C::MT + i) * 32, k0, lane);
+                fw[dd][i] = outer_frag<CT, TM>::read(wa[i] + dd * (TK * TM * C::ES), k0);
 #pragma unroll
         for (int j = 0; j < C::NT; ++j) {
-            const int idx0 = (wn * C::NT + j) * 32;
             if constexpr (BS_LAST) {
-                fx[0][j] = outer_frag<CT, TN>::get(xb, idx0, k0, lane);
+                fx[0][j] = outer_frag<CT, TN>::read(xa[j], k0);
             } else if constexpr (DD == 1) {
-                const int row = idx0 + (lane & 31), chunk = (k0 >> 3) + (lane >> 5);
-                fx[0][j] = *(const half8_t *)(xb + row * (TK * DD) + ((chunk ^ swz_inner<C::X_CPR>(row)) << 3));
+                typedef __attribute__((address_space(3))) half8_t *lds_ptr;
+                fx[0][j] = *(lds_ptr)(lds_bytes_t)(uintptr_t)(xa[j] ^ ((k0 >> 3) << 4));
             } else {
                 // 16 consecutive halves = 8 (k, d_i) pairs -> one operand per d_i
-                const int row = idx0 + (lane & 31), chunk = 2 * ((k0 >> 3) + (lane >> 5));
-                const int sw = swz_inner<C::X_CPR>(row);
-                const uint4_t lo = *(const uint4_t *)(xb + row * (TK * DD) + ((chunk ^ sw) << 3));
-                const uint4_t hi = *(const uint4_t *)(xb + row * (TK * DD) + (((chunk + 1) ^ sw) << 3));
+                typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
+                const uint32_t pa = xa[j] ^ ((k0 >> 2) << 4);
+                const uint4_t lo = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa);
+                const uint4_t hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ 16);
                 uint4_t e, o;
                 e[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100u);
                 e[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x05040100u);
@@ -221,56 +288,87 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     };
     constexpr int K0 = TK / C::KSTEP;                  // MFMA sub-steps per slab
     constexpr int PER_K0 = DD * C::MT * C::NT;         // MFMAs per sub-step
-    constexpr int STRIDE = (K0 * PER_K0) / C::L > 0 ? (K0 * PER_K0) / C::L : 1;  // MFMAs per load issued
+    static_assert(K0 >= 2 && K0 % 2 == 0, "operand double buffer alternates inside a slab");
+    // The L loads of slab it+ST-1 are spread between the MFMAs of sub-steps 0..K0-2 of slab it
+    // (the path into LDS moves 64 bytes per clock and CU: issued in one burst it would stall the
+    // wave for about half a slab).  Before the MFMAs of the last sub-step every wave waits for
+    // its loads of slab it+1 ((ST-2)*L newer ones may stay in flight; near the end the ring
+    // holds repeats of the last slab, so the count stays constant), meets the others at a
+    // barrier and requests the first operands of slab it+1, which arrive while the last
+    // sub-step multiplies; operands of sub-step k0+1 are read while k0 multiplies.
+    constexpr int SLOTS = (K0 - 1) * PER_K0;
+    constexpr int STRIDE = SLOTS / C::L > 0 ? SLOTS / C::L : 1;  // MFMAs per load issued
+    frag_t fw[2][DD][C::MT], fx[2][DD][C::NT];
+    uint32_t wa[C::MT], xa[C::NT];
+    auto stage_addrs = [&](int stg) {
+        const uint32_t base = lds_base + stg * C::STAGE_BYTES;
+        // opaque to the compiler from here on, so that the k0 / d_i parts of an operand address
+        // stay in the offset field of the LDS instructions instead of being re-added per read
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i) {
+            wa[i] = woff[i] + base;
+            asm volatile("" : "+v"(wa[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            xa[j] = xoff[j] + base;
+            asm volatile("" : "+v"(xa[j]));
+        }
+    };
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
+    __syncthreads();  // slab 0 landed for every wave
+    stage_addrs(0);
+    load_frags(wa, xa, 0, fw[0], fx[0]);
 
     for (int it = 0; it < steps; ++it) {
-        // slab `it` was requested ST-1 iterations ago; (ST-2)*L newer loads may stay in flight.
-        // Near the end the ring holds repeats of the last slab, so the count stays constant.
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
-        KG_STAMP(4 + 4 * it);
-        __syncthreads();  // slab `it` landed for every wave, and everyone left slab it-1
-        KG_STAMP(5 + 4 * it);
-        const CT *wb = (const CT *)(smem + (it % ST) * C::STAGE_BYTES);
-        const CT *xb = (const CT *)(smem + (it % ST) * C::STAGE_BYTES + C::W_BYTES);
-        // The L loads of slab it+ST-1 are spread between the MFMAs of this slab (the path into
-        // LDS moves 64 bytes per clock and CU: issued in one burst it would stall the wave for
-        // about half a slab), and the operands of sub-step k0+1 are read while k0 multiplies.
         const int nstep = min(it + ST - 1, steps - 1);
-        const size_t w_off = (size_t)nstep * w_step, x_off = (size_t)nstep * x_step;
+        const char *const wsrc = wbase + (size_t)nstep * w_step;
+        const char *const xsrc = xbase + (size_t)nstep * x_step;
         const uint32_t dst = lds_base + ((it + ST - 1) % ST) * C::STAGE_BYTES + wave * 1024;
-        frag_t fw[2][DD][C::MT], fx[2][DD][C::NT];
-        load_frags(wb, xb, 0, fw[0], fx[0]);
-        KG_STAMP(6 + 4 * it);
+        auto issue_one = [&](int q) {
+            if (q < C::LW)
+                dma16s(wsrc, wvoff[q < C::LW ? q : 0], dst + q * (C::THREADS * 16));
+            else
+                dma16s(xsrc, xvoff[q >= C::LW ? q - C::LW : 0], dst + C::W_BYTES + (q - C::LW) * (C::THREADS * 16));
+        };
 #pragma unroll
         for (int kk = 0; kk < K0; ++kk) {
-            if (kk + 1 < K0) load_frags(wb, xb, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], fx[(kk + 1) & 1]);
+            if (kk + 1 < K0) {
+                load_frags(wa, xa, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], fx[(kk + 1) & 1]);
+            } else {
+                KG_STAMP(4 + 4 * it);
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
+                __syncthreads();  // slab it+1 landed for every wave, and everyone left slab it
+                KG_STAMP(5 + 4 * it);
+                if (it + 1 < steps) {
+                    stage_addrs((it + 1) % ST);
+                    load_frags(wa, xa, 0, fw[0], fx[0]);
+                }
+                KG_STAMP(6 + 4 * it);
+            }
 #pragma unroll
             for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
                 for (int i = 0; i < C::MT; ++i)
 #pragma unroll
                     for (int j = 0; j < C::NT; ++j) {
+#ifdef KSMM_GABL_NOMFMA
+                        acc[dd][i][j][0] += abl_first(fw[kk & 1][dd][i]) + abl_first(fx[kk & 1][dd][j]);
+#else
                         acc[dd][i][j] = BS_LAST ? frag<CT>::mfma(fx[kk & 1][dd][j], fw[kk & 1][dd][i], acc[dd][i][j])
                                                 : frag<CT>::mfma(fw[kk & 1][dd][i], fx[kk & 1][dd][j], acc[dd][i][j]);
+#endif
                         const int m = kk * PER_K0 + (dd * C::MT + i) * C::NT + j;  // MFMA index in the slab
-                        if ((m + 1) % STRIDE == 0 && m / STRIDE < C::L) {
-                            const int q = m / STRIDE;  // load index
-                            if (q < C::LW)
-                                dma16(wptr[q < C::LW ? q : 0] + w_off, dst + q * (C::THREADS * 16));
-                            else
-                                dma16(xptr[q >= C::LW ? q - C::LW : 0] + x_off,
-                                      dst + C::W_BYTES + (q - C::LW) * (C::THREADS * 16));
+                        if (kk + 1 < K0 && (m + 1) % STRIDE == 0 && m / STRIDE < C::L) {
+                            issue_one(m / STRIDE);
                             __builtin_amdgcn_sched_barrier(0);
                         }
                     }
-        }
-        // loads that did not get a slot above (fewer MFMAs than loads)
+            if (kk == K0 - 2) {
+                // loads that did not get a slot above (fewer MFMAs than loads)
 #pragma unroll
-        for (int q = (K0 * PER_K0) / STRIDE; q < C::L; ++q) {
-            if (q < C::LW)
-                dma16(wptr[q < C::LW ? q : 0] + w_off, dst + q * (C::THREADS * 16));
-            else
-                dma16(xptr[q >= C::LW ? q - C::LW : 0] + x_off, dst + C::W_BYTES + (q - C::LW) * (C::THREADS * 16));
+                for (int q = SLOTS / STRIDE; q < C::L; ++q) issue_one(q);
+            }
         }
     }
     KG_STAMP(2);
@@ -380,10 +478,14 @@ const GemmInst gemm_insts[] = {
     GEMM_INST(1, half_t, false, 1, 256, 256, 32, 2, 2, 4),
     GEMM_INST(1, half_t, false, 1, 128, 128, 32, 2, 2, 4),
     // fp32, bs_last
-    GEMM_INST_O(0, float, true, 1, 128, 256, 16, 2, 2, 3, 2),
     GEMM_INST(0, float, true, 1, 128, 128, 16, 2, 2, 4),
+    GEMM_INST_O(0, float, true, 1, 128, 256, 16, 2, 2, 3, 2),
     GEMM_INST(0, float, true, 1, 256, 256, 16, 2, 2, 4),
     GEMM_INST(0, float, true, 1, 64, 256, 16, 1, 4, 4),
+    // fp16, bs_first, d == 2: 4 waves with 128 x 64 (x 2 d_i) wave tiles: half the LDS operand
+    // traffic per MFMA of the 8-wave tiles above
+    GEMM_INST(1, half_t, false, 2, 256, 128, 32, 2, 2, 3),
+    GEMM_INST(1, half_t, false, 2, 128, 256, 32, 1, 4, 3),
 };
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 
@@ -399,6 +501,12 @@ bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
         if (((int64_t)p.a * p.c * p.d) % t.epc || ((int64_t)p.c * p.d) % t.epc) return false;
         if (t.dd == 2 && (((int64_t)p.a * p.b * p.d) % 2)) return false;
     }
+    // per-lane byte offsets of the direct-to-LDS loads are 32-bit
+    const int64_t es = 16 / t.epc, lim = 0xffffffffLL;
+    if ((int64_t)t.dd * p.c * p.b * es >= lim) return false;
+    if (p.bs_last ? ((int64_t)t.tk * p.d * p.batch + p.batch) * es >= lim
+                  : ((int64_t)t.tn * p.a * p.c * p.d + (int64_t)p.c * p.d) * es >= lim)
+        return false;
     return true;
 }
 
