@@ -102,13 +102,14 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
 // LDS has 64 banks of 4 bytes: a ds_read_b64 is served 32 lanes per clock and a ds_read_b128
 // 16 lanes per clock, conflict-free when those lanes cover 256 bytes of distinct banks.
 //  k-outer fp16 rows (CPR chunks of 16 bytes): the 32 lanes of a transpose load read 4 rows x
-//  64 bytes -> XOR the 64-byte group index with row & 3 (32-byte groups when a row has only 8).
+//  64 bytes -> XOR the 64-byte group index with row & 3 (rows of 128 bytes alternate bank
+//  halves already: row / 2 & 1).
 //  k-outer fp32: 2 rows x 128 bytes per ds_read_b32 wave -> XOR the 128-byte half with row & 1.
 //  k-inner rows: 16 lanes read one chunk of 16 consecutive rows -> XOR the chunk so that the
 //  rows sharing a 256-byte bank line differ (rows of 64, 128, >= 256 bytes).
 template <typename CT, int CPR> __device__ __forceinline__ int swz_outer(int row)
 {
-    return sizeof(CT) == 2 ? (CPR >= 16 ? 4 : 2) * (row & 3) : 8 * (row & 1);
+    return sizeof(CT) == 2 ? (CPR >= 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1)) : 8 * (row & 1);
 }
 template <int CPR> __device__ __forceinline__ int swz_inner(int row)
 {

@@ -88,17 +88,23 @@ struct StreamCfg {
     static constexpr int N_FULL = (ST - 1) * (L + S);       // steady state
     static_assert(BB % (32 * WM) == 0 && TN % (32 * WN) == 0 && CC % KSTEP == 0, "wave tiling");
     static_assert(X_CHUNKS % THREADS == 0 && O_CHUNKS % THREADS == 0, "every wave issues L loads and S stores");
-    static_assert(X_CPR % (ES == 2 ? 8 : (BS_LAST ? 16 : 8)) == 0, "swizzle group");
+    static_assert(X_CPR % (ES == 2 ? 8 : 16) == 0, "swizzle group");
     static_assert(N_FULL <= 63, "vmcnt range");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
     static_assert(BB % W_EPV == 0, "weight vectors");
 };
 
-// swizzle of the 16-byte chunk index inside a row of the input stage
-template <typename CT, bool BS_LAST> __device__ __forceinline__ int swz(int row)
+// Swizzle of the 16-byte chunk index inside a row (CPR chunks) of the input stage.  LDS has 64
+// banks of 4 bytes; a ds_read_b64 is served 32 lanes per clock, a ds_read_b128 16 lanes:
+//  k-outer fp16: the 32 lanes of a transpose load read 4 rows x 64 bytes -> the 64-byte group
+//  index is XORed with row & 3 (rows of 128 bytes alternate bank halves already: row / 2 & 1);
+//  k-outer fp32: a ds_read_b32 wave reads 2 rows x 128 bytes -> XOR the 128-byte half;
+//  k-inner: 16 lanes read one chunk of 16 consecutive rows -> rows of 128 or 384 bytes
+//  alternate bank halves, the chunk is XORed with row / 2; rows of 256 bytes with row & 15.
+template <typename CT, bool BS_LAST, int CPR> __device__ __forceinline__ int swz(int row)
 {
-    if (BS_LAST) return sizeof(CT) == 2 ? 2 * (row & 3) : 8 * (row & 1);
-    return row & 7;
+    if (BS_LAST) return sizeof(CT) == 2 ? (CPR >= 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1)) : 8 * (row & 1);
+    return CPR % 16 == 0 ? (row & 15) : ((row >> 1) & 7);
 }
 
 // MFMA operand of the input from a swizzled stage
@@ -109,7 +115,7 @@ template <int X_COLS> struct xfrag<half_t, true, X_COLS> {  // k-outer, transpos
         const int kq = lane >> 5, i16 = lane & 15, hs = (lane >> 4) & 1;
         const int row = k0 + 8 * kq + (i16 >> 2);  // + 4 for the second load: same row & 3
         const int chunk = (idx0 >> 3) + 2 * hs + ((i16 & 3) >> 1);
-        const int off = ((chunk ^ (2 * ((i16 >> 2) & 3))) << 3) + 4 * (i16 & 1);
+        const int off = ((chunk ^ swz<half_t, true, X_COLS / 8>(row)) << 3) + 4 * (i16 & 1);
         typedef short4_t __attribute__((address_space(3))) * lds_ptr;
         const half_t *p = s + row * X_COLS + off;
         short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
@@ -124,7 +130,7 @@ template <int X_COLS> struct xfrag<half_t, false, X_COLS> {  // k-inner, 16-byte
     {
         const int row = idx0 + (lane & 31);
         const int chunk = (k0 >> 3) + (lane >> 5);
-        return *(const half8_t *)(s + row * X_COLS + ((chunk ^ (row & 7)) << 3));
+        return *(const half8_t *)(s + row * X_COLS + ((chunk ^ swz<half_t, false, X_COLS / 8>(row)) << 3));
     }
 };
 template <int X_COLS> struct xfrag<float, true, X_COLS> {  // k-outer, 4-byte loads
@@ -170,7 +176,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
     for (int i = 0; i < C::L; ++i) {
         const int q = tid + i * C::THREADS;
         const int row = q / C::X_CPR, pc = q % C::X_CPR;
-        const int col = (pc ^ swz<CT, BS_LAST>(row)) * C::EPC;  // logical column of this chunk
+        const int col = (pc ^ swz<CT, BS_LAST, C::X_CPR>(row)) * C::EPC;  // logical column of this chunk
         if (BS_LAST) {
             goff[i] = (size_t)row * x_kstride;
             gcol[i] = col;
