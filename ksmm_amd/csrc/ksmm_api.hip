@@ -42,11 +42,13 @@ int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *ti
     case KSMM_ALGO_WAVE: return wave_run(p, variant, launch, tile);
     case KSMM_ALGO_TILE: return tile_run(p, variant, launch, tile);
     case KSMM_ALGO_AUTO: {
-        // Table order from sweeps at batch 25088: 16-bit mid-sized blocks (64x64 .. 192x192) go to
-        // the stream kernels of the tile family, smaller blocks and fp32 to the wave family, the
-        // rest to the k-loop tiles; shapes none of them takes run on the generic kernel.
+        // Table order from sweeps at batch 25088: batch-size-first 16-bit mid-sized blocks
+        // (64x64 .. 192x192) go to the stream kernels of the tile family; batch-size-last blocks
+        // the wave family has an instance for (up to 96x96), and fp32, go to the wave family,
+        // larger 16-bit blocks to the stream kernels again (inside the tile family), the rest to
+        // the GEMM and k-loop tiles; shapes none of them takes run on the generic kernel.
         int rc = KSMM_ERR_BAD_ALGO;
-        if (p.x_dtype == KSMM_F16) rc = stream_run(p, -1, launch, tile);
+        if (p.x_dtype == KSMM_F16 && !p.bs_last) rc = stream_run(p, -1, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
         rc = wave_run(p, -1, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;

@@ -1,7 +1,7 @@
 // "Row" kernel: batch-size-first layout, d > 1, small b x c blocks, fp32.
 //
 // In this layout a batch row holds, for one a_i, the c*d inputs of all d blocks interleaved
-// (d_i fastest).  A workgroup owns one a_i and a range of batch rows; it has one wavefront per
+// (d_i fastest).  A workgroup owns one a_i and every wgs-th tile of batch rows; it has one wavefront per
 // d_i, and each wavefront keeps the b x c weight block of its d_i in registers as MFMA
 // operands (v_mfma_f32_16x16x4_f32, fp32 accumulation).  Whole row segments (c*d contiguous
 // floats) are copied to LDS with 16-byte loads, every wave picks the inputs of its own d_i
@@ -9,14 +9,16 @@
 // the b*d outputs of each row are written back as one contiguous run.  HBM sees only full,
 // coalesced rows; the stride-d gather the layout forces happens in LDS.
 //
-// Input tiles are double-buffered in LDS across batch tiles (the loads of tile t+1 are in
-// flight while tile t is multiplied and stored).
+// The loads of the next two tiles are in flight (in registers) while a tile is multiplied and
+// stored; tiles are dealt round-robin to the workgroups of an a_i, so that at any time they
+// work on one compact window of memory.
 //
 // Reference counterpart: kernel_bs_first_float
 // (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-286), whose strided scalar
 // gathers from global memory (:156-161) make this the slowest layout of the reference
 // (0.86 ms for (1,48,48,16) in kernel_bs_first_float.best:9).
 #include "ksmm_common.h"
+#include <type_traits>
 
 namespace ksmm {
 
@@ -47,8 +49,7 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
     float *const os = xs + 2 * TN * C::LDX;         // [TN][LDO]
     const int a_i = blockIdx.x / wgs_per_a;
     const int s = blockIdx.x - a_i * wgs_per_a;
-    const int per = (n_tiles + wgs_per_a - 1) / wgs_per_a;
-    const int t_begin = s * per, t_end = min(n_tiles, t_begin + per);
+    const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
     const int dd = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's d_i
@@ -66,35 +67,34 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
 
     const float *xg = x + (size_t)a_i * C::XROW;
     float *yg = y + (size_t)a_i * C::OROW;
-    float4_t xreg[C::X_PER_T];
-    auto gload = [&](int t) {
+    float4_t xreg[2][C::X_PER_T];
+    auto gload = [&](int t, auto P) {
 #pragma unroll
         for (int i = 0; i < C::X_PER_T; ++i) {
             const int v = tid + i * C::THREADS;
             if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
                 const int nn = v / (C::XROW / 4), e0 = (v % (C::XROW / 4)) * 4;
                 const int row = min(t * TN + nn, batch - 1);
-                xreg[i] = *(const float4_t *)(xg + (size_t)row * in_size + e0);
+                xreg[decltype(P)::value][i] = *(const float4_t *)(xg + (size_t)row * in_size + e0);
             }
         }
     };
-    auto lstore = [&](int buf) {
+    auto lstore = [&](int buf, auto P) {
 #pragma unroll
         for (int i = 0; i < C::X_PER_T; ++i) {
             const int v = tid + i * C::THREADS;
             if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
                 const int nn = v / (C::XROW / 4), e0 = (v % (C::XROW / 4)) * 4;
-                *(float4_t *)(xs + (buf * TN + nn) * C::LDX + e0) = xreg[i];
+                *(float4_t *)(xs + (buf * TN + nn) * C::LDX + e0) = xreg[decltype(P)::value][i];
             }
         }
     };
-
-    gload(t_begin);
-    lstore(0);
-    __syncthreads();
-    for (int t = t_begin; t < t_end; ++t) {
-        const int buf = (t - t_begin) & 1;
-        if (t + 1 < t_end) gload(t + 1);
+    // one tile: its inputs are in LDS buffer `buf`; register set P is refilled with the tile
+    // after the next one at the start, and set 1-P (the next tile) goes to the other LDS buffer
+    // at the end
+    auto do_tile = [&](int t, int buf, auto P) {
+        typedef std::integral_constant<int, 1 - decltype(P)::value> Q;
+        if (t + 2 * t_step < t_end) gload(t + 2 * t_step, P);
         const float *xb = xs + buf * TN * C::LDX;
         float4_t acc[C::MT][C::NT];
 #pragma unroll
@@ -138,8 +138,17 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
                 }
             }
         }
-        if (t + 1 < t_end) lstore(buf ^ 1);
+        if (t + t_step < t_end) lstore(buf ^ 1, Q{});
         __syncthreads();
+    };
+
+    gload(t_begin, std::integral_constant<int, 0>{});
+    if (t_begin + t_step < t_end) gload(t_begin + t_step, std::integral_constant<int, 1>{});
+    lstore(0, std::integral_constant<int, 0>{});
+    __syncthreads();
+    for (int t = t_begin; t < t_end; t += 2 * t_step) {
+        do_tile(t, 0, std::integral_constant<int, 0>{});
+        if (t + t_step < t_end) do_tile(t + t_step, 1, std::integral_constant<int, 1>{});
     }
 }
 

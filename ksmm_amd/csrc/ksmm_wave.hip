@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
                                                      const float *__restrict__ w,
                                                      float *__restrict__ y, int batch, int a, int b,
                                                      int c, int d, float scale, int n_slabs,
-                                                     int iters)
+                                                     int iters, int rr)
 {
     constexpr int VEC = 4, TN = 16 * VEC;
     const int lane = threadIdx.x & 63;
@@ -156,8 +156,11 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
     const uint32_t x_lane = (uint32_t)(q * row_stride) * 4u;      // + column offset
     const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 4u;  // + column offset
-    const int n_first = slab * iters * TN;                        // uniform
-    const int n_end = min(n_first + iters * TN, batch);           // uniform
+    // tiles of one wave: consecutive (rr == 0) or every n_slabs-th (rr == 1: the waves of a
+    // block then work on neighbouring tiles at any one time)
+    const int stride = rr ? n_slabs * TN : TN;                    // uniform
+    const int n_first = rr ? slab * TN : slab * iters * TN;       // uniform
+    const int n_end = rr ? batch : min(n_first + iters * TN, batch);
     const int last_vec = batch - VEC;
     if (n_first >= n_end) return;
 
@@ -178,12 +181,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     __builtin_amdgcn_s_waitcnt(0);
     KW_STAMP(3);
     int kw_slot = 4;
-    const int n_last = n_first + ((n_end - n_first - 1) / TN) * TN;  // first column of the last tile
+    const int n_last = n_first + ((n_end - n_first - 1) / stride) * stride;  // first column of the last tile
     // FULL tiles store without a predicate, which keeps the loop body free of branches; a
     // ragged last tile (batch not a multiple of the tile) runs once more with the predicate.
     auto do_tile = [&](int n0, auto full) {
         // the tile after the last one is the last one again (a cache hit that is not used)
-        const uint32_t next_off = x_lane + col_off(min(n0 + TN, n_last));
+        const uint32_t next_off = x_lane + col_off(min(n0 + stride, n_last));
         float4_t acc[MT][VEC];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -228,7 +231,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
 #endif
     };
     int n0 = n_first;
-    for (; n0 + TN <= n_end; n0 += TN) do_tile(n0, std::true_type{});
+    for (; n0 + TN <= n_end; n0 += stride) do_tile(n0, std::true_type{});
     if (n0 < n_end) do_tile(n0, std::false_type{});
     KW_STAMP(1);
 }
@@ -241,7 +244,7 @@ template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC, bo
 __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ x,
                                                    const TW *__restrict__ w,
                                                    half_t *__restrict__ y, int batch, int a, int b,
-                                                   int c, int d, float scale, int n_slabs, int iters)
+                                                   int c, int d, float scale, int n_slabs, int iters, int rr)
 {
     constexpr int TN = 16 * VEC, KSTEP = 4 * KL;
     typedef typename hvec<KL>::type frag_t;
@@ -271,8 +274,9 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
     char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
     const uint32_t x_lane = (uint32_t)(KL * q * row_stride) * (uint32_t)sizeof(TX);
     const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 2u;
-    const int n_first = slab * iters * TN;
-    const int n_end = min(n_first + iters * TN, batch);
+    const int stride = rr ? n_slabs * TN : TN;
+    const int n_first = rr ? slab * TN : slab * iters * TN;
+    const int n_end = rr ? batch : min(n_first + iters * TN, batch);
     const int last_vec = batch - VEC;
     if (n_first >= n_end) return;
 
@@ -290,9 +294,9 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
                          raw[ks][jj]);
     }
     __builtin_amdgcn_s_waitcnt(0);
-    const int n_last = n_first + ((n_end - n_first - 1) / TN) * TN;
+    const int n_last = n_first + ((n_end - n_first - 1) / stride) * stride;
     auto do_tile = [&](int n0, auto full) {
-        const uint32_t next_off = x_lane + col_off(min(n0 + TN, n_last));
+        const uint32_t next_off = x_lane + col_off(min(n0 + stride, n_last));
         float4_t acc[MT][VEC];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -347,7 +351,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
         }
     };
     int n0 = n_first;
-    for (; n0 + TN <= n_end; n0 += TN) do_tile(n0, std::true_type{});
+    for (; n0 + TN <= n_end; n0 += stride) do_tile(n0, std::true_type{});
     if (n0 < n_end) do_tile(n0, std::false_type{});
 }
 
@@ -358,9 +362,9 @@ struct WaveInst {
     const void *fn_once;  // one tile per wave: nothing is reloaded
 };
 
-typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, float, int, int);
+typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, float, int, int, int);
 template <typename TX, typename TW>
-using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int, float, int, int);
+using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int, float, int, int, int);
 
 // OCC_ = minimum waves per SIMD the register allocation must allow
 #define F32_INST(B_, C_, OCC_) \
@@ -411,6 +415,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     // (0: heuristic); -1: everything automatic
     const int want = variant < 0 ? 0xff : (variant & 0xff);
     int iters = variant < 0 ? 0 : ((variant >> 8) & 0xff);
+    int rr = variant < 0 ? 0 : ((variant >> 16) & 1);  // tiles of a wave: 0 consecutive, 1 every n_slabs-th
     int pick = -1;
     for (int i = 0; i < n_insts; ++i) {
         if (insts[i].b != p.b || insts[i].c != p.c) continue;
@@ -455,7 +460,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     }
     if (!launch) return KSMM_OK;
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, nullptr, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, nullptr, nullptr};
+                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, nullptr, nullptr, &rr};
     int batch_i = (int)p.batch, n_slabs_i = (int)n_slabs;
     args[3] = &batch_i;
     args[9] = &n_slabs_i;
