@@ -113,10 +113,31 @@ int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batc
                              int b, int c, int d, int x_dtype, int w_dtype, int y_dtype,
                              int bs_last, float scale, int algo, int variant, void *stream);
 
-/* Bytes of device workspace ksmm_chain_forward needs for these factors (two ping-pong
- * intermediates; 0 for a single factor).  Intermediates have type y_dtype. */
+/* Batch-size-first factors with d > 1 whose shape has no kernel of its own in that layout run
+ * in batch-size-last layout between two transposes when the caller lends a workspace.
+ * ksmm_factor_workspace returns the bytes ksmm_factor_forward_ws can use for a problem (0: a
+ * direct kernel exists, the workspace is ignored).  With a smaller workspace (or NULL) it
+ * returns KSMM_ERR_WORKSPACE; ksmm_factor_forward (no workspace) falls back to the generic
+ * kernel for such shapes.  The reference has no counterpart: its batch-size-first kernels
+ * gather with strided scalar loads (template_kernels_float.cuh:156-161). */
+int64_t ksmm_factor_workspace(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                              int y_dtype, int bs_last);
+int ksmm_factor_forward_ws(const void *x, const void *w, void *y, int64_t batch, int a, int b,
+                           int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                           float scale, void *workspace, int64_t workspace_bytes, void *stream);
+
+/* Bytes of device workspace ksmm_chain_forward needs for these factors in batch-size-last
+ * layout (two ping-pong intermediates; 0 for a single factor).  Intermediates have type
+ * y_dtype. */
 int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
                              int y_dtype);
+
+/* The same for a given layout and input type: a batch-size-first chain with a factor that
+ * needs the transposed route asks for room for the transposed input and for ping-pong buffers
+ * that also hold the (transposed) final output.  ksmm_chain_forward takes that route when the
+ * workspace it is given is at least this large, and the factor-by-factor route otherwise. */
+int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
+                                    int x_dtype, int y_dtype, int bs_last);
 
 /* A chain K_n ... K_1 x: factors[0] acts first.  Replaces the Python loop of
  * KSLinear.forward_bs_first / forward_bs_last

@@ -43,7 +43,12 @@ SIGNATURES = {
                                     c_int, c_int, ctypes.c_float, c_vp]),
     "ksmm_factor_forward_algo": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int,
                                          c_int, c_int, c_int, ctypes.c_float, c_int, c_int, c_vp]),
+    "ksmm_factor_workspace": (c_i64, [c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "ksmm_factor_forward_ws": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_int, c_int, ctypes.c_float, c_vp, c_i64, c_vp]),
     "ksmm_chain_workspace": (c_i64, [ctypes.POINTER(KsmmFactorDesc), c_int, c_i64, c_int]),
+    "ksmm_chain_workspace_layout": (c_i64, [ctypes.POINTER(KsmmFactorDesc), c_int, c_i64, c_int, c_int,
+                                            c_int]),
     "ksmm_chain_forward": (c_int, [ctypes.POINTER(KsmmFactorDesc), c_int, c_vp, c_vp, c_vp, c_i64,
                                    c_i64, c_int, c_int, c_int, c_int, c_vp]),
 }

@@ -60,6 +60,22 @@ int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *ti
     }
 }
 
+// A batch-size-first problem that only the generic kernel takes, while its batch-size-last
+// twin has a real kernel: worth two transposes.
+bool wants_transposed(const Problem &p)
+{
+    if (p.bs_last) return false;
+    ksmm_tile t;
+    memset(&t, 0, sizeof(t));
+    if (dispatch(p, KSMM_ALGO_AUTO, -1, false, &t) != KSMM_OK || t.algo != KSMM_ALGO_GENERIC) return false;
+    Problem q = p;
+    q.bs_last = 1;
+    memset(&t, 0, sizeof(t));
+    return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && t.algo != KSMM_ALGO_GENERIC;
+}
+
+int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
 }  // namespace
 
 extern "C" {
@@ -128,6 +144,38 @@ int ksmm_factor_forward(const void *x, const void *w, void *y, int64_t batch, in
                                     scale, KSMM_ALGO_AUTO, -1, stream);
 }
 
+int64_t ksmm_factor_workspace(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                              int y_dtype, int bs_last)
+{
+    int rc = check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    Problem p{nullptr, nullptr, nullptr, batch, a, b, c, d, x_dtype, w_dtype, y_dtype,
+              bs_last ? 1 : 0, 1.f, nullptr};
+    if (!wants_transposed(p)) return 0;
+    return align256((int64_t)a * c * d * batch * (int64_t)dtype_size(x_dtype)) +
+           align256((int64_t)a * b * d * batch * (int64_t)dtype_size(y_dtype));
+}
+
+int ksmm_factor_forward_ws(const void *x, const void *w, void *y, int64_t batch, int a, int b,
+                           int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                           float scale, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    const int64_t need = ksmm_factor_workspace(batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last);
+    if (need < 0) return (int)need;
+    if (need == 0)
+        return ksmm_factor_forward(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale, stream);
+    if (!x || !w || !y) return KSMM_ERR_NULL_POINTER;
+    if (!workspace || workspace_bytes < need) return KSMM_ERR_WORKSPACE;
+    const int64_t in_size = (int64_t)a * c * d, out_size = (int64_t)a * b * d;
+    char *xt = (char *)workspace;
+    char *yt = xt + align256(in_size * batch * (int64_t)dtype_size(x_dtype));
+    int rc = transpose_run(x, xt, batch, in_size, (int)dtype_size(x_dtype), (hipStream_t)stream);
+    if (rc != KSMM_OK) return rc;
+    rc = ksmm_factor_forward(xt, w, yt, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, 1, scale, stream);
+    if (rc != KSMM_OK) return rc;
+    return transpose_run(yt, y, out_size, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+}
+
 static int check_chain(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype)
 {
     if (!f) return KSMM_ERR_NULL_POINTER;
@@ -161,6 +209,36 @@ int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int
     return n_factors > 1 ? 2 * one : 0;
 }
 
+// batch-size-first chain with at least one factor that needs the transposed route
+static bool chain_wants_transposed(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype,
+                                   int bs_last)
+{
+    if (bs_last) return false;
+    for (int i = 0; i < n; ++i) {
+        Problem p{nullptr, nullptr, nullptr, batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
+                  f[i].w_dtype, y_dtype, 0, 1.f, nullptr};
+        if (wants_transposed(p)) return true;
+    }
+    return false;
+}
+
+int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
+                                    int x_dtype, int y_dtype, int bs_last)
+{
+    int rc = check_chain(factors, n_factors, batch, x_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    if (!chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last))
+        return ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
+    int64_t widest = 0;
+    for (int i = 0; i < n_factors; ++i) {
+        int64_t o = (int64_t)factors[i].a * factors[i].b * factors[i].d;
+        if (o > widest) widest = o;
+    }
+    const int64_t in0 = (int64_t)factors[0].a * factors[0].c * factors[0].d;
+    return align256(in0 * batch * (int64_t)dtype_size(x_dtype)) +
+           2 * align256(widest * batch * (int64_t)dtype_size(y_dtype));
+}
+
 int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
                        void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
                        int y_dtype, int bs_last, int fuse, void *stream)
@@ -170,6 +248,41 @@ int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const voi
     if (!x || !y) return KSMM_ERR_NULL_POINTER;
     for (int i = 0; i < n_factors; ++i)
         if (!factors[i].w) return KSMM_ERR_NULL_POINTER;
+    if (chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
+        // transpose once, run the whole chain in batch-size-last layout, transpose back
+        const int64_t need_t = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 0);
+        if (workspace && workspace_bytes >= need_t) {
+            const int64_t in0 = (int64_t)factors[0].a * factors[0].c * factors[0].d;
+            const int64_t out_n = (int64_t)factors[n_factors - 1].a * factors[n_factors - 1].b * factors[n_factors - 1].d;
+            const int64_t xt_bytes = align256(in0 * batch * (int64_t)dtype_size(x_dtype));
+            char *xt = (char *)workspace;
+            char *pp = xt + xt_bytes;
+            const int64_t one = (need_t - xt_bytes) / 2;
+            rc = transpose_run(x, xt, batch, in0, (int)dtype_size(x_dtype), (hipStream_t)stream);
+            if (rc != KSMM_OK) return rc;
+            const void *cur = xt;
+            int cur_dtype = x_dtype;
+            rc = KSMM_ERR_BAD_ALGO;
+            if (fuse)
+                rc = chain16_run(factors, n_factors, xt, pp, batch, x_dtype, y_dtype, 1, true, (hipStream_t)stream);
+            if (rc == KSMM_OK) {
+                cur = pp;
+            } else if (rc != KSMM_ERR_BAD_ALGO) {
+                return rc;
+            } else {
+                for (int i = 0; i < n_factors; ++i) {
+                    void *dst = pp + (i & 1) * one;
+                    rc = ksmm_factor_forward_algo(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b,
+                                                  factors[i].c, factors[i].d, cur_dtype, factors[i].w_dtype,
+                                                  y_dtype, 1, factors[i].scale, KSMM_ALGO_AUTO, -1, stream);
+                    if (rc != KSMM_OK) return rc;
+                    cur = dst;
+                    cur_dtype = y_dtype;
+                }
+            }
+            return transpose_run(cur, y, out_n, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+        }
+    }
     if (fuse) {
         // chains whose intermediates fit LDS run as one kernel (no workspace traffic)
         rc = chain16_run(factors, n_factors, x, y, batch, x_dtype, y_dtype, bs_last ? 1 : 0, true,

@@ -97,6 +97,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // p
 int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 
 // Fused radix-16 chain (intermediates in LDS); KSMM_ERR_BAD_ALGO when the chain does not qualify.
+int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream);
 int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_t batch, int x_dtype,
                 int y_dtype, int bs_last, bool launch, hipStream_t stream);
 

@@ -487,6 +487,9 @@ const GemmInst gemm_insts[] = {
     // traffic per MFMA of the 8-wave tiles above
     GEMM_INST(1, half_t, false, 2, 256, 128, 32, 2, 2, 3),
     GEMM_INST(1, half_t, false, 2, 128, 256, 32, 1, 4, 3),
+    // fp16, b a multiple of 64 only
+    GEMM_INST(1, half_t, true, 1, 64, 256, 32, 1, 4, 3),
+    GEMM_INST(1, half_t, false, 1, 64, 256, 32, 1, 4, 3),
 };
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 
@@ -513,7 +516,8 @@ bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
 
 }  // namespace
 
-// variant: index into the instance table (-1: first that fits with enough workgroups)
+// variant: index into the instance table; -1: first that fits with enough workgroups to fill
+// the chip; -2: first that fits
 int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
@@ -522,7 +526,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         if (variant >= 0 && variant != i) continue;
         const GemmInst &t = gemm_insts[i];
         if (!gemm_fits(t, p, combo)) continue;
-        if (variant < 0) {
+        if (variant == -1) {
             // the big tiles only pay when they still fill the chip
             const int64_t groups = t.dd == 1 ? (int64_t)p.a * p.d : p.a;
             const int64_t wgs = groups * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);

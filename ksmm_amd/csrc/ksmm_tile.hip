@@ -555,7 +555,8 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             }
         }
     }
-    if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    // nothing else takes it: a GEMM tile that does not fill the chip still beats the generic kernel
+    if (pick < 0) return variant == -1 ? gemm_run(p, -2, launch, tile) : KSMM_ERR_BAD_ALGO;
     const TileInst &t = tile_insts[pick];
     const int m_tiles = p.b / t.tm;
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;

@@ -1,0 +1,128 @@
+// Layout change between batch-size-first (batch, features) and batch-size-last (features,
+// batch): a plain 2-D transpose of 1-, 2- or 4-byte elements through a 64 x 64 LDS tile.
+//
+// It serves the batch-size-first factors with d > 1 that have no kernel of their own: in that
+// layout the inputs of one block are d elements apart, which the MFMA operand loads cannot
+// gather; the factor (or the whole chain) is run in batch-size-last layout between two
+// transposes instead, on a workspace the caller provides.
+//
+// Global memory is read and written with 16-byte vectors (128-byte runs per row of a tile) when
+// the sizes and addresses allow it, element by element otherwise.  The tile is kept in LDS with
+// an odd stride in 4-byte words, so that the column reads of the store phase spread over the
+// 64 banks.
+//
+// Reference counterpart: none as a kernel (the reference's batch-size-first kernels gather with
+// strided scalar loads, template_kernels_float.cuh:156-161); KSLinear permutes activations with
+// torch in its 'bmm' path (interface.py:213-267).
+#include "ksmm_common.h"
+
+namespace ksmm {
+
+namespace {
+
+constexpr int TT = 64;  // tile edge, elements
+
+template <int ES> struct elem_of;
+template <> struct elem_of<1> { typedef uint8_t type; };
+template <> struct elem_of<2> { typedef uint16_t type; };
+template <> struct elem_of<4> { typedef uint32_t type; };
+
+// in: rows x cols, row-major; out: cols x rows.  VIN / VOUT: 16-byte vectors on that side.
+template <int ES, bool VIN, bool VOUT>
+__global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restrict__ in_, void *__restrict__ out_,
+                                                          int rows, int cols, int tiles_c)
+{
+    typedef typename elem_of<ES>::type T;
+    constexpr int V = 16 / ES;             // elements per vector
+    constexpr int LD = TT + 4 / ES;        // row stride in elements: an odd number of 4-byte words
+    __shared__ __attribute__((aligned(16))) T tile[TT * LD + 8];
+    const T *in = (const T *)in_;
+    T *out = (T *)out_;
+    const int tr = blockIdx.x / tiles_c, tc = blockIdx.x - tr * tiles_c;
+    const int r0 = tr * TT, c0 = tc * TT;
+    const int tid = threadIdx.x;
+
+    // ---- load: tile[r][c] = in[r0 + r][c0 + c] ----
+    if (VIN) {
+        constexpr int VPR = TT / V;  // vectors per tile row
+#pragma unroll
+        for (int i = 0; i < TT * VPR / 256; ++i) {
+            const int q = tid + i * 256, r = q / VPR, cv = (q % VPR) * V;
+            if (r0 + r < rows && c0 + cv < cols) {  // cols % V == 0: whole vectors
+                const uint4_t v = *(const uint4_t *)(in + (size_t)(r0 + r) * cols + c0 + cv);
+                // 4-byte LDS writes (the odd stride leaves rows only 4-byte aligned)
+                uint32_t *dst = (uint32_t *)(tile + r * LD + cv);
+                dst[0] = v[0];
+                dst[1] = v[1];
+                dst[2] = v[2];
+                dst[3] = v[3];
+            }
+        }
+    } else {
+        for (int q = tid; q < TT * TT; q += 256) {
+            const int r = q / TT, c = q % TT;
+            if (r0 + r < rows && c0 + c < cols) tile[r * LD + c] = in[(size_t)(r0 + r) * cols + c0 + c];
+        }
+    }
+    __syncthreads();
+    // ---- store: out[c0 + c][r0 + r] = tile[r][c] ----
+    if (VOUT) {
+        constexpr int VPR = TT / V;
+#pragma unroll
+        for (int i = 0; i < TT * VPR / 256; ++i) {
+            const int q = tid + i * 256, c = q / VPR, rv = (q % VPR) * V;
+            if (c0 + c < cols && r0 + rv < rows) {  // rows % V == 0
+                T e[V];
+#pragma unroll
+                for (int j = 0; j < V; ++j) e[j] = tile[(rv + j) * LD + c];
+                uint4_t v;
+                if constexpr (ES == 4) {
+                    v = uint4_t{e[0], e[1], e[2], e[3]};
+                } else if constexpr (ES == 2) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        v[j] = (uint32_t)e[4 * j] | ((uint32_t)e[4 * j + 1] << 8) | ((uint32_t)e[4 * j + 2] << 16) |
+                               ((uint32_t)e[4 * j + 3] << 24);
+                }
+                *(uint4_t *)(out + (size_t)(c0 + c) * rows + r0 + rv) = v;
+            }
+        }
+    } else {
+        for (int q = tid; q < TT * TT; q += 256) {
+            const int c = q / TT, r = q % TT;
+            if (r0 + r < rows && c0 + c < cols) out[(size_t)(c0 + c) * rows + r0 + r] = tile[r * LD + c];
+        }
+    }
+}
+
+template <int ES> const void *transpose_fn(bool vin, bool vout)
+{
+    if (vin && vout) return (const void *)ks_transpose_kernel<ES, true, true>;
+    if (vin) return (const void *)ks_transpose_kernel<ES, true, false>;
+    if (vout) return (const void *)ks_transpose_kernel<ES, false, true>;
+    return (const void *)ks_transpose_kernel<ES, false, false>;
+}
+
+}  // namespace
+
+// out (cols x rows) = transpose of in (rows x cols); elem_bytes in {1, 2, 4}
+int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream)
+{
+    if (rows < 1 || cols < 1 || rows > 0x7fffffffLL || cols > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    const int v = 16 / elem_bytes;
+    const bool vin = cols % v == 0 && ((uintptr_t)in & 15) == 0;
+    const bool vout = rows % v == 0 && ((uintptr_t)out & 15) == 0;
+    const void *fn = elem_bytes == 4 ? transpose_fn<4>(vin, vout)
+                                     : elem_bytes == 2 ? transpose_fn<2>(vin, vout) : transpose_fn<1>(vin, vout);
+    const int64_t tiles_r = (rows + TT - 1) / TT, tiles_c = (cols + TT - 1) / TT;
+    if (tiles_r * tiles_c > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    int rows_i = (int)rows, cols_i = (int)cols, tiles_c_i = (int)tiles_c;
+    void *args[] = {(void *)&in, (void *)&out, &rows_i, &cols_i, &tiles_c_i};
+    hipError_t e = hipLaunchKernel(fn, dim3((unsigned)(tiles_r * tiles_c)), dim3(256), args, 0, stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm

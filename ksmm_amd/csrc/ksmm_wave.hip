@@ -384,7 +384,7 @@ const WaveInst f32_insts[] = {
         H_INST(TX_, TW_, 64, 64, 8, 8, 1), H_INST(TX_, TW_, 48, 48, 4, 4, 3),                \
         H_INST(TX_, TW_, 48, 48, 4, 8, 2), H_INST(TX_, TW_, 16, 16, 4, 8, 4),                \
         H_INST(TX_, TW_, 16, 16, 4, 4, 4), H_INST(TX_, TW_, 32, 32, 8, 8, 3),                \
-        H_INST(TX_, TW_, 96, 96, 8, 4, 1)
+        H_INST(TX_, TW_, 96, 96, 8, 4, 1), H_INST(TX_, TW_, 48, 192, 8, 4, 1)
 const WaveInst h_insts[] = {H_SET(half_t, half_t)};
 const WaveInst hq_insts[] = {H_SET(half_t, fp8_t)};
 const WaveInst q_insts[] = {

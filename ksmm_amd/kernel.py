@@ -44,14 +44,16 @@ class Kernel:
 
     @staticmethod
     def forward(input, factor, bs_last, a, b, c, d, dtype=None, vsize=4, scale=1.0,
-                algo=_lib.ALGO_AUTO, variant=-1, out=None):
+                algo=_lib.ALGO_AUTO, variant=-1, out=None, workspace=None):
         """y = K x for one factor.
 
         ``input``: (a*c*d, batch) if ``bs_last`` else (batch, a*c*d); ``factor``: kernel
         format (a*d*c, b).  ``dtype`` is accepted for signature compatibility: the element
         types are taken from the tensors.  ``vsize`` is accepted and ignored (vector widths
         are part of the tile table).  fp8 inputs/weights produce an fp16 result scaled by
-        ``scale``.
+        ``scale``.  Batch-size-first factors with d > 1 that have no kernel of their own run
+        in batch-size-last layout between two transposes; the scratch tensor for that is
+        allocated here unless ``workspace`` (uint8, large enough) is passed.
         """
         lib = _lib.load()
         _check_input(input, "input")
@@ -72,11 +74,22 @@ class Kernel:
             out = torch.empty(shape, dtype=out_dtype, device=input.device)
         else:
             assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
+        yd = dtype_code(out_dtype)
         with torch.cuda.device(input.device):
-            rc = lib.ksmm_factor_forward_algo(
-                input.data_ptr(), factor.data_ptr(), out.data_ptr(), batch, a, b, c, d, xd, wd,
-                dtype_code(out_dtype), int(bs_last), float(scale), int(algo), int(variant),
-                _stream_ptr(input))
+            if algo == _lib.ALGO_AUTO and variant < 0:
+                need = lib.ksmm_factor_workspace(batch, a, b, c, d, xd, wd, yd, int(bs_last))
+                if need < 0:
+                    _lib.check(int(need))
+                if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
+                    workspace = torch.empty(need, dtype=torch.uint8, device=input.device)
+                rc = lib.ksmm_factor_forward_ws(
+                    input.data_ptr(), factor.data_ptr(), out.data_ptr(), batch, a, b, c, d, xd, wd, yd,
+                    int(bs_last), float(scale), workspace.data_ptr() if need > 0 else None,
+                    workspace.numel() * workspace.element_size() if need > 0 else 0, _stream_ptr(input))
+            else:
+                rc = lib.ksmm_factor_forward_algo(
+                    input.data_ptr(), factor.data_ptr(), out.data_ptr(), batch, a, b, c, d, xd, wd, yd,
+                    int(bs_last), float(scale), int(algo), int(variant), _stream_ptr(input))
         _lib.check(rc)
         return out
 
@@ -107,7 +120,8 @@ class Kernel:
         out_size = al * bl * dl
         out = torch.empty((out_size, batch) if bs_last else (batch, out_size), dtype=out_dtype,
                           device=input.device)
-        need = lib.ksmm_chain_workspace(descs, n, batch, dtype_code(out_dtype))
+        need = lib.ksmm_chain_workspace_layout(descs, n, batch, dtype_code(input.dtype),
+                                               dtype_code(out_dtype), int(bs_last))
         if need < 0:
             _lib.check(int(need))
         if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):

@@ -19,6 +19,7 @@ SMALL_PATTERNS = [
     (16, 16, 16, 4), (64, 16, 16, 1), (2, 32, 64, 2), (1, 64, 32, 4), (3, 48, 16, 2),
     (1, 96, 96, 2), (1, 128, 128, 1), (2, 192, 192, 1), (1, 256, 64, 2), (1, 80, 48, 1),
     (1, 17, 33, 2), (2, 16, 16, 16), (1, 64, 64, 4), (2, 48, 48, 8), (2, 64, 32, 2), (1, 128, 64, 4), (3, 32, 32, 8), (1, 256, 128, 2),
+    (2, 48, 192, 2), (1, 64, 256, 2), (1, 192, 48, 3),
 ]
 BATCHES = [1, 7, 64, 200, 1024]
 
@@ -194,6 +195,60 @@ def test_fused_radix16_chain_matches_unfused_and_oracle(prec):
             assert O.rel_fro_error(outs[True], z) <= TOL[prec], (patterns, batch, "fused")
             assert O.rel_fro_error(outs[False], z) <= TOL[prec], (patterns, batch, "unfused")
             assert O.rel_fro_error(outs[True], outs[False]) <= 2e-3, (patterns, batch)
+
+
+@pytest.mark.parametrize("prec", ["fp32", "fp16", "fp8"])
+def test_bs_first_strided_blocks_take_the_transposed_route(prec):
+    """Batch-size-first factors with d > 1 and no kernel of their own: the library asks for a
+    workspace, runs them in batch-size-last layout between two transposes, and agrees with the
+    oracle and with the generic kernel; so does a whole chain (KSLinear), fused or not."""
+    import ctypes
+    from ksmm_amd import Kernel, KSLinear, generate_factor, _lib
+    from ksmm_amd.kernel import dtype_code, query_tile
+
+    lib = _lib.load()
+    dt = TORCH_DTYPE[prec]
+    for pattern, batch in [((1, 192, 192, 16), 512), ((2, 128, 128, 8), 328), ((4, 64, 64, 8), 1000),
+                           ((1, 96, 96, 6), 77), ((2, 64, 256, 8), 256)]:
+        a, b, c, d = pattern
+        ydt = torch.float16 if prec == "fp8" else dt
+        need = lib.ksmm_factor_workspace(batch, a, b, c, d, dtype_code(dt), dtype_code(dt), dtype_code(ydt), 0)
+        assert lib.ksmm_factor_workspace(batch, a, b, c, d, dtype_code(dt), dtype_code(dt), dtype_code(ydt), 1) == 0
+        y, z = _run_factor(pattern, batch, prec, False, "auto")
+        assert O.rel_fro_error(y, z) <= TOL[prec], (pattern, batch)
+        direct = query_tile(batch, pattern, dt, dt, False)["algo"] != 1   # e.g. the fp32 row kernel
+        twin = query_tile(batch, pattern, dt, dt, True)["algo"] != 1      # batch-size-last kernel
+        if direct or not twin:
+            assert need == 0, pattern
+            continue
+        assert need > 0, pattern
+        # too small a workspace is an error, not a silent fallback
+        (w4,) = seeded_weights([pattern], seed=0)
+        fac = generate_factor(a, b, c, d, "kernel", w4 if prec != "fp8" else round_to(w4, prec)[1].float(), dt, "cuda")
+        xin = torch.zeros(batch, a * c * d, device="cuda").to(dt)
+        out = torch.empty(batch, a * b * d, device="cuda", dtype=ydt)
+        small = torch.empty(256, dtype=torch.uint8, device="cuda")
+        rc = lib.ksmm_factor_forward_ws(xin.data_ptr(), fac.data_ptr(), out.data_ptr(), batch, a, b, c, d,
+                                        dtype_code(dt), dtype_code(dt), dtype_code(ydt), 0, 1.0,
+                                        small.data_ptr(), 256, None)
+        assert rc == -9
+    # chains: butterfly (fused between the transposes) and a mixed one
+    for patterns, batch in [([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], 400),
+                            ([(2, 64, 64, 8), (16, 64, 64, 1)], 264)]:
+        if prec == "fp32" and patterns[0][1] == 16:
+            continue
+        ws4 = seeded_weights(patterns, seed=41, bound=0.25)
+        n_in = patterns[0][0] * patterns[0][2] * patterns[0][3]
+        x = seeded_input(n_in, batch, False, seed=42)
+        ksl = KSLinear(patterns, weights=ws4, bias=False, algo="kernel", dtype=dt, bs_last=False, device="cuda")
+        if prec == "fp8":
+            xr, xq, xs = round_to(x, prec)
+            y = ksl(xq.cuda(), x_scale=xs).float().cpu().numpy()
+        else:
+            xr = round_to(x, prec)[0]
+            y = ksl(x.to(dt).cuda()).float().cpu().numpy()
+        z = oracle_chain([round_to(w, prec)[0] for w in ws4], xr, False)
+        assert O.rel_fro_error(y, z) <= TOL[prec], (patterns, batch)
 
 
 def test_layouts_agree_full_batch():

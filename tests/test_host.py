@@ -190,3 +190,27 @@ def test_kernel_forward_host_checks():
     w = torch.zeros(8, 2)
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):   # kernel.cpp:19
         Kernel.forward(x, w, False, 1, 2, 8, 1)
+
+
+def test_workspace_queries_need_no_gpu():
+    """ksmm_factor_workspace / ksmm_chain_workspace_layout are host-only: 0 for problems with a
+    kernel of their own, room for the transposed operands for batch-size-first d > 1 blocks."""
+    import ctypes
+    from ksmm_amd import _lib
+
+    lib = _lib.load()
+    F16 = _lib.KSMM_F16
+    assert lib.ksmm_factor_workspace(1024, 4, 192, 192, 1, F16, F16, F16, 0) == 0
+    assert lib.ksmm_factor_workspace(1024, 1, 192, 192, 16, F16, F16, F16, 1) == 0
+    need = lib.ksmm_factor_workspace(1024, 1, 192, 192, 16, F16, F16, F16, 0)
+    assert need == 2 * (192 * 16 * 1024 * 2)
+    assert lib.ksmm_factor_workspace(0, 1, 192, 192, 16, F16, F16, F16, 0) == -3
+    descs = (_lib.KsmmFactorDesc * 2)()
+    for i, (a, b, c, d) in enumerate([(2, 64, 64, 8), (16, 64, 64, 1)]):
+        descs[i].w = 0
+        descs[i].a, descs[i].b, descs[i].c, descs[i].d = a, b, c, d
+        descs[i].w_dtype = F16
+        descs[i].scale = 1.0
+    plain = lib.ksmm_chain_workspace(descs, 2, 512, F16)
+    assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 1) == plain
+    assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 0) == 3 * (1024 * 512 * 2)
