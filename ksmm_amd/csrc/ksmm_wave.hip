@@ -372,7 +372,7 @@ using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int,
      (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_, false>}
 const WaveInst f32_insts[] = {
     F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
-    F32_INST(16, 16, 4), F32_INST(32, 32, 3),
+    F32_INST(16, 16, 4), F32_INST(32, 32, 3), F32_INST(48, 192, 1),
 };
 
 #define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_)                           \
@@ -384,14 +384,15 @@ const WaveInst f32_insts[] = {
         H_INST(TX_, TW_, 64, 64, 8, 8, 1), H_INST(TX_, TW_, 48, 48, 4, 4, 3),                \
         H_INST(TX_, TW_, 48, 48, 4, 8, 2), H_INST(TX_, TW_, 16, 16, 4, 8, 4),                \
         H_INST(TX_, TW_, 16, 16, 4, 4, 4), H_INST(TX_, TW_, 32, 32, 8, 8, 3),                \
-        H_INST(TX_, TW_, 96, 96, 8, 4, 1), H_INST(TX_, TW_, 48, 192, 8, 4, 1)
+        H_INST(TX_, TW_, 96, 96, 8, 4, 1), H_INST(TX_, TW_, 48, 192, 8, 4, 1),              \
+        H_INST(TX_, TW_, 192, 48, 4, 4, 1)
 const WaveInst h_insts[] = {H_SET(half_t, half_t)};
 const WaveInst hq_insts[] = {H_SET(half_t, fp8_t)};
 const WaveInst q_insts[] = {
     H_INST(fp8_t, fp8_t, 64, 64, 8, 8, 2),  H_INST(fp8_t, fp8_t, 64, 64, 8, 8, 1),
     H_INST(fp8_t, fp8_t, 48, 48, 4, 8, 2),  H_INST(fp8_t, fp8_t, 16, 16, 4, 8, 4),
     H_INST(fp8_t, fp8_t, 16, 16, 4, 16, 3), H_INST(fp8_t, fp8_t, 32, 32, 8, 16, 2),
-    H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),
+    H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),  H_INST(fp8_t, fp8_t, 48, 192, 8, 8, 1),
 };
 
 }  // namespace
