@@ -101,6 +101,85 @@ def test_gemm_kernels_forced():
     assert ran >= 12
 
 
+def _forced_sweep(cases, variants, algo, min_ran):
+    """Every (case, variant) the family accepts must agree with the oracle; the others must be
+    refused with KSMM_ERR_BAD_ALGO."""
+    from ksmm_amd import Kernel, generate_factor, quantize_fp8, _lib
+
+    ran = 0
+    for prec, bs_last, pattern, batch in cases:
+        a, b, c, d = pattern
+        (w4,) = seeded_weights([pattern], seed=51)
+        x = seeded_input(a * c * d, batch, bs_last, seed=52)
+        if prec == "hq":  # fp16 activations, e4m3fn weights
+            wq, ws = quantize_fp8(w4)
+            fac = generate_factor(a, b, c, d, "kernel", wq.to(torch.float32), torch.float8_e4m3fn, "cuda")
+            xin, scale, tol = x.half().cuda(), float(ws), TOL["fp16"]
+            z = O.ks_apply_einsum((wq.to(torch.float32) * ws).double().numpy(), x.half().double().numpy(), bs_last)
+        elif prec == "fp8":
+            wr, wq, ws = round_to(w4, prec)
+            xr, xq, xs = round_to(x, prec)
+            fac = generate_factor(a, b, c, d, "kernel", wq.to(torch.float32), torch.float8_e4m3fn, "cuda")
+            xin, scale, tol = xq.cuda(), ws * xs, TOL["fp8"]
+            z = O.ks_apply_einsum(wr, xr, bs_last)
+        else:
+            dt = TORCH_DTYPE[prec]
+            fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+            xin, scale, tol = x.to(dt).cuda(), 1.0, TOL[prec]
+            z = O.ks_apply_einsum(round_to(w4, prec)[0], round_to(x, prec)[0], bs_last)
+        for variant in variants:
+            try:
+                y = Kernel.forward(xin, fac, bs_last, a, b, c, d, scale=scale, algo=algo, variant=variant)
+            except _lib.KsmmError as e:
+                assert e.status == -6, (prec, bs_last, pattern, variant, e)
+                continue
+            ran += 1
+            err = O.rel_fro_error(y.float().cpu().numpy(), z)
+            assert err <= tol, (prec, bs_last, pattern, batch, hex(variant), err)
+    assert ran >= min_ran, ran
+
+
+def test_wave_instances_forced():
+    """Every instance of the wave family (all four type combinations), one tile per wave and
+    several, consecutive and round-robin tiles, with a ragged last tile."""
+    shapes = [(2, 48, 48, 3), (2, 64, 64, 2), (3, 16, 16, 5), (2, 32, 32, 3), (1, 96, 96, 2), (2, 48, 192, 2),
+              (1, 192, 48, 3)]
+    cases = [(prec, True, p, 1040) for prec in ("fp32", "fp16", "hq", "fp8") for p in shapes]
+    variants = [inst | (it << 8) | (rr << 16) for inst in range(12) for it, rr in ((1, 0), (3, 0), (2, 1))]
+    _forced_sweep(cases, variants, 2, 100)
+
+
+def test_row_kernel_instances_forced():
+    """Every instance of the batch-size-first row kernel, full and ragged batch tiles."""
+    shapes = [(2, 48, 48, 16), (1, 48, 48, 8), (2, 48, 48, 4), (1, 64, 64, 8), (2, 64, 64, 4), (1, 16, 16, 16),
+              (3, 16, 16, 4), (2, 32, 32, 8)]
+    cases = [("fp32", False, p, batch) for p in shapes for batch in (512, 203)]
+    _forced_sweep(cases, [1000 + i for i in range(12)], 2, 16)
+
+
+def test_tile_subfamilies_forced():
+    """Stream, weight-stationary, k-loop and batch-size-first (d > 1) tiles: every instance on
+    shapes it can take."""
+    cases = []
+    for prec in ("fp16", "hq"):
+        for bs_last in (True, False):
+            for p in [(2, 64, 64, 1), (3, 128, 128, 1), (2, 192, 192, 1)]:
+                cases.append((prec, bs_last, p, 1000))
+    cases += [("fp32", True, (2, 64, 64, 1), 1000), ("fp32", True, (1, 128, 128, 1), 1000)]
+    _forced_sweep(cases, [(2 << 24) | i for i in range(28)], 3, 24)                      # stream
+    kcases = [("fp16", True, (2, 128, 64, 2), 520), ("fp16", False, (2, 128, 64, 1), 520),
+              ("fp32", True, (1, 128, 64, 3), 520), ("fp32", False, (2, 64, 32, 1), 520),
+              ("fp8", True, (2, 128, 64, 2), 528), ("hq", False, (1, 256, 128, 1), 520)]
+    _forced_sweep(kcases, [(0 << 24) | i for i in range(56)], 3, 20)                     # k-loop
+    wcases = [("fp32", True, (2, 64, 64, 2), 520), ("fp32", False, (2, 96, 96, 1), 520),
+              ("fp16", True, (2, 64, 64, 2), 520), ("fp16", False, (3, 64, 64, 1), 520),
+              ("fp8", True, (2, 64, 64, 1), 528), ("hq", False, (2, 96, 96, 1), 520)]
+    _forced_sweep(wcases, [(1 << 24) | i for i in range(64)], 3, 6)                      # weight-stationary
+    bcases = [("fp16", False, (2, 128, 64, 2), 520), ("fp16", False, (1, 64, 64, 4), 520),
+              ("fp32", False, (2, 64, 32, 2), 520), ("hq", False, (1, 128, 128, 2), 520)]
+    _forced_sweep(bcases, [(3 << 24) | i for i in range(16)], 3, 4)                      # d > 1 tiles
+
+
 def test_fp16_input_fp8_weight_factor():
     """Chain intermediate type: fp16 activations times e4m3fn weights."""
     from ksmm_amd import Kernel, generate_factor, quantize_fp8
