@@ -93,7 +93,11 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
             const int v = tid + i * C::THREADS;
             if (C::W_VECS % C::THREADS == 0 || v < C::W_VECS) {
                 const int kk = v / (TM / C::W_EPV), mm = (v % (TM / C::W_EPV)) * C::W_EPV;
-                wreg[i].load(wg + (size_t)(k0 + kk) * b + mm);
+                // batch-size-last: c need not be a multiple of TK; rows past the block are zeros
+                if (BS_LAST && k0 + kk >= c)
+                    wreg[i].v = uint4_t{0u, 0u, 0u, 0u};
+                else
+                    wreg[i].load(wg + (size_t)(k0 + kk) * b + mm);
             }
         }
 #pragma unroll
@@ -104,7 +108,10 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
                     const int kk = v / (TN / C::X_EPV), nn = (v % (TN / C::X_EPV)) * C::X_EPV;
                     // columns past the end are clamped to the last valid vector (never stored)
                     const int col = min(n0 + nn, batch - C::X_EPV);
-                    xreg[i].load(xg + (size_t)(k0 + kk) * x_kstride + col);
+                    if (k0 + kk >= c)
+                        xreg[i].v = uint4_t{0u, 0u, 0u, 0u};
+                    else
+                        xreg[i].load(xg + (size_t)(k0 + kk) * x_kstride + col);
                 } else {
                     const int nn = v / (TK / C::X_EPV), kk = (v % (TK / C::X_EPV)) * C::X_EPV;
                     const int row = min(n0 + nn, batch - 1);
@@ -145,7 +152,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int steps = c / TK;
+    const int steps = BS_LAST ? (c + TK - 1) / TK : c / TK;
     gload(0);
     lstore(0);
     __syncthreads();
@@ -498,7 +505,8 @@ constexpr int N_TILE_INSTS = sizeof(tile_insts) / sizeof(TileInst);
 bool tile_fits(const TileInst &t, const Problem &p, int combo)
 {
     if (t.combo != combo || t.bs_last != p.bs_last) return false;
-    if (p.b % t.tm || p.c % t.tk) return false;
+    if (p.b % t.tm) return false;
+    if (!p.bs_last && p.c % t.tk) return false;  // batch-size-last tiles zero-fill the K tail
     const int x_epv = 16 / (int)dtype_size(p.x_dtype), w_epv = 16 / (int)dtype_size(p.w_dtype);
     // 16-byte global vectors: weight rows (b elements) and input rows must keep alignment
     if (p.b % w_epv) return false;

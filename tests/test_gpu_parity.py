@@ -20,6 +20,7 @@ SMALL_PATTERNS = [
     (1, 96, 96, 2), (1, 128, 128, 1), (2, 192, 192, 1), (1, 256, 64, 2), (1, 80, 48, 1),
     (1, 17, 33, 2), (2, 16, 16, 16), (1, 64, 64, 4), (2, 48, 48, 8), (2, 64, 32, 2), (1, 128, 64, 4), (3, 32, 32, 8), (1, 256, 128, 2),
     (2, 48, 192, 2), (1, 64, 256, 2), (1, 192, 48, 3),
+    (1, 64, 50, 3), (2, 32, 18, 1), (1, 128, 70, 2),                            # c not a multiple of the K tile
 ]
 BATCHES = [1, 7, 64, 200, 1024]
 
