@@ -487,10 +487,11 @@ const GemmInst gemm_insts[] = {
     // traffic per MFMA of the 8-wave tiles above
     GEMM_INST(1, half_t, false, 2, 256, 128, 32, 2, 2, 3),
     GEMM_INST(1, half_t, false, 2, 128, 256, 32, 1, 4, 3),
-    // fp16, b a multiple of 64 only
+    // fp16, b a multiple of 64 only: last resort (variant -2), after the stream and k-loop tiles
     GEMM_INST(1, half_t, true, 1, 64, 256, 32, 1, 4, 3),
     GEMM_INST(1, half_t, false, 1, 64, 256, 32, 1, 4, 3),
 };
+constexpr int N_GEMM_FIRST_CHOICE = 19;  // entries the automatic choice (variant -1) looks at
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 
 bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
@@ -524,6 +525,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int pick = -1;
     for (int i = 0; i < N_GEMM_INSTS; ++i) {
         if (variant >= 0 && variant != i) continue;
+        if (variant == -1 && i >= N_GEMM_FIRST_CHOICE) break;
         const GemmInst &t = gemm_insts[i];
         if (!gemm_fits(t, p, combo)) continue;
         if (variant == -1) {
