@@ -30,15 +30,16 @@ __device__ __forceinline__ half_t fp8_to_half(uint8_t v)
     return __builtin_bit_cast(half_t, h) * (half_t)256.0f;
 }
 
-// Two e4m3fn bytes (bits 0-7 and 8-15 of `v`) -> packed fp16 pair.
+// Two e4m3fn bytes (bits 0-7 and 8-15 of `v`) -> packed fp16 pair: the hardware conversion
+// (v_cvt_scalef32_pk_f16_fp8 with unit scale; exact, every e4m3fn value is an fp16 value).
 __device__ __forceinline__ half2_t fp8x2_to_half2(uint32_t v)
 {
-    // bytes -> high byte of each 16-bit lane: 0x b1 00 b0 00
-    uint32_t u = __builtin_amdgcn_perm(0u, v, 0x010c000cu);
-    uint32_t t = ((u >> 1) & 0x3f803f80u) | (u & 0x80008000u);
-    half2_t h = __builtin_bit_cast(half2_t, t);
-    half2_t k = {(half_t)256.0f, (half_t)256.0f};
-    return h * k;
+    return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(v, 1.0f, false);
+}
+// the same for bits 16-23 and 24-31
+__device__ __forceinline__ half2_t fp8x2_hi_to_half2(uint32_t v)
+{
+    return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(v, 1.0f, true);
 }
 
 template <typename T> struct elem;

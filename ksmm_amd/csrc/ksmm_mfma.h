@@ -40,9 +40,9 @@ template <> struct stage<fp8_t, half_t> {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             lo[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[i]));
-            lo[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[i] >> 16));
+            lo[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_hi_to_half2(v[i]));
             hi[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[2 + i]));
-            hi[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(v[2 + i] >> 16));
+            hi[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_hi_to_half2(v[2 + i]));
         }
         *(uint4_t *)l = lo;
         *(uint4_t *)(l + 8) = hi;

@@ -85,7 +85,7 @@ template <int VEC> struct row_io<fp8_t, VEC> {
 #pragma unroll
         for (int i = 0; i < RAW; ++i) {
             o[2 * i] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(in[i]));
-            o[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(in[i] >> 16));
+            o[2 * i + 1] = __builtin_bit_cast(uint32_t, fp8x2_hi_to_half2(in[i]));
         }
     }
 };
