@@ -78,7 +78,10 @@ __device__ __forceinline__ half4_t fp8x4_to_half4(uint32_t v)
     return half4_t{lo[0], lo[1], hi[0], hi[1]};
 }
 
-template <typename TX, typename TW, int NF>
+// FULL: 1024 features (every wave has MAXB blocks per factor) and a batch that is a multiple of
+// the chunk: no tile is ragged, so the chunk loop has no branches and the compiler's memory
+// counters stay exact (a chunk's stores drain while the next chunk is staged and multiplied).
+template <typename TX, typename TW, int NF, bool FULL>
 __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__restrict__ x, half_t *__restrict__ y,
                                                          Chain16Args args, int batch, int n_feat)
 {
@@ -89,6 +92,7 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
     // workgroup takes chunks blockIdx.x, blockIdx.x + gridDim.x, ...
     const int c_begin = blockIdx.x * CH_TN, c_step = gridDim.x * CH_TN, c_end = batch;
     if (c_begin >= c_end) return;
+    const int c_last = c_begin + ((c_end - 1 - c_begin) / c_step) * c_step;  // this workgroup's last chunk
     const int n_blocks = n_feat / 16;  // blocks per factor
     KC_STAMP(0);
     int chunk_no = 0;
@@ -110,14 +114,15 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         for (int i = 0; i < X_PER_T; ++i) {
             const int p = tid + i * CH_THREADS, row = piece_row(p / X_PPR), pc = p % X_PPR;
             const int col = min(n0 + pc * (16 / (int)sizeof(TX)), c_end - 16 / (int)sizeof(TX));
-            if (row < n_feat) xreg[i] = *(const uint4_t *)(x + (size_t)row * batch + col);
+            // rows past the end repeat the last one (loaded, never staged): no branch here
+            xreg[i] = *(const uint4_t *)(x + (size_t)min(row, n_feat - 1) * batch + col);
         }
     };
     auto lstore = [&]() {
 #pragma unroll
         for (int i = 0; i < X_PER_T; ++i) {
             const int p = tid + i * CH_THREADS, row = piece_row(p / X_PPR), pc = p % X_PPR;
-            if (row < n_feat) {
+            if (FULL || row < n_feat) {
                 if constexpr (sizeof(TX) == 1) {
                     // e4m3fn: columns 16*pc .. +15 = pieces p0, p0+1 of slots 2t, 2t+1
                     const int off = lds_piece(row, 2 * (pc >> 1), 2 * (pc & 1));
@@ -150,14 +155,18 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                 const int v = min(tid + i * CH_THREADS, n_vec - 1);
                 wv[f][i] = *((const uint4_t *)args.w[f] + v);
             }
+        // the weights' loads go first and are waited for alone: staging them overlaps with the
+        // flight of the (HBM-bound) first chunk
+        __builtin_amdgcn_sched_barrier(0);
         gload(c_begin);
+        __builtin_amdgcn_sched_barrier(0);
         KC_STAMP(10);
 #pragma unroll
         for (int f = 0; f < NF; ++f)
 #pragma unroll
             for (int i = 0; i < W_PER_T; ++i) {
                 const int v = tid + i * CH_THREADS;
-                if (v < n_vec) {
+                if (FULL || v < n_vec) {
                     unsigned char *dst = smem + ((size_t)f * n_feat * 16 + (size_t)v * WV) * 2;
                     if constexpr (sizeof(TW) == 1) {
 #pragma unroll
@@ -195,7 +204,10 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         lstore();
         __syncthreads();
         KC_STAMP(4 + 8 * chunk_no);
-        if (n0 + c_step < c_end) gload(n0 + c_step);
+        if (FULL)
+            gload(min(n0 + c_step, c_last));  // the last chunk is requested again (not used)
+        else if (n0 + c_step < c_end)
+            gload(n0 + c_step);
         // an opaque zero: keeps the compiler from hoisting the per-block address arithmetic of
         // all NF x 8 blocks out of this loop (it would spill them)
         int opaque = 0;
@@ -214,13 +226,13 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                         half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(smem + (base ^ (s << 5)))));
             };
             half4_t xa[2][4];
-            if (wave + opaque < n_blocks) read_block(wave + opaque, xa[0]);
+            if (FULL || wave + opaque < n_blocks) read_block(wave + opaque, xa[0]);
 #pragma unroll
             for (int bi = 0; bi < MAXB; ++bi) {
                 const int g = wave + CH_WAVES * bi + opaque;
-                if (g >= n_blocks) break;  // uniform
+                if (!FULL && g >= n_blocks) break;  // uniform
                 // the next block's rows are not this block's: read them before this block writes
-                if (bi + 1 < MAXB && g + CH_WAVES < n_blocks) read_block(g + CH_WAVES, xa[(bi + 1) & 1]);
+                if (bi + 1 < MAXB && (FULL || g + CH_WAVES < n_blocks)) read_block(g + CH_WAVES, xa[(bi + 1) & 1]);
                 float4_t acc[4];
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
@@ -243,7 +255,7 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                     half_t *yrow = y + (size_t)(row0 | (r << ld)) * batch + n0 + 8 * q;
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
-                        if (n0 + 32 * t + 8 * q < c_end)
+                        if (FULL || n0 + 32 * t + 8 * q < c_end)
                             *(half8_t *)(yrow + 32 * t) = half8_t{o[2 * t][0], o[2 * t][1], o[2 * t][2], o[2 * t][3],
                                                                   o[2 * t + 1][0], o[2 * t + 1][1], o[2 * t + 1][2], o[2 * t + 1][3]};
                 }
@@ -256,12 +268,12 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
     KC_STAMP(2);
 }
 
-template <typename TX, typename TW> const void *chain16_fn(int nf)
+template <typename TX, typename TW> const void *chain16_fn(int nf, bool full)
 {
     switch (nf) {
-    case 2: return (const void *)ks_chain16_kernel<TX, TW, 2>;
-    case 3: return (const void *)ks_chain16_kernel<TX, TW, 3>;
-    case 4: return (const void *)ks_chain16_kernel<TX, TW, 4>;
+    case 2: return full ? (const void *)ks_chain16_kernel<TX, TW, 2, true> : (const void *)ks_chain16_kernel<TX, TW, 2, false>;
+    case 3: return full ? (const void *)ks_chain16_kernel<TX, TW, 3, true> : (const void *)ks_chain16_kernel<TX, TW, 3, false>;
+    case 4: return full ? (const void *)ks_chain16_kernel<TX, TW, 4, true> : (const void *)ks_chain16_kernel<TX, TW, 4, false>;
     default: return nullptr;
     }
 }
@@ -289,13 +301,14 @@ int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_
     for (int i = 0; i < n; ++i)
         if ((uintptr_t)f[i].w & 15) return KSMM_ERR_BAD_ALGO;
     if (!launch) return KSMM_OK;
+    const bool full = n_feat == 1024 && batch % CH_TN == 0;
     const void *fn;
     if (x_dtype == KSMM_FP8_E4M3)
-        fn = chain16_fn<fp8_t, fp8_t>(n);
+        fn = chain16_fn<fp8_t, fp8_t>(n, full);
     else if (f[0].w_dtype == KSMM_FP8_E4M3)
-        fn = chain16_fn<half_t, fp8_t>(n);
+        fn = chain16_fn<half_t, fp8_t>(n, full);
     else
-        fn = chain16_fn<half_t, half_t>(n);
+        fn = chain16_fn<half_t, half_t>(n, full);
     Chain16Args args;
     for (int i = 0; i < 4; ++i) {
         const int j = i < n ? i : n - 1;
