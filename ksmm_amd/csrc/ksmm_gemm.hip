@@ -434,11 +434,12 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
                 if constexpr (BS_LAST) {
                     const int n = n0 + cc;
                     if (n < batch)
-                        *(uint4_t *)(y + ((size_t)(a_i * b + m0 + row) * d + d_i) * batch + n) = v;
+                        __builtin_nontemporal_store(v, (uint4_t *)(y + ((size_t)(a_i * b + m0 + row) * d + d_i) * batch + n));
                 } else {
                     const int n = n0 + row;
+                    // whole runs of TM*DD outputs per batch row: streaming stores
                     if (n < batch)
-                        *(uint4_t *)(y + (size_t)n * out_size + ((size_t)a_i * b + m0) * DD + cc) = v;
+                        __builtin_nontemporal_store(v, (uint4_t *)(y + (size_t)n * out_size + ((size_t)a_i * b + m0) * DD + cc));
                 }
             }
         }
