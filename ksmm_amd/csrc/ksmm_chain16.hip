@@ -109,13 +109,16 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
     auto piece_row = [](int u) {
         return sizeof(TX) == 1 ? (u & ~6) | ((u & 2) << 1) | ((u & 4) >> 1) : u;
     };
-    auto gload = [&](int n0) {
+    // `real` == false (uniform): nothing to fetch, every lane reads the same 16 bytes instead, so
+    // that the instruction count stays the same without the traffic
+    auto gload = [&](int n0, bool real) {
 #pragma unroll
         for (int i = 0; i < X_PER_T; ++i) {
             const int p = tid + i * CH_THREADS, row = piece_row(p / X_PPR), pc = p % X_PPR;
             const int col = min(n0 + pc * (16 / (int)sizeof(TX)), c_end - 16 / (int)sizeof(TX));
             // rows past the end repeat the last one (loaded, never staged): no branch here
-            xreg[i] = *(const uint4_t *)(x + (size_t)min(row, n_feat - 1) * batch + col);
+            const TX *src = x + (size_t)min(row, n_feat - 1) * batch + col;
+            xreg[i] = *(const uint4_t *)(real ? src : x + c_begin);
         }
     };
     auto lstore = [&]() {
@@ -158,7 +161,7 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         // the weights' loads go first and are waited for alone: staging them overlaps with the
         // flight of the (HBM-bound) first chunk
         __builtin_amdgcn_sched_barrier(0);
-        gload(c_begin);
+        gload(c_begin, true);
         __builtin_amdgcn_sched_barrier(0);
         KC_STAMP(10);
 #pragma unroll
@@ -205,9 +208,9 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         __syncthreads();
         KC_STAMP(4 + 8 * chunk_no);
         if (FULL)
-            gload(min(n0 + c_step, c_last));  // the last chunk is requested again (not used)
+            gload(min(n0 + c_step, c_last), n0 + c_step < c_end);  // after the last chunk: a dummy request
         else if (n0 + c_step < c_end)
-            gload(n0 + c_step);
+            gload(n0 + c_step, true);
         // an opaque zero: keeps the compiler from hoisting the per-block address arithmetic of
         // all NF x 8 blocks out of this loop (it would spill them)
         int opaque = 0;
