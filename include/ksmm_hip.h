@@ -100,6 +100,20 @@ int ksmm_validate(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_
 int ksmm_query_tile(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
                     int y_dtype, int bs_last, int algo, ksmm_tile *out);
 
+/* The same for one forced instance: `variant` as in ksmm_factor_forward_algo; with
+ * KSMM_ALGO_AUTO, -1 = measured table first, then the heuristics, -3 = heuristics only. */
+int ksmm_query_tile_variant(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                            int y_dtype, int bs_last, int algo, int variant, ksmm_tile *out);
+
+/* The measured table KSMM_ALGO_AUTO consults for batches of 8192 and more: the counterpart
+ * of the reference's tuned `*.best` files and the if-chains generated from them
+ * (src/ksmm_py/layer/kronecker_sparse/kernel.py:151-257).  Row i is
+ * {a, b, c, d, combo, bs_last, algo, variant}, combo 0 = fp32, 1 = fp16, 2 = e4m3 -> fp16;
+ * rows are sorted by (a, b, c, d, combo, bs_last).  Patterns without a row use the
+ * heuristic order of kernel families. */
+int ksmm_tuned_count(void);
+int ksmm_tuned_row(int index, int row[8]);
+
 /* One factor.  Replaces `kernel.forward(input, factor, bs_last, a, b, c, d, dtype, vsize)`
  * (src/ksmm_py/layer/kronecker_sparse/kernel.cpp:25-45 -> kernel.cu:40-127); the caller
  * allocates y. */

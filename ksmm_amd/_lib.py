@@ -39,6 +39,10 @@ SIGNATURES = {
     "ksmm_validate": (c_int, [c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "ksmm_query_tile": (c_int, [c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                 ctypes.POINTER(KsmmTile)]),
+    "ksmm_query_tile_variant": (c_int, [c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_int, ctypes.POINTER(KsmmTile)]),
+    "ksmm_tuned_count": (c_int, []),
+    "ksmm_tuned_row": (c_int, [c_int, ctypes.POINTER(c_int * 8)]),
     "ksmm_factor_forward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, ctypes.c_float, c_vp]),
     "ksmm_factor_forward_algo": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int,

@@ -33,6 +33,42 @@ int check_shape(int64_t batch, int a, int b, int c, int d, int xd, int wd, int y
     return KSMM_OK;
 }
 
+// Measured choices for known patterns (the counterpart of the reference's *.best tables,
+// src/ksmm_py/layer/kronecker_sparse/kernel.py:151-239): rows sorted by key.
+struct TunedRow {
+    int a, b, c, d, combo, bs_last, algo, variant;
+};
+const TunedRow tuned_rows[] = {
+#include "ksmm_tuned.inc"
+    {0, 0, 0, 0, 0, 0, 0, 0},  // sentinel: keeps the array non-empty
+};
+constexpr int N_TUNED = (int)(sizeof(tuned_rows) / sizeof(TunedRow)) - 1;
+constexpr int64_t TUNED_MIN_BATCH = 8192;  // the table was measured at batch 25088
+
+int cmp_key(const TunedRow &r, const Problem &p, int combo)
+{
+    const int k[6] = {p.a, p.b, p.c, p.d, combo, p.bs_last};
+    const int q[6] = {r.a, r.b, r.c, r.d, r.combo, r.bs_last};
+    for (int i = 0; i < 6; ++i)
+        if (q[i] != k[i]) return q[i] < k[i] ? -1 : 1;
+    return 0;
+}
+
+const TunedRow *tuned_lookup(const Problem &p)
+{
+    const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
+    int lo = 0, hi = N_TUNED - 1;
+    while (lo <= hi) {
+        const int mid = (lo + hi) / 2, c = cmp_key(tuned_rows[mid], p, combo);
+        if (c == 0) return &tuned_rows[mid];
+        if (c < 0)
+            lo = mid + 1;
+        else
+            hi = mid - 1;
+    }
+    return nullptr;
+}
+
 // Family order for KSMM_ALGO_AUTO: the table inside each family decides whether it takes the
 // problem; the generic family always does.
 int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *tile)
@@ -42,6 +78,15 @@ int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *ti
     case KSMM_ALGO_WAVE: return wave_run(p, variant, launch, tile);
     case KSMM_ALGO_TILE: return tile_run(p, variant, launch, tile);
     case KSMM_ALGO_AUTO: {
+        // variant -1: the tuned table first (large batches), then the heuristics below;
+        // variant -3: heuristics only (what the tuner compares against)
+        if (variant == -1 && p.batch >= TUNED_MIN_BATCH) {
+            const TunedRow *row = tuned_lookup(p);
+            if (row && row->algo != KSMM_ALGO_AUTO) {
+                const int rc = dispatch(p, row->algo, row->variant, launch, tile);
+                if (rc != KSMM_ERR_BAD_ALGO) return rc;
+            }
+        }
         // Table order from sweeps at batch 25088: batch-size-first 16-bit mid-sized blocks
         // (64x64 .. 192x192) go to the stream kernels of the tile family; batch-size-last blocks
         // the wave family has an instance for (up to 96x96), and fp32, go to the wave family,
@@ -118,6 +163,30 @@ int ksmm_query_tile(int64_t batch, int a, int b, int c, int d, int x_dtype, int 
               bs_last ? 1 : 0, 1.f, nullptr};
     memset(out, 0, sizeof(*out));
     return dispatch(p, algo, -1, false, out);
+}
+
+int ksmm_query_tile_variant(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
+                            int y_dtype, int bs_last, int algo, int variant, ksmm_tile *out)
+{
+    if (!out) return KSMM_ERR_NULL_POINTER;
+    int rc = check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    Problem p{nullptr, nullptr, nullptr, batch, a, b, c, d, x_dtype, w_dtype, y_dtype,
+              bs_last ? 1 : 0, 1.f, nullptr};
+    memset(out, 0, sizeof(*out));
+    return dispatch(p, algo, variant, false, out);
+}
+
+int ksmm_tuned_count(void) { return N_TUNED; }
+
+int ksmm_tuned_row(int index, int row[8])
+{
+    if (!row) return KSMM_ERR_NULL_POINTER;
+    if (index < 0 || index >= N_TUNED) return KSMM_ERR_BAD_ALGO;
+    const TunedRow &r = tuned_rows[index];
+    const int v[8] = {r.a, r.b, r.c, r.d, r.combo, r.bs_last, r.algo, r.variant};
+    for (int i = 0; i < 8; ++i) row[i] = v[i];
+    return KSMM_OK;
 }
 
 int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batch, int a,

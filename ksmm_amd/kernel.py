@@ -76,7 +76,7 @@ class Kernel:
             assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
         yd = dtype_code(out_dtype)
         with torch.cuda.device(input.device):
-            if algo == _lib.ALGO_AUTO and variant < 0:
+            if algo == _lib.ALGO_AUTO and variant == -1:
                 need = lib.ksmm_factor_workspace(batch, a, b, c, d, xd, wd, yd, int(bs_last))
                 if need < 0:
                     _lib.check(int(need))
@@ -136,14 +136,27 @@ class Kernel:
         return out
 
 
-def query_tile(batch, pattern, x_dtype, w_dtype=None, bs_last=True, algo=_lib.ALGO_AUTO):
-    """What the tile table picks for one factor (host only; no GPU needed)."""
+def query_tile(batch, pattern, x_dtype, w_dtype=None, bs_last=True, algo=_lib.ALGO_AUTO, variant=-1):
+    """What the tile table picks for one factor (host only; no GPU needed).  With the automatic
+    choice, variant -1 consults the measured table first and -3 only the heuristics."""
     lib = _lib.load()
     w_dtype = x_dtype if w_dtype is None else w_dtype
     y_dtype = torch.float16 if w_dtype == torch.float8_e4m3fn else x_dtype
     t = _lib.KsmmTile()
     a, b, c, d = pattern
-    _lib.check(lib.ksmm_query_tile(batch, a, b, c, d, dtype_code(x_dtype), dtype_code(w_dtype),
-                                   dtype_code(y_dtype), int(bool(bs_last)), int(algo),
-                                   ctypes.byref(t)))
+    _lib.check(lib.ksmm_query_tile_variant(batch, a, b, c, d, dtype_code(x_dtype), dtype_code(w_dtype),
+                                           dtype_code(y_dtype), int(bool(bs_last)), int(algo), int(variant),
+                                           ctypes.byref(t)))
     return t.as_dict()
+
+
+def tuned_table():
+    """Rows (a, b, c, d, combo, bs_last, algo, variant) of the measured table compiled into the
+    library (combo 0 = fp32, 1 = fp16, 2 = e4m3 -> fp16)."""
+    lib = _lib.load()
+    rows = []
+    buf = (ctypes.c_int * 8)()
+    for i in range(lib.ksmm_tuned_count()):
+        _lib.check(lib.ksmm_tuned_row(i, ctypes.byref(buf)))
+        rows.append(tuple(buf))
+    return rows

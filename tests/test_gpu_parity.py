@@ -181,6 +181,44 @@ def test_tile_subfamilies_forced():
     _forced_sweep(bcases, [(3 << 24) | i for i in range(16)], 3, 4)                      # d > 1 tiles
 
 
+def test_tuned_table_rows_match_oracle():
+    """A sample of the measured table's rows (every element type and layout), run through the
+    automatic choice at a batch that consults the table, against the oracle; the tile the
+    library reports must be the row's."""
+    from ksmm_amd import Kernel, generate_factor
+    from ksmm_amd.kernel import query_tile, tuned_table
+
+    rows = [r for r in tuned_table() if r[0] * r[1] * r[2] * r[3] <= 1 << 16]
+    assert len(rows) >= 40
+    prec_of = {0: "fp32", 1: "fp16", 2: "fp8"}
+    batch = 8192
+    ran = {}
+    for a, b, c, d, combo, bs_last, algo, variant in rows[::max(1, len(rows) // 40)]:
+        prec = prec_of[combo]
+        dt = TORCH_DTYPE[prec]
+        pattern = (a, b, c, d)
+        tile = query_tile(batch, pattern, dt, None, bool(bs_last))
+        assert tile == query_tile(batch, pattern, dt, None, bool(bs_last), algo, variant)
+        (w4,) = seeded_weights([pattern], seed=11)
+        x = seeded_input(a * c * d, batch, bool(bs_last), seed=12)
+        wr, wq, ws = round_to(w4, prec)
+        xr, xq, xs = round_to(x, prec)
+        if prec == "fp8":
+            fac = generate_factor(a, b, c, d, "kernel", wq.to(torch.float32), dt, "cuda")
+            xin, scale = xq.cuda(), ws * xs
+        else:
+            fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+            xin, scale = x.to(dt).cuda(), 1.0
+        print("tuned row", pattern, prec, bs_last, algo, hex(variant), flush=True)
+        y = Kernel.forward(xin, fac, bool(bs_last), a, b, c, d, dtype=dt, scale=scale)
+        torch.cuda.synchronize()
+        z = O.ks_apply_einsum(wr, xr, bool(bs_last))
+        err = O.rel_fro_error(y.float().cpu().numpy(), z)
+        assert err <= TOL[prec], (pattern, prec, bs_last, algo, hex(variant), err)
+        ran[(combo, bs_last)] = ran.get((combo, bs_last), 0) + 1
+    assert len(ran) >= 4, ran
+
+
 def test_fp16_input_fp8_weight_factor():
     """Chain intermediate type: fp16 activations times e4m3fn weights."""
     from ksmm_amd import Kernel, generate_factor, quantize_fp8

@@ -214,3 +214,23 @@ def test_workspace_queries_need_no_gpu():
     plain = lib.ksmm_chain_workspace(descs, 2, 512, F16)
     assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 1) == plain
     assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 0) == 3 * (1024 * 512 * 2)
+
+
+def test_tuned_table_is_sorted_and_every_row_names_a_kernel_that_fits():
+    """The measured table (the counterpart of the reference's *.best files, kernel.py:151-257):
+    keys strictly ascending (binary search), every row a forced instance that takes the problem
+    at the batch it was measured on, and the automatic choice follows it there, not below 8192."""
+    from ksmm_amd.kernel import query_tile, tuned_table
+
+    rows = tuned_table()
+    keys = [r[:6] for r in rows]
+    assert keys == sorted(keys) and len(set(keys)) == len(keys)
+    dts = {0: torch.float32, 1: torch.float16, 2: torch.float8_e4m3fn}
+    for a, b, c, d, combo, bs_last, algo, variant in rows:
+        assert combo in dts and algo in (2, 3) and variant >= 0
+        forced = query_tile(25088, (a, b, c, d), dts[combo], None, bool(bs_last), algo, variant)
+        auto = query_tile(25088, (a, b, c, d), dts[combo], None, bool(bs_last))
+        assert auto == forced, (a, b, c, d, combo, bs_last)
+        small = query_tile(4096, (a, b, c, d), dts[combo], None, bool(bs_last))
+        heur = query_tile(4096, (a, b, c, d), dts[combo], None, bool(bs_last), variant=-3)
+        assert small == heur
