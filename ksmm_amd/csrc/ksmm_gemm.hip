@@ -88,6 +88,7 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
     static constexpr int W_BYTES = W_CHUNKS * 16, X_BYTES = X_CHUNKS * 16, STAGE_BYTES = W_BYTES + X_BYTES;
     static constexpr int LDS_BYTES = ST * STAGE_BYTES;
     static constexpr int N_WAIT = (ST - 2) * L;
+    static constexpr int PF = 4;  // L2 prefetch loads per thread (128-byte lines of the successor's input tile)
     static_assert(!BS_LAST || DD == 1, "DD > 1 is a batch-size-first variant");
     static_assert(ES == 2 || BS_LAST, "fp32 batch-size-first uses the plain tile kernel");
     static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0 && TK % KSTEP == 0, "wave tiling");
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
                                                               const CT *__restrict__ w,
                                                               TY *__restrict__ y, int batch, int a,
                                                               int b, int c, int d, float scale,
-                                                              int m_tiles, int n_tiles, int blocks)
+                                                              int m_tiles, int n_tiles, int blocks, int pf_dist)
 {
     typedef GemmCfg<CT, BS_LAST, DD, TM, TN, TK, WM, WN, ST> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -244,6 +245,40 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 
     const int steps = c / TK;
     KG_STAMP(0);
+    // L2 prefetch for the workgroup that will take this one's place: the input tile of logical
+    // id lid + pf_dist (same XCD, pf_dist = workgroups resident per XCD), this workgroup's
+    // share of its rows (the TM-tiles of one input tile split it).  One 4-byte load per
+    // 128-byte line, result unused.
+    // The loads are direct-to-LDS ones (no destination register to keep alive) into the last
+    // ring stage: they are older than the loads of slab 0, so they have landed when the first
+    // wait ends, before anything is requested into that stage.
+    constexpr int PF = C::PF;
+    if constexpr (BS_LAST) {
+        const int flid = lid + pf_dist;
+        if (pf_dist > 0 && flid < min(((int)blockIdx.x % 8 + 1) * per_xcd, blocks)) {
+            const int f_mt = flid % m_tiles, f_rest = flid / m_tiles;
+            const int f_nt = f_rest % n_tiles, f_g = f_rest / n_tiles;
+            const int f_a = f_g / d, f_d = f_g - f_a * d, f_n0 = f_nt * TN;
+            constexpr int LPR = TN * C::ES / 128;  // lines per row of the tile
+            const int rows_per = (c + m_tiles - 1) / m_tiles;
+            const int r_begin = f_mt * rows_per, r_end = min(c, r_begin + rows_per);
+            const CT *fx = x + ((size_t)f_a * c * d + f_d) * batch + f_n0;
+#pragma unroll
+            for (int i = 0; i < PF; ++i) {
+                const int q = tid + i * C::THREADS;
+                const int r = r_begin + q / LPR, col = (q % LPR) * (128 / C::ES);
+                if (r < r_end) {
+                    const CT *ptr = fx + (size_t)r * d * batch + min(col, batch - 4 / C::ES - f_n0);
+                    const uint32_t sink = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem +
+                                          (ST - 1) * C::STAGE_BYTES + wave * 256;
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                                 :
+                                 : "v"(ptr), "s"(sink)
+                                 : "memory", "m0");
+                }
+            }
+        }
+    }
 #pragma unroll
     for (int p = 0; p < ST - 1; ++p) issue(min(p, steps - 1), p);
     KG_STAMP(1);
@@ -492,6 +527,7 @@ const GemmInst gemm_insts[] = {
     GEMM_INST(1, half_t, true, 1, 64, 256, 32, 1, 4, 3),
     GEMM_INST(1, half_t, false, 1, 64, 256, 32, 1, 4, 3),
 };
+constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_FIRST_CHOICE = 19;  // entries the automatic choice (variant -1) looks at
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 
@@ -563,8 +599,18 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             return KSMM_ERR_LAUNCH;
     }
     int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
+    // L2 prefetch for the successor workgroup (bs_last): when the TM-tiles of an input tile can
+    // cover it with PF lines per thread; distance = workgroups resident on an XCD (32 CUs)
+    int pf_dist = 0;
+    if (p.bs_last && m_tiles >= 2) {
+        const int es = 16 / t.epc, resident = t.lds <= 80 * 1024 ? 64 : 32;  // workgroups per XCD
+        const int64_t lines = ((int64_t)p.c + m_tiles - 1) / m_tiles * (t.tn * es / 128);
+        // current and prefetched input tiles of an XCD must leave room in its 4 MB L2
+        const int64_t in_l2 = 2 * (int64_t)p.c * t.tn * es * ((resident + m_tiles - 1) / m_tiles);
+        if (lines <= (int64_t)GEMM_PF * t.threads && in_l2 <= (5 << 19)) pf_dist = resident;
+    }
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i};
+                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i, &pf_dist};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
