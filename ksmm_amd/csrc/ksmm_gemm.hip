@@ -90,11 +90,11 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
     static constexpr int N_WAIT = (ST - 2) * L;
     static constexpr int PF = 4;  // L2 prefetch loads per thread (128-byte lines of the successor's input tile)
     static_assert(!BS_LAST || DD == 1, "DD > 1 is a batch-size-first variant");
-    static_assert(ES == 2 || BS_LAST, "fp32 batch-size-first uses the plain tile kernel");
+    static_assert(ES == 2 || BS_LAST, "fp32 and e4m3 batch-size-first use other kernels");
     static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0 && TK % KSTEP == 0, "wave tiling");
     static_assert(W_CHUNKS % THREADS == 0 && X_CHUNKS % THREADS == 0, "every wave issues L loads per slab");
-    static_assert(ES == 2 ? (W_CPR == 8 || W_CPR % 16 == 0) : W_CPR % 16 == 0, "weight swizzle group");
-    static_assert(BS_LAST ? (ES == 2 ? (X_CPR == 8 || X_CPR % 16 == 0) : X_CPR % 16 == 0) : (X_CPR == 4 || X_CPR == 8 || X_CPR % 16 == 0), "input swizzle group");
+    static_assert(ES <= 2 ? (W_CPR == 8 || W_CPR % 16 == 0) : W_CPR % 16 == 0, "weight swizzle group");
+    static_assert(BS_LAST ? (ES <= 2 ? (X_CPR == 8 || X_CPR % 16 == 0) : X_CPR % 16 == 0) : (X_CPR == 4 || X_CPR == 8 || X_CPR % 16 == 0), "input swizzle group");
     static_assert(ST >= 2 && N_WAIT <= 63 && LDS_BYTES <= 160 * 1024, "ring");
     static_assert(DD * MT * NT * 16 <= 256, "accumulators");
 };
@@ -105,11 +105,14 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
 //  k-outer fp16 rows (CPR chunks of 16 bytes): the 32 lanes of a transpose load read 4 rows x
 //  64 bytes -> XOR the 64-byte group index with row & 3 (rows of 128 bytes alternate bank
 //  halves already: row / 2 & 1).
+//  k-outer e4m3 rows: the 32 lanes of a transpose load read 8 rows x 32 bytes -> XOR the
+//  32-byte group index with row & 7 (rows of 128 bytes: two rows per bank line, (row / 2) & 3).
 //  k-outer fp32: 2 rows x 128 bytes per ds_read_b32 wave -> XOR the 128-byte half with row & 1.
 //  k-inner rows: 16 lanes read one chunk of 16 consecutive rows -> XOR the chunk so that the
 //  rows sharing a 256-byte bank line differ (rows of 64, 128, >= 256 bytes).
 template <typename CT, int CPR> __device__ __forceinline__ int swz_outer(int row)
 {
+    if (sizeof(CT) == 1) return CPR >= 16 ? 2 * (row & 7) : 2 * ((row >> 1) & 3);
     return sizeof(CT) == 2 ? (CPR >= 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1)) : 8 * (row & 1);
 }
 template <int CPR> __device__ __forceinline__ int swz_inner(int row)
@@ -139,6 +142,24 @@ template <int COLS> struct outer_frag<half_t, COLS> {
         typedef short short8_t __attribute__((ext_vector_type(8)));
         short8_t r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return __builtin_bit_cast(half8_t, r);
+    }
+};
+template <int COLS> struct outer_frag<fp8_t, COLS> {
+    // ds_read_b64_tr_b8: 16 lanes address 8 rows x 16 bytes (lanes 2i, 2i+1: the two halves of
+    // row i) and lane j receives column j, i.e. 8 consecutive k of one index
+    __device__ static __forceinline__ uint32_t off(int idx0, int lane)
+    {
+        const int kq = lane >> 5, l16 = lane & 15, hs = (lane >> 4) & 1;
+        const int row = 8 * kq + (l16 >> 1);  // + k0 (a multiple of 16): same row & 7
+        const int chunk = (idx0 >> 4) + hs;
+        return (uint32_t)(row * COLS + ((chunk ^ swz_outer<fp8_t, COLS / 16>(row)) << 4) + 8 * (l16 & 1));
+    }
+    __device__ static __forceinline__ long read(uint32_t addr, int k0)
+    {
+        typedef int int2_t __attribute__((ext_vector_type(2)));
+        typedef int2_t __attribute__((address_space(3))) * lds_ptr;
+        const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr)(lds_bytes_t)(uintptr_t)(addr + k0 * COLS));
+        return __builtin_bit_cast(long, r);
     }
 };
 template <int COLS> struct outer_frag<float, COLS> {
@@ -418,12 +439,13 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     //   bs_first: out[n][(m..m+3) x d_i interleaved]   row = TM*DD elements
     // The tile is written in passes of as many rows as fit in the LDS of the ring.
     {
-        constexpr int RC = (BS_LAST ? TN : TM * DD) + C::EPC;  // padded row, elements
+        constexpr int OES = (int)sizeof(TY), OEPC = 16 / OES;  // output element, elements per 16 bytes
+        constexpr int RC = (BS_LAST ? TN : TM * DD) + OEPC;     // padded row, elements
         constexpr int LR = BS_LAST ? TM : TN;                   // rows of the whole tile
-        constexpr int RPP_RAW = C::LDS_BYTES / (RC * C::ES) / 32 * 32;
+        constexpr int RPP_RAW = C::LDS_BYTES / (RC * OES) / 32 * 32;
         constexpr int RPP = RPP_RAW > LR ? LR : RPP_RAW;        // rows per pass (multiple of 32)
         constexpr int PASSES = (LR + RPP - 1) / RPP;
-        constexpr int CPR = (RC - C::EPC) / C::EPC;             // 16-byte chunks per row
+        constexpr int CPR = (RC - OEPC) / OEPC;                 // 16-byte chunks per row
         static_assert(RPP >= 32, "output pass");
         TY *const out = (TY *)smem;
         const int l32 = lane & 31, lq = lane >> 5;
@@ -462,7 +484,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
                 }
             __syncthreads();
             for (int q = tid; q < RPP * CPR; q += C::THREADS) {
-                const int r = q / CPR, cc = (q % CPR) * C::EPC;
+                const int r = q / CPR, cc = (q % CPR) * OEPC;
                 const int row = pass * RPP + r;  // row of the tile
                 if (row >= LR) break;
                 const uint4_t v = *(const uint4_t *)(out + r * RC + cc);
@@ -488,11 +510,13 @@ struct GemmInst {
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
 // so that one multiplies while the other stores its output tile)
-#define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
+#define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
     {COMBO_, BL_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES,                                 \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::EPC,                                       \
-     (const void *)ks_gemm_kernel<CT_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_>}
+     (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_>}
+#define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
+    GEMM_INST_T(COMBO_, CT_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)
 #define GEMM_INST(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_)                                \
     GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, 1)
 // The first instance that fits (and still yields >= 256 workgroups) is the default; the order
@@ -526,9 +550,14 @@ const GemmInst gemm_insts[] = {
     // fp16, b a multiple of 64 only: last resort (variant -2), after the stream and k-loop tiles
     GEMM_INST(1, half_t, true, 1, 64, 256, 32, 1, 4, 3),
     GEMM_INST(1, half_t, false, 1, 64, 256, 32, 1, 4, 3),
+    // e4m3 x e4m3 -> fp16, bs_last: the bytes go to LDS as they are and into the fp8 MFMA
+    GEMM_INST_T(2, fp8_t, half_t, true, 1, 128, 256, 64, 2, 2, 3, 2),
+    GEMM_INST_T(2, fp8_t, half_t, true, 1, 256, 256, 64, 2, 4, 4, 1),
+    GEMM_INST_T(2, fp8_t, half_t, true, 1, 128, 128, 64, 2, 2, 4, 2),
+    GEMM_INST_T(2, fp8_t, half_t, true, 1, 128, 256, 32, 2, 2, 4, 2),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
-constexpr int N_GEMM_FIRST_CHOICE = 19;  // entries the automatic choice (variant -1) looks at
+constexpr int GEMM_LAST_RESORT_BEGIN = 19, GEMM_LAST_RESORT_END = 21;  // skipped by variant -1
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 
 bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
@@ -562,7 +591,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int pick = -1;
     for (int i = 0; i < N_GEMM_INSTS; ++i) {
         if (variant >= 0 && variant != i) continue;
-        if (variant == -1 && i >= N_GEMM_FIRST_CHOICE) break;
+        if (variant == -1 && i >= GEMM_LAST_RESORT_BEGIN && i < GEMM_LAST_RESORT_END) continue;
         const GemmInst &t = gemm_insts[i];
         if (!gemm_fits(t, p, combo)) continue;
         if (variant == -1) {

@@ -14,6 +14,9 @@ template <> struct compute<float> {
 template <> struct compute<half_t> {
     static constexpr int KSTEP = 16;
 };
+template <> struct compute<fp8_t> {  // e4m3 operands straight into the fp8 MFMA
+    static constexpr int KSTEP = 16;
+};
 
 // 16 bytes of global memory -> EPV elements of CT, written to LDS contiguously;
 // register-staged variant: load now, write to LDS later
@@ -88,6 +91,14 @@ template <> struct frag<half_t> {
     __device__ static __forceinline__ float16_t mfma(half8_t a, half8_t b, float16_t c)
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <> struct frag<fp8_t> {
+    typedef long type;  // 8 e4m3 values: k = 8 * (lane / 32) .. + 7 of row / column lane % 32
+    __device__ static __forceinline__ float16_t mfma(long a, long b, float16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
     }
 };
 

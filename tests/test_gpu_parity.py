@@ -102,6 +102,14 @@ def test_gemm_kernels_forced():
     assert ran >= 12
 
 
+def test_gemm_kernels_forced_e4m3():
+    """The e4m3 instances of the GEMM sub-family (bytes straight into the fp8 MFMA): batch tails,
+    several blocks, d > 1, c = 1, 2 and 3 slabs."""
+    cases = [("fp8", True, (2, 256, 64, 3), 1008), ("fp8", True, (1, 128, 128, 2), 272),
+             ("fp8", True, (2, 256, 192, 1), 528), ("fp8", True, (1, 256, 96, 2), 1024)]
+    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 32)], 3, 10)
+
+
 def _forced_sweep(cases, variants, algo, min_ran):
     """Every (case, variant) the family accepts must agree with the oracle; the others must be
     refused with KSMM_ERR_BAD_ALGO."""
