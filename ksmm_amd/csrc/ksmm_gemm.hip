@@ -175,7 +175,7 @@ template <int COLS> struct outer_frag<float, COLS> {
     }
 };
 
-template <typename CT, typename TY, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC>
+template <typename CT, typename TY, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool KT>
 __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__restrict__ x,
                                                               const CT *__restrict__ w,
                                                               TY *__restrict__ y, int batch, int a,
@@ -204,7 +204,15 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     const char *const wbase = (const char *)(w + ((size_t)(DD == 1 ? g : a_i * DD) * c) * b + m0);
     const char *const xbase = BS_LAST ? (const char *)(x + ((size_t)a_i * c * d + d_i) * batch + n0)
                                       : (const char *)(x + (size_t)n0 * in_size + (size_t)a_i * c * DD);
+    // KT (bs_last): c need not be a multiple of TK.  The last slab then has rem < TK rows of its
+    // own: the loads of the rows behind them are pointed at row rem-1 (valid memory, finite
+    // whenever the data are), and the weight rows behind rem are cleared in LDS once they have
+    // landed, so that they add nothing.
+    static_assert(!KT || (BS_LAST && DD == 1), "K tails: batch-size-last only");
+    const int steps = KT ? (c + TK - 1) / TK : c / TK;
+    const int rem = KT ? c - (steps - 1) * TK : TK;  // rows of the last slab
     uint32_t wvoff[C::LW], xvoff[C::LX];
+    uint32_t wvoff_t[KT ? C::LW : 1], xvoff_t[KT ? C::LX : 1];  // the same for the last slab
 #pragma unroll
     for (int i = 0; i < C::LW; ++i) {
         const int q = tid + i * C::THREADS;
@@ -212,6 +220,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
         const int row = r / C::W_CPR, pc = r % C::W_CPR;
         const int col = (pc ^ swz_outer<CT, C::W_CPR>(row)) * C::EPC;
         wvoff[i] = (uint32_t)((((size_t)dd * c + row) * b + col) * C::ES);
+        if constexpr (KT) wvoff_t[i] = (uint32_t)(((size_t)min(row, rem - 1) * b + col) * C::ES);
     }
 #pragma unroll
     for (int i = 0; i < C::LX; ++i) {
@@ -220,6 +229,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
         if (BS_LAST) {
             const int col = (pc ^ swz_outer<CT, C::X_CPR>(row)) * C::EPC;
             xvoff[i] = (uint32_t)(((size_t)row * d * batch + min(col, batch - C::EPC - n0)) * C::ES);
+            if constexpr (KT)
+                xvoff_t[i] = (uint32_t)(((size_t)min(row, rem - 1) * d * batch + min(col, batch - C::EPC - n0)) * C::ES);
         } else {
             const int col = (pc ^ swz_inner<C::X_CPR>(row)) * C::EPC;
             xvoff[i] = (uint32_t)(((size_t)min(row, batch - 1 - n0) * in_size + col) * C::ES);
@@ -230,11 +241,26 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     auto issue = [&](int step, int stg) {
         const uint32_t dst = lds_base + stg * C::STAGE_BYTES + wave * 1024;
+        const bool tail = KT && step == steps - 1;
 #pragma unroll
-        for (int i = 0; i < C::LW; ++i) dma16s(wbase + step * w_step, wvoff[i], dst + i * (C::THREADS * 16));
+        for (int i = 0; i < C::LW; ++i)
+            dma16s(wbase + step * w_step, tail ? wvoff_t[KT ? i : 0] : wvoff[i], dst + i * (C::THREADS * 16));
 #pragma unroll
         for (int i = 0; i < C::LX; ++i)
-            dma16s(xbase + step * x_step, xvoff[i], dst + C::W_BYTES + i * (C::THREADS * 16));
+            dma16s(xbase + step * x_step, tail ? xvoff_t[KT ? i : 0] : xvoff[i], dst + C::W_BYTES + i * (C::THREADS * 16));
+    };
+    // clear this thread's chunks of the weight rows behind rem in stage stg (its own loads have
+    // landed; the barrier that follows publishes the zeros with the rest)
+    auto clear_tail = [&](int stg) {
+#pragma unroll
+        for (int i = 0; i < C::LW; ++i) {
+            const int q = tid + i * C::THREADS;
+            const int row = (q % (TK * C::W_CPR)) / C::W_CPR;
+            if (row >= rem) {
+                typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
+                *(lds_ptr)(lds_bytes_t)(uintptr_t)(lds_base + stg * C::STAGE_BYTES + q * 16) = uint4_t{0, 0, 0, 0};
+            }
+        }
     };
 
     // ---- per-lane byte offsets of the MFMA operands inside a stage (sub-step 0) --------------
@@ -264,7 +290,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = 0.f;
 
-    const int steps = c / TK;
     KG_STAMP(0);
     // L2 prefetch for the workgroup that will take this one's place: the input tile of logical
     // id lid + pf_dist (same XCD, pf_dist = workgroups resident per XCD), this workgroup's
@@ -373,6 +398,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
         }
     };
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
+    if (KT && steps == 1 && rem < TK) clear_tail(0);
     __syncthreads();  // slab 0 landed for every wave
     stage_addrs(0);
     load_frags(wa, xa, 0, fw[0], fx[0]);
@@ -382,11 +408,13 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
         const char *const wsrc = wbase + (size_t)nstep * w_step;
         const char *const xsrc = xbase + (size_t)nstep * x_step;
         const uint32_t dst = lds_base + ((it + ST - 1) % ST) * C::STAGE_BYTES + wave * 1024;
+        const bool tail = KT && nstep == steps - 1;
         auto issue_one = [&](int q) {
             if (q < C::LW)
-                dma16s(wsrc, wvoff[q < C::LW ? q : 0], dst + q * (C::THREADS * 16));
+                dma16s(wsrc, tail ? wvoff_t[KT && q < C::LW ? q : 0] : wvoff[q < C::LW ? q : 0], dst + q * (C::THREADS * 16));
             else
-                dma16s(xsrc, xvoff[q >= C::LW ? q - C::LW : 0], dst + C::W_BYTES + (q - C::LW) * (C::THREADS * 16));
+                dma16s(xsrc, tail ? xvoff_t[KT && q >= C::LW ? q - C::LW : 0] : xvoff[q >= C::LW ? q - C::LW : 0],
+                       dst + C::W_BYTES + (q - C::LW) * (C::THREADS * 16));
         };
 #pragma unroll
         for (int kk = 0; kk < K0; ++kk) {
@@ -395,6 +423,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
             } else {
                 KG_STAMP(4 + 4 * it);
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
+                if (KT && it + 2 == steps && rem < TK) clear_tail((it + 1) % ST);
                 __syncthreads();  // slab it+1 landed for every wave, and everyone left slab it
                 KG_STAMP(5 + 4 * it);
                 if (it + 1 < steps) {
@@ -506,15 +535,18 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 
 struct GemmInst {
     int combo, bs_last, dd, tm, tn, tk, threads, lds, epc;
+    int ktail;  // takes c that is not a multiple of tk
     const void *fn;
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
 // so that one multiplies while the other stores its output tile)
-#define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
+#define GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_)              \
     {COMBO_, BL_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES,                                 \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::EPC,                                       \
-     (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_>}
+     KT_, (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_>}
+#define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
+    GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
     GEMM_INST_T(COMBO_, CT_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)
 #define GEMM_INST(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_)                                \
@@ -555,6 +587,12 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_T(2, fp8_t, half_t, true, 1, 256, 256, 64, 2, 4, 4, 1),
     GEMM_INST_T(2, fp8_t, half_t, true, 1, 128, 128, 64, 2, 2, 4, 2),
     GEMM_INST_T(2, fp8_t, half_t, true, 1, 128, 256, 32, 2, 2, 4, 2),
+    // bs_last, any c (partial last slab)
+    GEMM_INST_K(1, half_t, half_t, true, 1, 128, 256, 32, 2, 2, 3, 2, true),
+    GEMM_INST_K(1, half_t, half_t, true, 1, 64, 256, 32, 1, 4, 3, 1, true),
+    GEMM_INST_K(0, float, float, true, 1, 128, 128, 16, 2, 2, 4, 1, true),
+    GEMM_INST_K(0, float, float, true, 1, 64, 256, 16, 1, 4, 4, 1, true),
+    GEMM_INST_K(2, fp8_t, half_t, true, 1, 128, 256, 32, 2, 2, 4, 2, true),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int GEMM_LAST_RESORT_BEGIN = 19, GEMM_LAST_RESORT_END = 21;  // skipped by variant -1
@@ -563,7 +601,7 @@ constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
 {
     if (t.combo != combo || t.bs_last != p.bs_last) return false;
-    if (p.b % t.tm || p.c % t.tk) return false;
+    if (p.b % t.tm || (p.c % t.tk && !t.ktail)) return false;
     if (p.b % t.epc) return false;  // 16-byte weight vectors
     if (p.bs_last) {
         if (p.batch % t.epc || p.batch < t.epc) return false;

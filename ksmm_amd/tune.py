@@ -64,7 +64,7 @@ def candidates():
         out.append((2, 1000 + inst))
     for inst in range(28):                       # stream
         out.append((3, (2 << 24) | inst))
-    for inst in range(24):                       # direct-to-LDS GEMM
+    for inst in range(40):                       # direct-to-LDS GEMM
         out.append((3, (4 << 24) | inst))
     for inst in range(64):                       # weight-stationary
         out.append((3, (1 << 24) | inst))

@@ -80,7 +80,10 @@ def test_gemm_kernels_forced():
     from ksmm_amd import Kernel, generate_factor, _lib
 
     cases = [("fp16", True, (2, 256, 64, 3)), ("fp16", False, (2, 256, 64, 1)), ("fp16", False, (2, 256, 64, 2)),
-             ("fp16", False, (1, 128, 128, 2)), ("fp32", True, (1, 256, 64, 2)), ("fp32", True, (2, 128, 32, 1))]
+             ("fp16", False, (1, 128, 128, 2)), ("fp32", True, (1, 256, 64, 2)), ("fp32", True, (2, 128, 32, 1)),
+             # c not a multiple of the K tile (partial last slab), c below one K tile
+             ("fp16", True, (2, 128, 70, 2)), ("fp16", True, (1, 64, 50, 3)), ("fp16", True, (1, 128, 18, 1)),
+             ("fp32", True, (1, 128, 50, 2)), ("fp32", True, (2, 64, 18, 1)), ("fp32", True, (1, 64, 7, 2))]
     ran = 0
     for prec, bs_last, pattern in cases:
         a, b, c, d = pattern
@@ -99,15 +102,16 @@ def test_gemm_kernels_forced():
                 ran += 1
                 err = O.rel_fro_error(y.float().cpu().numpy(), z)
                 assert err <= TOL[prec], (prec, bs_last, pattern, batch, inst, err)
-    assert ran >= 12
+    assert ran >= 24
 
 
 def test_gemm_kernels_forced_e4m3():
     """The e4m3 instances of the GEMM sub-family (bytes straight into the fp8 MFMA): batch tails,
     several blocks, d > 1, c = 1, 2 and 3 slabs."""
     cases = [("fp8", True, (2, 256, 64, 3), 1008), ("fp8", True, (1, 128, 128, 2), 272),
-             ("fp8", True, (2, 256, 192, 1), 528), ("fp8", True, (1, 256, 96, 2), 1024)]
-    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 32)], 3, 10)
+             ("fp8", True, (2, 256, 192, 1), 528), ("fp8", True, (1, 256, 96, 2), 1024),
+             ("fp8", True, (1, 128, 70, 2), 1008), ("fp8", True, (2, 256, 40, 1), 272), ("fp8", True, (1, 128, 9, 1), 64)]
+    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 32)], 3, 13)
 
 
 def _forced_sweep(cases, variants, algo, min_ran):
