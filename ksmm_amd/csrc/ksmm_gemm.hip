@@ -93,7 +93,7 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
     static_assert(ES == 2 || BS_LAST, "fp32 and e4m3 batch-size-first use other kernels");
     static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0 && TK % KSTEP == 0, "wave tiling");
     static_assert(W_CHUNKS % THREADS == 0 && X_CHUNKS % THREADS == 0, "every wave issues L loads per slab");
-    static_assert(ES <= 2 ? (W_CPR == 8 || W_CPR % 16 == 0) : W_CPR % 16 == 0, "weight swizzle group");
+    static_assert(ES <= 2 ? (W_CPR == 8 || W_CPR % 16 == 0 || (ES == 1 && W_CPR == 4)) : W_CPR % 16 == 0, "weight swizzle group");
     static_assert(BS_LAST ? (ES <= 2 ? (X_CPR == 8 || X_CPR % 16 == 0) : X_CPR % 16 == 0) : (X_CPR == 4 || X_CPR == 8 || X_CPR % 16 == 0), "input swizzle group");
     static_assert(ST >= 2 && N_WAIT <= 63 && LDS_BYTES <= 160 * 1024, "ring");
     static_assert(DD * MT * NT * 16 <= 256, "accumulators");
@@ -106,13 +106,14 @@ template <typename CT, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int
 //  64 bytes -> XOR the 64-byte group index with row & 3 (rows of 128 bytes alternate bank
 //  halves already: row / 2 & 1).
 //  k-outer e4m3 rows: the 32 lanes of a transpose load read 8 rows x 32 bytes -> XOR the
-//  32-byte group index with row & 7 (rows of 128 bytes: two rows per bank line, (row / 2) & 3).
+//  32-byte group index with row & 7 (rows of 128 bytes: two rows per bank line, (row / 2) & 3;
+//  rows of 64 bytes: four per bank line, (row / 4) & 1).
 //  k-outer fp32: 2 rows x 128 bytes per ds_read_b32 wave -> XOR the 128-byte half with row & 1.
 //  k-inner rows: 16 lanes read one chunk of 16 consecutive rows -> XOR the chunk so that the
 //  rows sharing a 256-byte bank line differ (rows of 64, 128, >= 256 bytes).
 template <typename CT, int CPR> __device__ __forceinline__ int swz_outer(int row)
 {
-    if (sizeof(CT) == 1) return CPR >= 16 ? 2 * (row & 7) : 2 * ((row >> 1) & 3);
+    if (sizeof(CT) == 1) return CPR >= 16 ? 2 * (row & 7) : CPR == 8 ? 2 * ((row >> 1) & 3) : 2 * ((row >> 2) & 1);
     return sizeof(CT) == 2 ? (CPR >= 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1)) : 8 * (row & 1);
 }
 template <int CPR> __device__ __forceinline__ int swz_inner(int row)
@@ -593,6 +594,9 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_K(0, float, float, true, 1, 128, 128, 16, 2, 2, 4, 1, true),
     GEMM_INST_K(0, float, float, true, 1, 64, 256, 16, 1, 4, 4, 1, true),
     GEMM_INST_K(2, fp8_t, half_t, true, 1, 128, 256, 32, 2, 2, 4, 2, true),
+    // e4m3, b a multiple of 64 only
+    GEMM_INST_T(2, fp8_t, half_t, true, 1, 64, 256, 64, 1, 4, 3, 2),
+    GEMM_INST_K(2, fp8_t, half_t, true, 1, 64, 256, 64, 1, 4, 3, 2, true),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int GEMM_LAST_RESORT_BEGIN = 19, GEMM_LAST_RESORT_END = 21;  // skipped by variant -1

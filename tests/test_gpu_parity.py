@@ -110,8 +110,9 @@ def test_gemm_kernels_forced_e4m3():
     several blocks, d > 1, c = 1, 2 and 3 slabs."""
     cases = [("fp8", True, (2, 256, 64, 3), 1008), ("fp8", True, (1, 128, 128, 2), 272),
              ("fp8", True, (2, 256, 192, 1), 528), ("fp8", True, (1, 256, 96, 2), 1024),
-             ("fp8", True, (1, 128, 70, 2), 1008), ("fp8", True, (2, 256, 40, 1), 272), ("fp8", True, (1, 128, 9, 1), 64)]
-    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 32)], 3, 13)
+             ("fp8", True, (1, 128, 70, 2), 1008), ("fp8", True, (2, 256, 40, 1), 272), ("fp8", True, (1, 128, 9, 1), 64),
+             ("fp8", True, (1, 192, 128, 2), 528), ("fp8", True, (2, 64, 72, 1), 1008)]
+    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 36)], 3, 18)
 
 
 def _forced_sweep(cases, variants, algo, min_ran):
