@@ -599,7 +599,6 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_K(2, fp8_t, half_t, true, 1, 64, 256, 64, 1, 4, 3, 2, true),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
-constexpr int GEMM_LAST_RESORT_BEGIN = 19, GEMM_LAST_RESORT_END = 21;  // skipped by variant -1
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 
 bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
@@ -633,8 +632,11 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int pick = -1;
     for (int i = 0; i < N_GEMM_INSTS; ++i) {
         if (variant >= 0 && variant != i) continue;
-        if (variant == -1 && i >= GEMM_LAST_RESORT_BEGIN && i < GEMM_LAST_RESORT_END) continue;
         const GemmInst &t = gemm_insts[i];
+        // TM = 64 tiles are a first choice only where nothing better exists: e4m3 (no stream
+        // kernels, slow k-loop tiles) and partial K slabs; otherwise the stream,
+        // weight-stationary and k-loop tiles come first and variant -2 comes back here
+        if (variant == -1 && t.tm < 128 && t.combo != 2 && !(t.ktail && p.c % t.tk)) continue;
         if (!gemm_fits(t, p, combo)) continue;
         if (variant == -1) {
             // the big tiles only pay when they still fill the chip

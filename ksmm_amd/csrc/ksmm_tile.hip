@@ -499,6 +499,11 @@ const TileInst tile_insts[] = {
     TILE_SET_H(2, fp8_t, fp8_t, false),
     TILE_SET_H(3, half_t, fp8_t, true),
     TILE_SET_H(3, half_t, fp8_t, false),
+    // b = 96 blocks, bs_last (appended: the indices above are referenced by the measured table)
+    TILE_INST(1, half_t, half_t, half_t, half_t, true, 96, 128, 32, 1, 4),
+    TILE_INST(1, half_t, half_t, half_t, half_t, true, 96, 256, 32, 1, 4),
+    TILE_INST(2, half_t, fp8_t, fp8_t, half_t, true, 96, 128, 32, 1, 4),
+    TILE_INST(2, half_t, fp8_t, fp8_t, half_t, true, 96, 256, 32, 1, 4),
 };
 constexpr int N_TILE_INSTS = sizeof(tile_insts) / sizeof(TileInst);
 

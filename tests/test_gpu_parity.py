@@ -183,8 +183,9 @@ def test_tile_subfamilies_forced():
     _forced_sweep(cases, [(2 << 24) | i for i in range(28)], 3, 24)                      # stream
     kcases = [("fp16", True, (2, 128, 64, 2), 520), ("fp16", False, (2, 128, 64, 1), 520),
               ("fp32", True, (1, 128, 64, 3), 520), ("fp32", False, (2, 64, 32, 1), 520),
-              ("fp8", True, (2, 128, 64, 2), 528), ("hq", False, (1, 256, 128, 1), 520)]
-    _forced_sweep(kcases, [(0 << 24) | i for i in range(56)], 3, 20)                     # k-loop
+              ("fp8", True, (2, 128, 64, 2), 528), ("hq", False, (1, 256, 128, 1), 520),
+              ("fp16", True, (2, 96, 64, 2), 520), ("fp8", True, (1, 96, 96, 3), 528), ("fp32", True, (1, 96, 48, 2), 520)]
+    _forced_sweep(kcases, [(0 << 24) | i for i in range(64)], 3, 26)                     # k-loop
     wcases = [("fp32", True, (2, 64, 64, 2), 520), ("fp32", False, (2, 96, 96, 1), 520),
               ("fp16", True, (2, 64, 64, 2), 520), ("fp16", False, (3, 64, 64, 1), 520),
               ("fp8", True, (2, 64, 64, 1), 528), ("hq", False, (2, 96, 96, 1), 520)]
