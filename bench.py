@@ -2,6 +2,7 @@
 """Benchmark of the KS hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--all 0|1]
+    python bench.py --factor fp16:last:1,768,192,16     (one factor only: per-kernel profiling runs)
 
 A step is one forward pass of one KS factor over a batch of 25 088 columns.  The headline
 workload is BASELINE configuration 2: a single fp32 factor with pattern (1,48,48,16)
@@ -249,6 +250,9 @@ def main():
     ap.add_argument("--cpu", type=int, default=1, help="time the CPU baseline")
     ap.add_argument("--copy-calib", type=int, default=0,
                     help="also run N plain device copies of 77 MB (counter calibration for profiling runs)")
+    ap.add_argument("--factor", default=None,
+                    help="time one factor only, e.g. fp16:last:1,768,192,16 (per-kernel profiling runs); "
+                         "prints that configuration's JSON instead of the headline line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU (the KS path shards on the batch axis without "
@@ -270,6 +274,12 @@ def main():
         for _ in range(args.copy_calib):
             torch.add(src, 1.0, out=dst)  # one elementwise kernel per call: 1 read + 1 write stream
         torch.cuda.synchronize()
+    if args.factor:
+        prec, layout, pat = args.factor.split(":")
+        pattern = tuple(int(v) for v in pat.split(","))
+        res = bench_config("factor", [pattern], prec, layout == "last", None, args.steps, args.warmup)
+        print(json.dumps(res))
+        return
     head = bench_config(*CONFIGS[0], steps=args.steps, warmup=args.warmup)
     sec = head["factors"][0]["us"] / 1e6
     roof = factor_roofline(BATCH, CONFIGS[0][1][0], torch.float32, torch.float32, torch.float32, sec)
