@@ -1,13 +1,14 @@
 // "Row" kernel: batch-size-first layout, d > 1, small b x c blocks, fp32.
 //
 // In this layout a batch row holds, for one a_i, the c*d inputs of all d blocks interleaved
-// (d_i fastest).  A workgroup owns one a_i and every wgs-th tile of batch rows; it has one wavefront per
-// d_i, and each wavefront keeps the b x c weight block of its d_i in registers as MFMA
-// operands (v_mfma_f32_16x16x4_f32, fp32 accumulation).  Whole row segments (c*d contiguous
-// floats) are copied to LDS with 16-byte loads, every wave picks the inputs of its own d_i
-// out of LDS (stride d), the d result blocks are interleaved again in an LDS output tile, and
-// the b*d outputs of each row are written back as one contiguous run.  HBM sees only full,
-// coalesced rows; the stride-d gather the layout forces happens in LDS.
+// (d_i fastest).  A workgroup owns one a_i, a group of DD consecutive d_i (all of them when
+// d == DD) and every wgs-th tile of batch rows; it has one wavefront per d_i of its group, and
+// each wavefront keeps the b x c weight block of its d_i in registers as MFMA operands
+// (v_mfma_f32_16x16x4_f32, fp32 accumulation).  Row segments (c runs of DD contiguous floats,
+// one run of c*d floats when d == DD) are copied to LDS with 16-byte loads, every wave picks
+// the inputs of its own d_i out of LDS (stride DD), the DD result blocks are interleaved again
+// in an LDS output tile, and the outputs of each row are written back as b runs of DD floats.
+// HBM sees coalesced runs only; the stride-d gather the layout forces happens in LDS.
 //
 // The loads of the next two tiles are in flight (in registers) while a tile is multiplied and
 // stored; tiles are dealt round-robin to the workgroups of an a_i, so that at any time they
@@ -41,32 +42,37 @@ template <int BB, int CC, int DD, int TN, bool NT_STORE>
 __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a,
-                                                            float scale, int wgs_per_a, int n_tiles)
+                                                            int d, float scale, int wgs_per_a, int n_tiles)
 {
     typedef RowCfg<BB, CC, DD, TN> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *const xs = (float *)smem;                // [2][TN][LDX]
     float *const os = xs + 2 * TN * C::LDX;         // [TN][LDO]
-    const int a_i = blockIdx.x / wgs_per_a;
-    const int s = blockIdx.x - a_i * wgs_per_a;
+    // blockIdx -> (a_i, group of DD d_i, share of the tiles)
+    const int groups = d / DD;
+    const int ag = blockIdx.x / wgs_per_a;
+    const int s = blockIdx.x - ag * wgs_per_a;
+    const int a_i = ag / groups, d0 = (ag - a_i * groups) * DD;
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
     const int dd = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's d_i
-    const size_t in_size = (size_t)a * C::XROW, out_size = (size_t)a * C::OROW;
+    const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
 
     // weights of block (a_i, dd): element (k, m) at ((a_i*d + dd)*c + k)*b + m -> A operands
     float wreg[C::MT][C::KS];
     {
-        const float *wg = w + (size_t)(a_i * DD + dd) * CC * BB;
+        const float *wg = w + (size_t)(a_i * d + d0 + dd) * CC * BB;
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
             for (int mt = 0; mt < C::MT; ++mt) wreg[mt][ks] = wg[(4 * ks + q) * BB + 16 * mt + r];
     }
 
-    const float *xg = x + (size_t)a_i * C::XROW;
-    float *yg = y + (size_t)a_i * C::OROW;
+    // element e of a tile row (e = k * DD + j) lives at k * d + j behind the group's origin
+    const float *xg = x + (size_t)a_i * CC * d + d0;
+    float *yg = y + (size_t)a_i * BB * d + d0;
+    auto row_off = [&](int e0) { return (e0 / DD) * d + e0 % DD; };
     float4_t xreg[2][C::X_PER_T];
     auto gload = [&](int t, auto P) {
 #pragma unroll
@@ -75,7 +81,7 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
             if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
                 const int nn = v / (C::XROW / 4), e0 = (v % (C::XROW / 4)) * 4;
                 const int row = min(t * TN + nn, batch - 1);
-                xreg[decltype(P)::value][i] = *(const float4_t *)(xg + (size_t)row * in_size + e0);
+                xreg[decltype(P)::value][i] = *(const float4_t *)(xg + (size_t)row * in_size + row_off(e0));
             }
         }
     };
@@ -132,9 +138,9 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
                 if (row < batch) {
                     const float4_t o = *(const float4_t *)(os + nn * C::LDO + e0);
                     if (NT_STORE)
-                        __builtin_nontemporal_store(o, (float4_t *)(yg + (size_t)row * out_size + e0));
+                        __builtin_nontemporal_store(o, (float4_t *)(yg + (size_t)row * out_size + row_off(e0)));
                     else
-                        *(float4_t *)(yg + (size_t)row * out_size + e0) = o;
+                        *(float4_t *)(yg + (size_t)row * out_size + row_off(e0)) = o;
                 }
             }
         }
@@ -162,6 +168,13 @@ const RowInst row_insts[] = {
     ROW_INST(48, 48, 16, 16, true), ROW_INST(48, 48, 8, 32, true), ROW_INST(48, 48, 4, 64, true),
     ROW_INST(64, 64, 8, 16, true),  ROW_INST(64, 64, 4, 32, true), ROW_INST(16, 16, 16, 32, true),
     ROW_INST(16, 16, 4, 128, true), ROW_INST(32, 32, 8, 32, true), ROW_INST(48, 48, 16, 16, false),
+    // more group sizes (d = DD, or a multiple of DD when DD is a multiple of 4) and block shapes
+    ROW_INST(48, 48, 12, 16, true), ROW_INST(48, 48, 6, 32, true),  ROW_INST(48, 48, 3, 64, true),
+    ROW_INST(48, 48, 2, 64, true),  ROW_INST(64, 64, 12, 16, true), ROW_INST(64, 64, 6, 16, true),
+    ROW_INST(64, 64, 3, 32, true),  ROW_INST(64, 64, 2, 64, true),  ROW_INST(96, 96, 4, 16, true),
+    ROW_INST(96, 96, 3, 32, true),   ROW_INST(48, 192, 4, 16, true),
+    ROW_INST(48, 192, 3, 16, true), ROW_INST(48, 192, 2, 16, true), ROW_INST(192, 48, 4, 16, true),
+    ROW_INST(192, 48, 3, 32, true), ROW_INST(32, 32, 16, 16, true),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 
@@ -176,17 +189,28 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int pick = -1;
     for (int i = 0; i < N_ROW_INSTS; ++i) {
         if (want != 0x7f && want != i) continue;
-        if (row_insts[i].bb == p.b && row_insts[i].cc == p.c && row_insts[i].dd == p.d) {
+        const RowInst &t = row_insts[i];
+        if (t.bb != p.b || t.cc != p.c) continue;
+        // all d blocks in one workgroup, or groups of dd whose runs keep the 16-byte alignment
+        if (t.dd == p.d || want != 0x7f) {
+            if (t.dd == p.d || (t.dd % 4 == 0 && p.d % t.dd == 0)) pick = i;
+            if (pick == i) break;
+        } else if (t.dd % 4 == 0 && p.d % t.dd == 0 && (t.dd >= 8 || p.b <= p.c) &&
+                   (pick < 0 || t.dd > row_insts[pick].dd)) {
+            // the largest group that divides d, unless an exact match follows; 16-byte output
+            // runs (groups of 4) only where the output is not the larger side
             pick = i;
-            break;
         }
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
     const RowInst &t = row_insts[pick];
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
-    if (wgs <= 0) wgs = (256 + p.a - 1) / p.a;
+    const int64_t ag = (int64_t)p.a * (p.d / t.dd);  // (a_i, group) pairs
+    // one round of workgroups, 8 or more waves per CU
+    const int per_cu_lds = 160 * 1024 / t.lds, per_cu_waves = 16 / t.dd > 0 ? 16 / t.dd : 1;
+    if (wgs <= 0) wgs = (256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves) + ag - 1) / ag;
     if (wgs > n_tiles) wgs = n_tiles;
-    const int64_t grid = (int64_t)p.a * wgs;
+    const int64_t grid = ag * wgs;
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_WAVE;
@@ -205,8 +229,8 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             return KSMM_ERR_LAUNCH;
     }
     int batch_i = (int)p.batch, wgs_i = (int)wgs, n_tiles_i = (int)n_tiles;
-    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.scale,
-                    &wgs_i, &n_tiles_i};
+    void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
+                    (void *)&p.scale, &wgs_i, &n_tiles_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(64 * t.dd), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

@@ -166,9 +166,15 @@ def test_wave_instances_forced():
 def test_row_kernel_instances_forced():
     """Every instance of the batch-size-first row kernel, full and ragged batch tiles."""
     shapes = [(2, 48, 48, 16), (1, 48, 48, 8), (2, 48, 48, 4), (1, 64, 64, 8), (2, 64, 64, 4), (1, 16, 16, 16),
-              (3, 16, 16, 4), (2, 32, 32, 8)]
+              (3, 16, 16, 4), (2, 32, 32, 8),
+              # all d blocks of an a_i in one workgroup, other group sizes and block shapes
+              (1, 48, 48, 12), (2, 48, 48, 6), (1, 48, 48, 3), (2, 48, 48, 2), (1, 64, 64, 12), (1, 64, 64, 6),
+              (2, 64, 64, 3), (1, 64, 64, 2), (1, 96, 96, 4), (2, 96, 96, 3), (1, 48, 192, 4), (1, 48, 192, 3),
+              (2, 48, 192, 2), (1, 192, 48, 4), (1, 192, 48, 3), (1, 32, 32, 16),
+              # d a multiple of the group: several workgroups per a_i, runs of DD floats
+              (1, 48, 48, 32), (2, 48, 48, 24), (1, 64, 64, 16), (1, 16, 16, 64), (2, 96, 96, 8), (1, 192, 48, 16)]
     cases = [("fp32", False, p, batch) for p in shapes for batch in (512, 203)]
-    _forced_sweep(cases, [1000 + i for i in range(12)], 2, 16)
+    _forced_sweep(cases, [1000 + i for i in range(32)], 2, 70)
 
 
 def test_tile_subfamilies_forced():
