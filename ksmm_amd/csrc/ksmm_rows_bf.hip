@@ -158,12 +158,159 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
     }
 }
 
+// ---- the same for 16-bit and 8-bit inputs --------------------------------------------------
+// fp16 or e4m3 inputs and weights, fp16 MFMA (v_mfma_f32_16x16x16_f16, e4m3 decoded exactly
+// when an operand is picked out of LDS or loaded as a weight), fp32 accumulation, fp16
+// output.  Row segments travel as 16-byte vectors (8 halves / 16 e4m3), so c * DD and b * DD
+// must be multiples of the vector (and DD itself when d > DD: runs of DD elements).
+template <typename TX, int BB, int CC, int DD, int TN> struct RowCfgH {
+    static constexpr int NW = DD, THREADS = 64 * NW;
+    static constexpr int ES = (int)sizeof(TX), EPV = 16 / ES;   // input element, elements per vector
+    static constexpr int MT = BB / 16, KS = CC / 16, NT = TN / 16;
+    static constexpr int XROW = CC * DD, OROW = BB * DD;         // elements per row segment
+    static constexpr int LDX = XROW + EPV, LDO = OROW + 8;       // padded LDS rows (elements)
+    static constexpr int X_VECS = TN * XROW / EPV, O_VECS = TN * OROW / 8;
+    static constexpr int X_PER_T = (X_VECS + THREADS - 1) / THREADS, O_PER_T = (O_VECS + THREADS - 1) / THREADS;
+    static constexpr int X_BYTES = 2 * TN * LDX * ES, LDS_BYTES = X_BYTES + TN * LDO * 2;
+    static_assert(BB % 16 == 0 && CC % 16 == 0 && TN % 16 == 0, "MFMA tiling");
+    static_assert(NW <= 16 && XROW % EPV == 0 && OROW % 8 == 0, "shape");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+__device__ __forceinline__ half_t row_to_half(half_t v) { return v; }
+__device__ __forceinline__ half_t row_to_half(fp8_t v) { return fp8_to_half(v.bits); }
+
+template <typename TX, int BB, int CC, int DD, int TN>
+__global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restrict__ x, const TX *__restrict__ w,
+                                                              half_t *__restrict__ y, int batch, int a, int d,
+                                                              float scale, int wgs_per_a, int n_tiles)
+{
+    typedef RowCfgH<TX, BB, CC, DD, TN> C;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    TX *const xs = (TX *)smem;                         // [2][TN][LDX]
+    half_t *const os = (half_t *)(smem + C::X_BYTES);  // [TN][LDO]
+    const int groups = d / DD;
+    const int ag = blockIdx.x / wgs_per_a;
+    const int s = blockIdx.x - ag * wgs_per_a;
+    const int a_i = ag / groups, d0 = (ag - a_i * groups) * DD;
+    const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
+    if (t_begin >= t_end) return;
+    const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
+    const int dd = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's d_i inside the group
+    const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
+
+    // weights of block (a_i, d0 + dd): element (k, m) at ((a_i*d + d0 + dd)*c + k)*b + m;
+    // A operand of sub-step ks: lane (r, q) holds k = 16*ks + 4*q .. + 3 of row m = 16*mt + r
+    half4_t wreg[C::MT][C::KS];
+    {
+        const TX *wg = w + (size_t)(a_i * d + d0 + dd) * CC * BB;
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) wreg[mt][ks][j] = row_to_half(wg[(16 * ks + 4 * q + j) * BB + 16 * mt + r]);
+    }
+
+    const TX *xg = x + (size_t)a_i * CC * d + d0;
+    half_t *yg = y + (size_t)a_i * BB * d + d0;
+    auto row_off = [&](int e0) { return (e0 / DD) * d + e0 % DD; };
+    uint4_t xreg[2][C::X_PER_T];
+    auto gload = [&](int t, auto P) {
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                const int nn = v / (C::XROW / C::EPV), e0 = (v % (C::XROW / C::EPV)) * C::EPV;
+                const int row = min(t * TN + nn, batch - 1);
+                xreg[decltype(P)::value][i] = *(const uint4_t *)(xg + (size_t)row * in_size + row_off(e0));
+            }
+        }
+    };
+    auto lstore = [&](int buf, auto P) {
+#pragma unroll
+        for (int i = 0; i < C::X_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
+                const int nn = v / (C::XROW / C::EPV), e0 = (v % (C::XROW / C::EPV)) * C::EPV;
+                *(uint4_t *)(xs + (buf * TN + nn) * C::LDX + e0) = xreg[decltype(P)::value][i];
+            }
+        }
+    };
+    auto do_tile = [&](int t, int buf, auto P) {
+        typedef std::integral_constant<int, 1 - decltype(P)::value> Q;
+        if (t + 2 * t_step < t_end) gload(t + 2 * t_step, P);
+        const TX *xb = xs + buf * TN * C::LDX;
+        float4_t acc[C::MT][C::NT];
+#pragma unroll
+        for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt) acc[mt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+        // B operand: lane (r, q) = inputs k = 16*ks + 4*q .. + 3 of batch row 16*nt + r, for this d_i
+        half4_t xf[C::KS][C::NT];
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    xf[ks][nt][j] = row_to_half(xb[(16 * nt + r) * C::LDX + (16 * ks + 4 * q + j) * DD + dd]);
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < C::MT; ++mt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x16f16(wreg[mt][ks], xf[ks][nt], acc[mt][nt], 0, 0, 0);
+        // D: lane (r, q) holds batch row 16*nt + r, outputs m = 16*mt + 4*q + i
+#pragma unroll
+        for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < C::NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = (half_t)(acc[mt][nt][i] * scale);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < C::O_PER_T; ++i) {
+            const int v = tid + i * C::THREADS;
+            if (C::O_VECS % C::THREADS == 0 || v < C::O_VECS) {
+                const int nn = v / (C::OROW / 8), e0 = (v % (C::OROW / 8)) * 8;
+                const int row = t * TN + nn;
+                if (row < batch) {
+                    const uint4_t o = *(const uint4_t *)(os + nn * C::LDO + e0);
+                    __builtin_nontemporal_store(o, (uint4_t *)(yg + (size_t)row * out_size + row_off(e0)));
+                }
+            }
+        }
+        if (t + t_step < t_end) lstore(buf ^ 1, Q{});
+        __syncthreads();
+    };
+
+    gload(t_begin, std::integral_constant<int, 0>{});
+    if (t_begin + t_step < t_end) gload(t_begin + t_step, std::integral_constant<int, 1>{});
+    lstore(0, std::integral_constant<int, 0>{});
+    __syncthreads();
+    for (int t = t_begin; t < t_end; t += 2 * t_step) {
+        do_tile(t, 0, std::integral_constant<int, 0>{});
+        if (t + t_step < t_end) do_tile(t + t_step, 1, std::integral_constant<int, 1>{});
+    }
+}
+
+
 struct RowInst {
-    int bb, cc, dd, tn, lds;
+    int combo, bb, cc, dd, tn, lds;
+    int vec;  // elements per 16-byte vector of the input
     const void *fn;
 };
 #define ROW_INST(BB_, CC_, DD_, TN_, NT_) \
-    {BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
+    {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, 4, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
+#define ROW_INST_H(BB_, CC_, DD_, TN_)                                                                      \
+    {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 8,                             \
+     (const void *)ks_rows_bf_h_kernel<half_t, BB_, CC_, DD_, TN_>}
+#define ROW_INST_Q(BB_, CC_, DD_, TN_)                                                                      \
+    {2, BB_, CC_, DD_, TN_, RowCfgH<fp8_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 16,                             \
+     (const void *)ks_rows_bf_h_kernel<fp8_t, BB_, CC_, DD_, TN_>}
 const RowInst row_insts[] = {
     ROW_INST(48, 48, 16, 16, true), ROW_INST(48, 48, 8, 32, true), ROW_INST(48, 48, 4, 64, true),
     ROW_INST(64, 64, 8, 16, true),  ROW_INST(64, 64, 4, 32, true), ROW_INST(16, 16, 16, 32, true),
@@ -175,6 +322,16 @@ const RowInst row_insts[] = {
     ROW_INST(96, 96, 3, 32, true),   ROW_INST(48, 192, 4, 16, true),
     ROW_INST(48, 192, 3, 16, true), ROW_INST(48, 192, 2, 16, true), ROW_INST(192, 48, 4, 16, true),
     ROW_INST(192, 48, 3, 32, true), ROW_INST(32, 32, 16, 16, true),
+    // fp16
+    ROW_INST_H(48, 48, 16, 16), ROW_INST_H(48, 48, 8, 32), ROW_INST_H(48, 48, 4, 64), ROW_INST_H(48, 48, 12, 32),
+    ROW_INST_H(48, 48, 6, 32),  ROW_INST_H(48, 48, 3, 64), ROW_INST_H(48, 48, 2, 64), ROW_INST_H(64, 64, 16, 16),
+    ROW_INST_H(64, 64, 8, 32),  ROW_INST_H(64, 64, 4, 64), ROW_INST_H(64, 64, 12, 16), ROW_INST_H(64, 64, 6, 32),
+    ROW_INST_H(64, 64, 3, 64),  ROW_INST_H(64, 64, 2, 64), ROW_INST_H(96, 96, 8, 16), ROW_INST_H(96, 96, 4, 32),
+    ROW_INST_H(96, 96, 3, 32),  ROW_INST_H(96, 96, 6, 16), ROW_INST_H(96, 96, 2, 32), ROW_INST_H(48, 192, 8, 16),
+    ROW_INST_H(48, 192, 4, 32), ROW_INST_H(48, 192, 2, 16), ROW_INST_H(48, 192, 3, 32), ROW_INST_H(48, 192, 6, 16),
+    ROW_INST_H(192, 48, 2, 32), ROW_INST_H(192, 48, 8, 16), ROW_INST_H(192, 48, 4, 32), ROW_INST_H(192, 48, 3, 32),
+    ROW_INST_H(192, 48, 6, 16), ROW_INST_H(32, 32, 4, 64), ROW_INST_H(192, 48, 2, 64), ROW_INST_H(16, 16, 16, 64),
+    ROW_INST_H(32, 32, 16, 32), ROW_INST_H(32, 32, 8, 64), ROW_INST_H(128, 128, 4, 16), ROW_INST_H(128, 128, 2, 32),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 
@@ -183,22 +340,28 @@ constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 // variant: bits 0-6 instance (0x7f: first that fits), bits 7.. workgroups per a_i (0: heuristic)
 int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
-    if (p.bs_last || combo_of(p.x_dtype, p.w_dtype, p.y_dtype) != 0) return KSMM_ERR_BAD_ALGO;
+    const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
+    if (p.bs_last || combo < 0 || combo > 2) return KSMM_ERR_BAD_ALGO;
     const int want = variant < 0 ? 0x7f : (variant & 0x7f);
     int64_t wgs = variant < 0 ? 0 : (variant >> 7);
     int pick = -1;
     for (int i = 0; i < N_ROW_INSTS; ++i) {
         if (want != 0x7f && want != i) continue;
         const RowInst &t = row_insts[i];
-        if (t.bb != p.b || t.cc != p.c) continue;
+        if (t.combo != combo || t.bb != p.b || t.cc != p.c) continue;
+        // row segments start on 16-byte boundaries (output vectors: 4 floats / 8 halves)
+        const int ovec = combo == 0 ? 4 : 8;
+        if (((int64_t)p.a * p.c * p.d) % t.vec || ((int64_t)p.a * p.b * p.d) % ovec) continue;
         // all d blocks in one workgroup, or groups of dd whose runs keep the 16-byte alignment
+        const bool grouped_ok = t.dd % t.vec == 0 && t.dd % ovec == 0 && p.d % t.dd == 0;
+        const int run_bytes = t.dd * (combo == 0 ? 4 : 2);  // output run of a group
         if (t.dd == p.d || want != 0x7f) {
-            if (t.dd == p.d || (t.dd % 4 == 0 && p.d % t.dd == 0)) pick = i;
+            if (t.dd == p.d || grouped_ok) pick = i;
             if (pick == i) break;
-        } else if (t.dd % 4 == 0 && p.d % t.dd == 0 && (t.dd >= 8 || p.b <= p.c) &&
+        } else if (grouped_ok && (run_bytes >= 32 || (combo == 0 && p.b <= p.c)) &&
                    (pick < 0 || t.dd > row_insts[pick].dd)) {
-            // the largest group that divides d, unless an exact match follows; 16-byte output
-            // runs (groups of 4) only where the output is not the larger side
+            // the largest group that divides d, unless an exact match follows; 16-byte runs
+            // only for fp32 (groups of 4) where the output is not the larger side
             pick = i;
         }
     }
