@@ -311,6 +311,16 @@ struct RowInst {
 #define ROW_INST_Q(BB_, CC_, DD_, TN_)                                                                      \
     {2, BB_, CC_, DD_, TN_, RowCfgH<fp8_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 16,                             \
      (const void *)ks_rows_bf_h_kernel<fp8_t, BB_, CC_, DD_, TN_>}
+#define ROW_SET_16(M) \
+    M(48, 48, 16, 16), M(48, 48, 8, 32), M(48, 48, 4, 64), M(48, 48, 12, 32), \
+    M(48, 48, 6, 32), M(48, 48, 3, 64), M(48, 48, 2, 64), M(64, 64, 16, 16), \
+    M(64, 64, 8, 32), M(64, 64, 4, 64), M(64, 64, 12, 16), M(64, 64, 6, 32), \
+    M(64, 64, 3, 64), M(64, 64, 2, 64), M(96, 96, 8, 16), M(96, 96, 4, 32), \
+    M(96, 96, 3, 32), M(96, 96, 6, 16), M(96, 96, 2, 32), M(48, 192, 8, 16), \
+    M(48, 192, 4, 32), M(48, 192, 2, 16), M(48, 192, 3, 32), M(48, 192, 6, 16), \
+    M(192, 48, 2, 32), M(192, 48, 8, 16), M(192, 48, 4, 32), M(192, 48, 3, 32), \
+    M(192, 48, 6, 16), M(32, 32, 4, 64), M(192, 48, 2, 64), M(16, 16, 16, 64), \
+    M(32, 32, 16, 32), M(32, 32, 8, 64), M(128, 128, 4, 16), M(128, 128, 2, 32)
 const RowInst row_insts[] = {
     ROW_INST(48, 48, 16, 16, true), ROW_INST(48, 48, 8, 32, true), ROW_INST(48, 48, 4, 64, true),
     ROW_INST(64, 64, 8, 16, true),  ROW_INST(64, 64, 4, 32, true), ROW_INST(16, 16, 16, 32, true),
@@ -322,16 +332,9 @@ const RowInst row_insts[] = {
     ROW_INST(96, 96, 3, 32, true),   ROW_INST(48, 192, 4, 16, true),
     ROW_INST(48, 192, 3, 16, true), ROW_INST(48, 192, 2, 16, true), ROW_INST(192, 48, 4, 16, true),
     ROW_INST(192, 48, 3, 32, true), ROW_INST(32, 32, 16, 16, true),
-    // fp16
-    ROW_INST_H(48, 48, 16, 16), ROW_INST_H(48, 48, 8, 32), ROW_INST_H(48, 48, 4, 64), ROW_INST_H(48, 48, 12, 32),
-    ROW_INST_H(48, 48, 6, 32),  ROW_INST_H(48, 48, 3, 64), ROW_INST_H(48, 48, 2, 64), ROW_INST_H(64, 64, 16, 16),
-    ROW_INST_H(64, 64, 8, 32),  ROW_INST_H(64, 64, 4, 64), ROW_INST_H(64, 64, 12, 16), ROW_INST_H(64, 64, 6, 32),
-    ROW_INST_H(64, 64, 3, 64),  ROW_INST_H(64, 64, 2, 64), ROW_INST_H(96, 96, 8, 16), ROW_INST_H(96, 96, 4, 32),
-    ROW_INST_H(96, 96, 3, 32),  ROW_INST_H(96, 96, 6, 16), ROW_INST_H(96, 96, 2, 32), ROW_INST_H(48, 192, 8, 16),
-    ROW_INST_H(48, 192, 4, 32), ROW_INST_H(48, 192, 2, 16), ROW_INST_H(48, 192, 3, 32), ROW_INST_H(48, 192, 6, 16),
-    ROW_INST_H(192, 48, 2, 32), ROW_INST_H(192, 48, 8, 16), ROW_INST_H(192, 48, 4, 32), ROW_INST_H(192, 48, 3, 32),
-    ROW_INST_H(192, 48, 6, 16), ROW_INST_H(32, 32, 4, 64), ROW_INST_H(192, 48, 2, 64), ROW_INST_H(16, 16, 16, 64),
-    ROW_INST_H(32, 32, 16, 32), ROW_INST_H(32, 32, 8, 64), ROW_INST_H(128, 128, 4, 16), ROW_INST_H(128, 128, 2, 32),
+    // fp16, then e4m3: the same shapes
+    ROW_SET_16(ROW_INST_H),
+    ROW_SET_16(ROW_INST_Q),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 

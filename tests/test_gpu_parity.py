@@ -182,6 +182,9 @@ def test_row_kernel_instances_forced():
                 (1, 48, 48, 32), (2, 48, 48, 24), (1, 64, 64, 64), (1, 16, 16, 64), (1, 192, 48, 16)]
     cases = [("fp16", False, p, batch) for p in shapes16 for batch in (512, 203)]
     _forced_sweep(cases, [1000 + i for i in range(28, 70)], 2, 36)
+    # e4m3: 16-byte vectors of 16 elements
+    cases = [("fp8", False, p, batch) for p in shapes16 for batch in (512, 203)]
+    _forced_sweep(cases, [1000 + i for i in range(64, 110)], 2, 30)
 
 
 def test_tile_subfamilies_forced():

@@ -206,14 +206,14 @@ def test_workspace_queries_need_no_gpu():
     assert need == 2 * (192 * 16 * 1024 * 2)
     assert lib.ksmm_factor_workspace(0, 1, 192, 192, 16, F16, F16, F16, 0) == -3
     descs = (_lib.KsmmFactorDesc * 2)()
-    for i, (a, b, c, d) in enumerate([(2, 64, 64, 8), (16, 64, 64, 1)]):
+    for i, (a, b, c, d) in enumerate([(2, 192, 192, 8), (16, 192, 192, 1)]):
         descs[i].w = 0
         descs[i].a, descs[i].b, descs[i].c, descs[i].d = a, b, c, d
         descs[i].w_dtype = F16
         descs[i].scale = 1.0
     plain = lib.ksmm_chain_workspace(descs, 2, 512, F16)
     assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 1) == plain
-    assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 0) == 3 * (1024 * 512 * 2)
+    assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 0) == 3 * (3072 * 512 * 2)
 
 
 def test_tuned_table_is_sorted_and_every_row_names_a_kernel_that_fits():
