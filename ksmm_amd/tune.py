@@ -52,16 +52,18 @@ def _time_graph(fn, n_sets, steps):
     return t0.elapsed_time(t1) / 1e3 / steps
 
 
-def candidates():
+def candidates(bs_last=True):
     """(algo, variant) pairs worth trying; the library refuses those that do not fit."""
     out = []
-    for inst in range(16):                       # wave family: instance x tiles per wave
-        for it in (0, 1, 2, 4, 8):
-            out.append((2, inst | (it << 8)))
-        for it in (0, 2, 4):                     # the same with tiles dealt round-robin
-            out.append((2, inst | (it << 8) | (1 << 16)))
-    for inst in range(110):                      # batch-size-first row kernel
-        out.append((2, 1000 + inst))
+    if bs_last:
+        for inst in range(16):                   # wave family: instance x tiles per wave
+            for it in (0, 1, 2, 4, 8):
+                out.append((2, inst | (it << 8)))
+            for it in (0, 2, 4):                 # the same with tiles dealt round-robin
+                out.append((2, inst | (it << 8) | (1 << 16)))
+    else:
+        for inst in range(110):                  # batch-size-first row kernel
+            out.append((2, 1000 + inst))
     for inst in range(28):                       # stream
         out.append((3, (2 << 24) | inst))
     for inst in range(40):                       # direct-to-LDS GEMM
@@ -115,7 +117,7 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
     t_auto = _time_graph(lambda j: run(0, -3, j), n_sets, 6)
     steps = int(min(40, max(6, 1.5e-3 / max(t_auto, 1e-6))))
     results = []
-    cands = candidates()
+    cands = candidates(bs_last)
     tried_any = False
     for pool in (cands, KLOOP):
         for algo, variant in pool:
