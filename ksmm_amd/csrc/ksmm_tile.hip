@@ -50,8 +50,11 @@ struct TileCfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
+// RB ("ragged b"): b need not be a multiple of TM nor of the 16-byte weight vector.  The weight
+// tile is then fetched element by element (its rows are not 16-byte aligned; it comes from L2
+// and is small next to the input tile), columns behind b are zeros and are not stored.
 template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int TM, int TN, int TK,
-          int WM, int WN>
+          int WM, int WN, bool RB>
 __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restrict__ x,
                                                               const TW *__restrict__ w,
                                                               TY *__restrict__ y, int batch, int a,
@@ -94,10 +97,22 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
             if (C::W_VECS % C::THREADS == 0 || v < C::W_VECS) {
                 const int kk = v / (TM / C::W_EPV), mm = (v % (TM / C::W_EPV)) * C::W_EPV;
                 // batch-size-last: c need not be a multiple of TK; rows past the block are zeros
-                if (BS_LAST && k0 + kk >= c)
+                if (BS_LAST && k0 + kk >= c) {
                     wreg[i].v = uint4_t{0u, 0u, 0u, 0u};
-                else
+                } else if constexpr (RB) {
+                    union {
+                        uint4_t v;
+                        TW e[C::W_EPV];
+                    } u;
+                    u.v = uint4_t{0u, 0u, 0u, 0u};
+                    const TW *src = wg + (size_t)(k0 + kk) * b + mm;
+#pragma unroll
+                    for (int j = 0; j < C::W_EPV; ++j)
+                        if (m0 + mm + j < b) u.e[j] = src[j];
+                    wreg[i].v = u.v;
+                } else {
                     wreg[i].load(wg + (size_t)(k0 + kk) * b + mm);
+                }
             }
         }
 #pragma unroll
@@ -194,11 +209,11 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
                 const float v = acc[i][j][e] * scale;
                 if (BS_LAST) {
                     const int m = mb + rr, n = nb + l32;
-                    if (n < batch)
+                    if (n < batch && (!RB || m < b))
                         elem<TY>::store(y + ((size_t)(a_i * b + m) * d + d_i) * batch + n, v);
                 } else {
                     const int n = nb + rr, m = mb + l32;
-                    if (n < batch) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * b + m, v);
+                    if (n < batch && (!RB || m < b)) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * b + m, v);
                 }
             }
         }
@@ -467,13 +482,16 @@ int ws_run(const Problem &p, int variant, int wgs_hint, bool launch, ksmm_tile *
 // ---- instance table -----------------------------------------------------------------------
 struct TileInst {
     int combo, bs_last, tm, tn, tk, threads, lds;
+    int ragged_b;
     const void *fn;
 };
 
-#define TILE_INST(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_)                          \
+#define TILE_INST_R(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_, RB_)                    \
     {COMBO_, BL_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                    \
-     TileCfg<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES,                           \
-     (const void *)ks_tile_kernel<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>}
+     TileCfg<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, RB_,                      \
+     (const void *)ks_tile_kernel<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_, RB_>}
+#define TILE_INST(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_)                          \
+    TILE_INST_R(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_, false)
 #define TILE_SET_F32(BL_)                                                                           \
     TILE_INST(0, float, float, float, float, BL_, 128, 128, 16, 2, 2),                              \
         TILE_INST(0, float, float, float, float, BL_, 64, 128, 16, 1, 4),                           \
@@ -504,17 +522,33 @@ const TileInst tile_insts[] = {
     TILE_INST(1, half_t, half_t, half_t, half_t, true, 96, 256, 32, 1, 4),
     TILE_INST(2, half_t, fp8_t, fp8_t, half_t, true, 96, 128, 32, 1, 4),
     TILE_INST(2, half_t, fp8_t, fp8_t, half_t, true, 96, 256, 32, 1, 4),
+    // any b (partial last TM-tile, unaligned weight rows), both layouts
+    TILE_INST_R(0, float, float, float, float, true, 64, 256, 16, 1, 4, true),
+    TILE_INST_R(0, float, float, float, float, true, 128, 256, 16, 2, 2, true),
+    TILE_INST_R(0, float, float, float, float, false, 64, 256, 16, 1, 4, true),
+    TILE_INST_R(0, float, float, float, float, false, 128, 256, 16, 2, 2, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, true, 64, 256, 64, 1, 4, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, true, 128, 256, 32, 2, 2, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, false, 64, 256, 64, 1, 4, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, false, 128, 256, 32, 2, 2, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, true, 64, 256, 64, 1, 4, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, true, 128, 256, 32, 2, 2, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, false, 64, 256, 64, 1, 4, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, false, 128, 256, 32, 2, 2, true),
 };
 constexpr int N_TILE_INSTS = sizeof(tile_insts) / sizeof(TileInst);
 
 bool tile_fits(const TileInst &t, const Problem &p, int combo)
 {
     if (t.combo != combo || t.bs_last != p.bs_last) return false;
-    if (p.b % t.tm) return false;
     if (!p.bs_last && p.c % t.tk) return false;  // batch-size-last tiles zero-fill the K tail
     const int x_epv = 16 / (int)dtype_size(p.x_dtype), w_epv = 16 / (int)dtype_size(p.w_dtype);
     // 16-byte global vectors: weight rows (b elements) and input rows must keep alignment
-    if (p.b % w_epv) return false;
+    if (t.ragged_b) {
+        if (p.b % t.tm == 0 && p.b % w_epv == 0) return false;  // the aligned instances are faster
+    } else if (p.b % t.tm || p.b % w_epv) {
+        return false;
+    }
     if (p.bs_last) {
         if (p.batch % x_epv || p.batch < x_epv) return false;
     } else {
@@ -559,7 +593,7 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         for (int i = 0; i < N_TILE_INSTS; ++i) {
             const TileInst &t = tile_insts[i];
             if (!tile_fits(t, p, combo)) continue;
-            const int64_t wgs = (int64_t)p.a * p.d * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
+            const int64_t wgs = (int64_t)p.a * p.d * ((p.b + t.tm - 1) / t.tm) * ((p.batch + t.tn - 1) / t.tn);
             int64_t score = (int64_t)t.tm * 1000 + t.tn;
             if (wgs < 512) score -= 100000;
             if (score > best_score) {
@@ -571,7 +605,7 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     // nothing else takes it: a GEMM tile that does not fill the chip still beats the generic kernel
     if (pick < 0) return variant == -1 ? gemm_run(p, -2, launch, tile) : KSMM_ERR_BAD_ALGO;
     const TileInst &t = tile_insts[pick];
-    const int m_tiles = p.b / t.tm;
+    const int m_tiles = (p.b + t.tm - 1) / t.tm;
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
     const int64_t blocks = (int64_t)p.a * p.d * m_tiles * n_tiles;
     const int64_t grid = (blocks + 7) / 8 * 8;

@@ -75,7 +75,7 @@ def candidates(bs_last=True):
     return out
 
 
-KLOOP = [(3, inst) for inst in range(64)]        # k-loop tiles: only when nothing else fits
+KLOOP = [(3, inst) for inst in range(80)]        # k-loop tiles: only when nothing else fits
 
 
 def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
