@@ -546,6 +546,9 @@ bool tile_fits(const TileInst &t, const Problem &p, int combo)
     // 16-byte global vectors: weight rows (b elements) and input rows must keep alignment
     if (t.ragged_b) {
         if (p.b % t.tm == 0 && p.b % w_epv == 0) return false;  // the aligned instances are faster
+        // blocks of a few elements fill a sliver of a 32 x 32 MFMA tile: the vector form of the
+        // generic kernel is faster there (measured: (1,16,32,896) fp16 1.55 ms against 2.35 ms)
+        if ((int64_t)p.b * p.c <= 1024) return false;
     } else if (p.b % t.tm || p.b % w_epv) {
         return false;
     }

@@ -215,6 +215,16 @@ def test_tile_subfamilies_forced():
     _forced_sweep(bcases, [(3 << 24) | i for i in range(16)], 3, 4)                      # d > 1 tiles
 
 
+def test_generic_kernel_forms_forced():
+    """One thread per output (variant 0) and the 16-byte vector form for small blocks (variant 1,
+    batch-size-last): blocks of a few elements with large d, b above one chunk of 8 outputs."""
+    cases = [(prec, True, p, batch) for prec in ("fp32", "fp16", "fp8")
+             for p in [(1, 2, 4, 112), (3, 1, 2, 40), (64, 7, 1, 1), (1, 14, 28, 16), (2, 16, 32, 8), (1, 20, 3, 5)]
+             for batch in (64, 1040)]
+    cases += [("fp16", False, (1, 2, 4, 112), 64), ("fp32", True, (1, 2, 4, 112), 7)]
+    _forced_sweep(cases, [0, 1], 1, 70)
+
+
 def test_tuned_table_rows_match_oracle():
     """A sample of the measured table's rows (every element type and layout), run through the
     automatic choice at a batch that consults the table, against the oracle; the tile the
