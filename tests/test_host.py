@@ -234,3 +234,27 @@ def test_tuned_table_is_sorted_and_every_row_names_a_kernel_that_fits():
         small = query_tile(4096, (a, b, c, d), dts[combo], None, bool(bs_last))
         heur = query_tile(4096, (a, b, c, d), dts[combo], None, bool(bs_last), variant=-3)
         assert small == heur
+
+
+def test_every_pattern_shape_class_has_a_kernel_family():
+    """Host-only view of the dispatch for the shape classes of the reference's pattern list that
+    used to end on the one-thread-per-output kernel: b not a multiple of 16, c not a multiple of the
+    K tile, blocks of a few elements, batch-size-first blocks with d > 1."""
+    from ksmm_amd.kernel import query_tile
+
+    f16, f32, f8 = torch.float16, torch.float32, torch.float8_e4m3fn
+    B = 25088
+    for dt in (f32, f16, f8):
+        for bs_last in (True, False):  # ragged b, d = 1: k-loop tiles with a partial last TM-tile
+            t = query_tile(B, (64, 460, 64, 1), dt, None, bs_last, variant=-3)
+            assert t["algo"] == 3 and t["grid"] >= 64 * 98 * 4, (dt, bs_last, t)
+        t = query_tile(B, (1, 448, 910, 32), dt, None, True, variant=-3)       # c = 910: partial K slab
+        assert t["algo"] == 3 and (t["variant"] >> 24) == 4, (dt, t)
+        t = query_tile(B, (1, 2, 4, 7168), dt, None, True, variant=-3)         # tiny block: vector form
+        assert (t["algo"], t["variant"]) == (1, 1), (dt, t)
+        assert query_tile(B + 1, (1, 2, 4, 7168), dt, None, True, variant=-3)["variant"] == 0   # odd batch
+        t = query_tile(B, (1, 48, 48, 32), dt, None, False, variant=-3)        # rows kernel, groups of 16 d_i
+        assert t["algo"] == 2 and t["variant"] >= 1000 and t["tile_d"] == 16, (dt, t)
+    t = query_tile(B, (1, 768, 192, 16), f8, None, True, variant=-3)           # e4m3 GEMM tiles
+    assert t["algo"] == 3 and (t["variant"] >> 24) == 4
+    assert query_tile(B, (1, 192, 192, 16), f16, None, False, variant=-3)["algo"] == 1  # transposed route
