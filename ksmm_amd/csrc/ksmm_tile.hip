@@ -51,8 +51,9 @@ struct TileCfg {
 };
 
 // RB ("ragged b"): b need not be a multiple of TM nor of the 16-byte weight vector.  The weight
-// tile is then fetched element by element (its rows are not 16-byte aligned; it comes from L2
-// and is small next to the input tile), columns behind b are zeros and are not stored.
+// rows are then not 16-byte aligned: vectors that lie inside the block are fetched with one
+// unaligned 16-byte load, the vector that straddles b element by element; columns behind b are
+// zeros and are not stored.
 template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int TM, int TN, int TK,
           int WM, int WN, bool RB>
 __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restrict__ x,
@@ -106,9 +107,15 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
                     } u;
                     u.v = uint4_t{0u, 0u, 0u, 0u};
                     const TW *src = wg + (size_t)(k0 + kk) * b + mm;
+                    if (m0 + mm + C::W_EPV <= b) {
+                        // whole vector inside the block: one 16-byte load at element alignment
+                        // (global memory takes unaligned vector accesses)
+                        __builtin_memcpy(&u.v, src, 16);
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < C::W_EPV; ++j)
-                        if (m0 + mm + j < b) u.e[j] = src[j];
+                        for (int j = 0; j < C::W_EPV; ++j)
+                            if (m0 + mm + j < b) u.e[j] = src[j];
+                    }
                     wreg[i].v = u.v;
                 } else {
                     wreg[i].load(wg + (size_t)(k0 + kk) * b + mm);
@@ -189,34 +196,75 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
             for (int i = 0; i < C::MT; ++i)
 #pragma unroll
                 for (int j = 0; j < C::NT; ++j)
-                    acc[i][j] = BS_LAST ? frag<CT>::mfma(fw[i], fx[j], acc[i][j])
-                                        : frag<CT>::mfma(fx[j], fw[i], acc[i][j]);
+                    // A = input rows along the batch, B = weights: a lane ends up with 4 consecutive
+                    // batch elements of one output feature (batch-size-last: the contiguous axis)
+                    acc[i][j] = frag<CT>::mfma(fx[j], fw[i], acc[i][j]);
         }
         if (s + 1 < steps) lstore(buf ^ 1);
         __syncthreads();
     }
 
-    // D tile: lane holds column (lane % 32) of the B operand and rows 8*(e/4) + 4*(lane/32) + e%4
+    // D tile: lane holds column (lane % 32) of the B operand (an output feature) and rows
+    // 8*(e/4) + 4*(lane/32) + e%4 of the A operand (batch elements)
     const int l32 = lane & 31, lq = lane >> 5;
+    if constexpr (BS_LAST) {
+        // 4 consecutive batch elements per lane and 8-row group: the tile goes through LDS (the
+        // staging buffers are free now) in passes of RPP rows and leaves as 16-byte row pieces
+        constexpr int OES = (int)sizeof(TY), OEPC = 16 / OES;
+        constexpr int RC = TN + OEPC;  // padded row, elements
+        constexpr int RPP_RAW = C::LDS_BYTES / (RC * OES) / 32 * 32;
+        constexpr int RPP = RPP_RAW > TM ? TM : RPP_RAW;
+        constexpr int PASSES = (TM + RPP - 1) / RPP;
+        constexpr int CPR = TN / OEPC;
+        static_assert(RPP >= 32, "output pass");
+        TY *const out = (TY *)smem;
 #pragma unroll
-    for (int i = 0; i < C::MT; ++i)
+        for (int pass = 0; pass < PASSES; ++pass) {
+            if (pass > 0) __syncthreads();
 #pragma unroll
-        for (int j = 0; j < C::NT; ++j) {
-            const int mb = m0 + (wm * C::MT + i) * 32, nb = n0 + (wn * C::NT + j) * 32;
+            for (int i = 0; i < C::MT; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int rr = 8 * (e >> 2) + 4 * lq + (e & 3);
-                const float v = acc[i][j][e] * scale;
-                if (BS_LAST) {
-                    const int m = mb + rr, n = nb + l32;
-                    if (n < batch && (!RB || m < b))
-                        elem<TY>::store(y + ((size_t)(a_i * b + m) * d + d_i) * batch + n, v);
-                } else {
+                for (int j = 0; j < C::NT; ++j) {
+                    const int lrow = (wm * C::MT + i) * 32 + l32, rcol = (wn * C::NT + j) * 32 + 4 * lq;
+                    if (lrow / RPP != pass) continue;  // uniform per wave (32-row tiles)
+                    TY *dst = out + (lrow - pass * RPP) * RC + rcol;
+#pragma unroll
+                    for (int eg = 0; eg < 4; ++eg) {
+                        if constexpr (sizeof(TY) == 4) {
+                            *(float4_t *)(dst + 8 * eg) = float4_t{acc[i][j][4 * eg] * scale, acc[i][j][4 * eg + 1] * scale,
+                                                                   acc[i][j][4 * eg + 2] * scale, acc[i][j][4 * eg + 3] * scale};
+                        } else {
+                            *(half4_t *)(dst + 8 * eg) =
+                                half4_t{(half_t)(acc[i][j][4 * eg] * scale), (half_t)(acc[i][j][4 * eg + 1] * scale),
+                                        (half_t)(acc[i][j][4 * eg + 2] * scale), (half_t)(acc[i][j][4 * eg + 3] * scale)};
+                        }
+                    }
+                }
+            __syncthreads();
+            for (int q = tid; q < RPP * CPR; q += C::THREADS) {
+                const int r = q / CPR, cc = (q % CPR) * OEPC;
+                const int row = pass * RPP + r;
+                if (row >= TM) break;
+                const int m = m0 + row, n = n0 + cc;
+                if (n < batch && (!RB || m < b))
+                    *(uint4_t *)(y + ((size_t)(a_i * b + m) * d + d_i) * batch + n) = *(const uint4_t *)(out + r * RC + cc);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j) {
+                const int mb = m0 + (wm * C::MT + i) * 32, nb = n0 + (wn * C::NT + j) * 32;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int rr = 8 * (e >> 2) + 4 * lq + (e & 3);
+                    const float v = acc[i][j][e] * scale;
                     const int n = nb + rr, m = mb + l32;
                     if (n < batch && (!RB || m < b)) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * b + m, v);
                 }
             }
-        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------
