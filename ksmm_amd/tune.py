@@ -62,7 +62,7 @@ def candidates(bs_last=True):
             for it in (0, 2, 4):                 # the same with tiles dealt round-robin
                 out.append((2, inst | (it << 8) | (1 << 16)))
     else:
-        for inst in range(110):                  # batch-size-first row kernel
+        for inst in range(150):                  # batch-size-first row kernel
             out.append((2, 1000 + inst))
     for inst in range(28):                       # stream
         out.append((3, (2 << 24) | inst))
