@@ -633,6 +633,8 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
         rc = ws_run(p, -1, 0, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        rc = gemm_run(p, -4, launch, tile);  // GEMM tiles with TM = 64
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
     }
     int pick = -1;
     if (variant >= 0) {
