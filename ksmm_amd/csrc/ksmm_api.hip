@@ -116,7 +116,8 @@ bool wants_transposed(const Problem &p)
     Problem q = p;
     q.bs_last = 1;
     memset(&t, 0, sizeof(t));
-    return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && t.algo != KSMM_ALGO_GENERIC;
+    // (the vector form of the generic kernel counts as a real kernel: variant 1)
+    return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && (t.algo != KSMM_ALGO_GENERIC || t.variant == 1);
 }
 
 int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
