@@ -121,8 +121,14 @@ int ksmm_factor_forward(const void *x, const void *w, void *y, int64_t batch, in
                         int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
                         float scale, void *stream);
 
-/* Same, with the kernel family (and optionally a variant, -1 = table default) forced; used
- * by the tuner and by tests that must exercise one family. */
+/* Same, with the kernel family (and optionally a variant, -1 = the family's own choice) forced;
+ * used by the tuner and by tests that must exercise one family.  Variants: KSMM_ALGO_GENERIC
+ * 0 = one thread per output, 1 = 16-byte vector form (batch-size-last); KSMM_ALGO_WAVE
+ * instance | tiles-per-wave << 8 | round-robin << 16, 1000 + i = batch-size-first row kernel i;
+ * KSMM_ALGO_TILE sub-family << 24 | instance (0 k-loop, 1 weight-stationary, 2 stream,
+ * 3 batch-size-first d > 1, 4 direct-to-LDS GEMM); KSMM_ALGO_AUTO -1 = measured table, then
+ * heuristics, -3 = heuristics only.  An instance that cannot run the problem returns
+ * KSMM_ERR_BAD_ALGO. */
 int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batch, int a,
                              int b, int c, int d, int x_dtype, int w_dtype, int y_dtype,
                              int bs_last, float scale, int algo, int variant, void *stream);

@@ -1,4 +1,5 @@
-// "Row" kernel: batch-size-first layout, d > 1, small b x c blocks, fp32.
+// "Row" kernels: batch-size-first layout, d > 1, small b x c blocks.  The fp32 kernel first; the
+// fp16 / e4m3 one further down has the same structure.
 //
 // In this layout a batch row holds, for one a_i, the c*d inputs of all d blocks interleaved
 // (d_i fastest).  A workgroup owns one a_i, a group of DD consecutive d_i (all of them when

@@ -12,11 +12,11 @@
 // contiguous: both "k-outer".  They are copied to LDS as they are and read back with
 // ds_read_b64_tr_b16, the gfx950 LDS transpose load (within 16 lanes, lane i receives
 // element i of each of the four 32-byte rows the group addresses).  Batch-size-first input
-// rows are already k-contiguous (d == 1) and are read with plain 16-byte LDS loads.  The
-// operand whose index runs along the contiguous output axis is the MFMA B operand, so that
-// the 32 lanes of a tile row store 32 consecutive elements:
-//   bs_last : A = W (rows = outputs), B = X (lanes = batch)    -> y[(.)*d*B + n]
-//   bs_first: A = X (rows = batch),   B = W (lanes = outputs)  -> y[n*out + (.)]
+// rows are already k-contiguous (d == 1) and are read with plain 16-byte LDS loads.  In both
+// layouts A = X (rows = batch) and B = W (lanes = outputs):
+//   bs_last : a lane holds 4 consecutive batch elements of one output; the tile is transposed
+//             through LDS after the k loop and stored as 16-byte row pieces  -> y[(.)*d*B + n]
+//   bs_first: the 32 lanes of a tile row store 32 consecutive outputs       -> y[n*out + (.)]
 //
 // Workgroup ids are remapped so that the workgroups that share an input tile (the TM-tiles of
 // one batch tile) run on the same XCD and hit the same L2.
