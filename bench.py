@@ -238,7 +238,7 @@ def cpu_baseline(patterns, bs_last, budget_s=12.0):
 # counter reads for the torch.add calibration kernel per KiB it moves (0.5002 and 1.0000).
 # Counters cannot be collected from inside a timed run, so the figure is carried here; it
 # belongs to that kernel and workload only and is dropped if another kernel is dispatched.
-MEASURED_TRAFFIC = {"algo": 2, "variant": 0, "bytes": int((39421.1 / 0.5002 + 75264.0 / 1.0000) * 1024)}
+MEASURED_TRAFFIC = {"algo": 2, "variant": 0, "bytes": int((39421.5 / 0.5002 + 75264.0 / 1.0000) * 1024)}
 
 
 def main():
