@@ -640,6 +640,9 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         // of the reference's list), then the k-loop tiles
         if (variant == -1 && t.tm < 128 && t.combo != 2 && !(t.ktail && p.c % t.tk)) continue;
         if (variant == -4 && t.tm >= 128) continue;  // -4: the TM = 64 tiles, after stream / weight-stationary
+        // few K slabs: the 8-wave 256 x 256 tiles spend their time in prologue and epilogue; two
+        // 4-wave workgroups per CU do better (measured on the (., 256, 64, .) fp16 patterns: 10 %)
+        if (variant == -1 && t.threads == 512 && t.dd == 1 && p.c <= 128) continue;
         if (!gemm_fits(t, p, combo)) continue;
         if (variant == -1 || variant == -4) {
             // the big tiles only pay when they still fill the chip
