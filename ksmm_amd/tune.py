@@ -163,7 +163,7 @@ def emit(entries, path, batch):
         a, b, c, d = e["pattern"]
         rows.append((a, b, c, d, COMBO[e["prec"]], 1 if e["bs_last"] else 0, e["algo"], e["variant"],
                      e["best_us"], e["auto_us"]))
-    rows.sort()
+    rows.sort(key=lambda r: (r[:6], r[8]))  # by key, fastest first
     rows = [r for i, r in enumerate(rows) if i == 0 or r[:6] != rows[i - 1][:6]]  # one row per key
     with open(path, "w") as f:
         f.write("// Generated by `python -m ksmm_amd.tune` on MI355X (gfx950) at batch %d: fastest measured\n" % batch)

@@ -258,3 +258,24 @@ def test_every_pattern_shape_class_has_a_kernel_family():
     t = query_tile(B, (1, 768, 192, 16), f8, None, True, variant=-3)           # e4m3 GEMM tiles
     assert t["algo"] == 3 and (t["variant"] >> 24) == 4
     assert query_tile(B, (1, 192, 192, 16), f16, None, False, variant=-3)["algo"] == 1  # transposed route
+
+
+def test_tuner_emit_keeps_one_sorted_row_per_key_above_the_threshold(tmp_path):
+    """ksmm_amd.tune.emit: rows only where the measured winner beats the heuristic by more than
+    3 %, one per (pattern, types, layout), sorted for the library's binary search."""
+    from ksmm_amd.tune import emit
+
+    def entry(p, prec, bs_last, auto, best, algo=3, variant=5):
+        return {"pattern": list(p), "prec": prec, "bs_last": bs_last, "auto_us": auto, "best_us": best,
+                "algo": algo, "variant": variant}
+
+    entries = [entry((2, 64, 64, 1), "fp16", True, 10.0, 9.0),
+               entry((1, 48, 48, 16), "fp32", True, 10.0, 9.9),            # within 3 %: dropped
+               entry((1, 48, 48, 16), "fp32", False, 10.0, 8.0, 2, 1000),
+               entry((2, 64, 64, 1), "fp16", True, 10.0, 8.5, 3, 7),        # duplicate key: the faster one
+               entry((1, 16, 16, 4), "fp8", True, None, None, 0, -1)]       # nothing measured
+    path = tmp_path / "t.inc"
+    assert emit(entries, str(path), 25088) == 2
+    rows = [l for l in path.read_text().splitlines() if l.startswith("{")]
+    assert rows[0].startswith("{1, 48, 48, 16, 0, 0, 2, 1000}")
+    assert rows[1].startswith("{2, 64, 64, 1, 1, 1, 3, 7}")
