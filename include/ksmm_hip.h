@@ -17,10 +17,16 @@
  * the per-tensor dequantisation scales and is applied to the fp32 accumulator before the
  * result is rounded to the output type.
  *
- * The library never allocates device memory and keeps no mutable global state.  All
- * launches go to the stream the caller passes (a hipStream_t cast to void*; NULL is the
- * legacy default stream).  Every entry point returns KSMM_OK or a negative error code;
- * ksmm_strerror() names it.  Only ksmm_factor_forward*, ksmm_chain_forward* touch the GPU.
+ * Alignment: x, w and y that start on 16-byte boundaries run on the vector kernels; tensors
+ * that do not are still computed, by the one-thread-per-output kernel (a forced family
+ * refuses them with KSMM_ERR_BAD_ALGO).  A bias vector needs the alignment of its element
+ * type only.  Workspaces must be 16-byte aligned.
+ *
+ * The library never allocates device memory and keeps no caller-visible mutable state (it
+ * only remembers which kernels had their LDS limit raised).  All launches go to the stream the caller passes (a
+ * hipStream_t cast to void*; NULL is the legacy default stream).  Every entry point returns
+ * KSMM_OK or a negative error code; ksmm_strerror() names it.  Only ksmm_factor_forward*,
+ * ksmm_chain_forward* and ksmm_factor_backward* touch the GPU.
  */
 #ifndef KSMM_HIP_H
 #define KSMM_HIP_H
@@ -32,7 +38,7 @@
 extern "C" {
 #endif
 
-#define KSMM_VERSION 1
+#define KSMM_VERSION 2
 
 typedef enum ksmm_dtype {
     KSMM_F32 = 0,
@@ -52,7 +58,8 @@ typedef enum ksmm_status {
     KSMM_ERR_CHAIN_MISMATCH = -8, /* output size of factor i != input size of factor i+1      */
     KSMM_ERR_WORKSPACE = -9,      /* workspace missing or smaller than ksmm_chain_workspace   */
     KSMM_ERR_BAD_CHAIN = -10,     /* n_factors < 1 or > KSMM_MAX_FACTORS                      */
-    KSMM_ERR_ALIAS = -11          /* y overlaps x                                             */
+    KSMM_ERR_ALIAS = -11,         /* y overlaps x, or the workspace overlaps x or y           */
+    KSMM_ERR_BAD_EPILOGUE = -12   /* ksmm_epilogue.act is not a ksmm_act                      */
 } ksmm_status;
 
 /* Kernel families.  KSMM_ALGO_AUTO lets the tile table decide. */
@@ -78,6 +85,21 @@ typedef struct ksmm_tile {
     int lds_bytes;    /* LDS per workgroup                                                 */
     int64_t grid;     /* number of workgroups                                              */
 } ksmm_tile;
+
+/* What the last factor of a call does to its fp32 accumulator before rounding to y's type:
+ *     y = act(scale * acc + bias[output feature]).
+ * Replaces the separate bias pass of KSLinear.post_process
+ * (src/ksmm_py/layer/kronecker_sparse/interface.py:457-466) and the GELU between the two
+ * projections of the ViT feed-forward block (src/ksmm_py/model/vit.py:416-431). */
+typedef enum ksmm_act {
+    KSMM_ACT_NONE = 0,
+    KSMM_ACT_GELU = 1 /* x * Phi(x), the erf form (torch.nn.GELU() default)                 */
+} ksmm_act;
+
+typedef struct ksmm_epilogue {
+    const void *bias; /* NULL, or a*b*d values of y's element type on the device           */
+    int act;          /* ksmm_act                                                          */
+} ksmm_epilogue;
 
 typedef struct ksmm_factor_desc {
     const void *w;    /* kernel-format weight (a*d*c, b)                                   */
@@ -146,6 +168,15 @@ int ksmm_factor_forward_ws(const void *x, const void *w, void *y, int64_t batch,
                            int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
                            float scale, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ksmm_factor_forward_ws with an epilogue (NULL: none) on the accumulator.  The bias add of
+ * KSLinear.post_process (src/ksmm_py/layer/kronecker_sparse/interface.py:457-466) and an
+ * activation that follows the layer (src/ksmm_py/model/vit.py:416-431) then cost no pass
+ * over y of their own. */
+int ksmm_factor_forward_ep(const void *x, const void *w, void *y, int64_t batch, int a, int b,
+                           int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                           float scale, const ksmm_epilogue *epilogue, void *workspace,
+                           int64_t workspace_bytes, void *stream);
+
 /* Bytes of device workspace ksmm_chain_forward needs for these factors in batch-size-last
  * layout (two ping-pong intermediates; 0 for a single factor).  Intermediates have type
  * y_dtype. */
@@ -167,6 +198,14 @@ int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_facto
 int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
                        void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
                        int y_dtype, int bs_last, int fuse, void *stream);
+
+/* ksmm_chain_forward with an epilogue (NULL: none) applied by the last factor:
+ * y = act(scale_n * acc + bias).  Replaces the chain loop plus the bias pass of
+ * KSLinear.post_process (src/ksmm_py/layer/kronecker_sparse/interface.py:269-291, 457-466). */
+int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
+                          void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
+                          int y_dtype, int bs_last, int fuse, const ksmm_epilogue *epilogue,
+                          void *stream);
 
 #ifdef __cplusplus
 }

@@ -12,6 +12,8 @@ LIB_PATH = os.path.join(HERE, "libksmm_hip.so")
 KSMM_F32, KSMM_F16, KSMM_FP8_E4M3 = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_WAVE, ALGO_TILE = 0, 1, 2, 3
 MAX_FACTORS = 16
+ACT_NONE, ACT_GELU = 0, 1
+ABI_VERSION = 2
 
 c_i64 = ctypes.c_int64
 c_int = ctypes.c_int
@@ -30,6 +32,10 @@ class KsmmTile(ctypes.Structure):
 class KsmmFactorDesc(ctypes.Structure):
     _fields_ = [("w", c_vp), ("a", c_int), ("b", c_int), ("c", c_int), ("d", c_int),
                 ("w_dtype", c_int), ("scale", ctypes.c_float)]
+
+
+class KsmmEpilogue(ctypes.Structure):
+    _fields_ = [("bias", c_vp), ("act", c_int)]
 
 
 # name -> (restype, argtypes); every symbol include/ksmm_hip.h declares
@@ -55,6 +61,11 @@ SIGNATURES = {
                                             c_int]),
     "ksmm_chain_forward": (c_int, [ctypes.POINTER(KsmmFactorDesc), c_int, c_vp, c_vp, c_vp, c_i64,
                                    c_i64, c_int, c_int, c_int, c_int, c_vp]),
+    "ksmm_factor_forward_ep": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_int, c_int, ctypes.c_float, ctypes.POINTER(KsmmEpilogue), c_vp, c_i64,
+                                       c_vp]),
+    "ksmm_chain_forward_ep": (c_int, [ctypes.POINTER(KsmmFactorDesc), c_int, c_vp, c_vp, c_vp, c_i64,
+                                      c_i64, c_int, c_int, c_int, c_int, ctypes.POINTER(KsmmEpilogue), c_vp]),
 }
 
 _lib = None
@@ -80,8 +91,9 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.ksmm_version() != 1:
-        raise ImportError("libksmm_hip.so has ABI version %d, expected 1" % lib.ksmm_version())
+    if lib.ksmm_version() != ABI_VERSION:
+        raise ImportError("libksmm_hip.so has ABI version %d, expected %d: rebuild it with "
+                          "`python -m ksmm_amd.build`" % (lib.ksmm_version(), ABI_VERSION))
     _lib = lib
     return lib
 

@@ -1,9 +1,44 @@
 // C ABI of libksmm_hip.so: argument checks, kernel-family dispatch, factor chains.
 #include <string.h>
 
+#include <atomic>
+
 #include "ksmm_common.h"
 
 using namespace ksmm;
+
+namespace ksmm {
+
+// (kernel, device) pairs whose dynamic-LDS limit has been raised: a fixed open-addressing set
+// of atomics.  Insert-only and idempotent, so concurrent callers need no lock; it holds no
+// caller-visible state (a lost race only repeats the attribute call).
+int ensure_dynamic_lds(const void *fn, int bytes)
+{
+    if (bytes <= 64 * 1024) return KSMM_OK;
+    constexpr unsigned SLOTS = 4096;  // far more than kernels x devices
+    static std::atomic<uintptr_t> seen[SLOTS];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return KSMM_ERR_LAUNCH;
+    const uintptr_t key = ((uintptr_t)fn << 8) ^ (uintptr_t)(dev + 1);
+    unsigned h = (unsigned)((key * 0x9E3779B97F4A7C15ull) >> 40) % SLOTS;
+    for (unsigned probe = 0; probe < SLOTS; ++probe, h = (h + 1) % SLOTS) {
+        const uintptr_t cur = seen[h].load(std::memory_order_acquire);
+        if (cur == key) return KSMM_OK;
+        if (cur != 0) continue;
+        // every instance declares its full ring; the limit never has to grow afterwards
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+            return KSMM_ERR_LAUNCH;
+        uintptr_t expected = 0;
+        seen[h].compare_exchange_strong(expected, key, std::memory_order_release);
+        return KSMM_OK;
+    }
+    // table full (cannot happen with the instance counts of this library): set it every time
+    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess
+               ? KSMM_OK
+               : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm
 
 namespace {
 
@@ -122,6 +157,181 @@ bool wants_transposed(const Problem &p)
 
 int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
+bool overlaps(const void *p, int64_t p_bytes, const void *q, int64_t q_bytes)
+{
+    const char *pb = (const char *)p, *qb = (const char *)q;
+    return pb < qb + q_bytes && qb < pb + p_bytes;
+}
+
+
+int check_epilogue(const ksmm_epilogue *ep)
+{
+    if (!ep) return KSMM_OK;
+    if (ep->act != KSMM_ACT_NONE && ep->act != KSMM_ACT_GELU) return KSMM_ERR_BAD_EPILOGUE;
+    return KSMM_OK;
+}
+
+int factor_forward_impl(const void *x, const void *w, void *y, int64_t batch, int a, int b, int c, int d,
+                        int x_dtype, int w_dtype, int y_dtype, int bs_last, float scale, int algo, int variant,
+                        const ksmm_epilogue *ep, void *stream)
+{
+    int rc = check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    if ((rc = check_epilogue(ep)) != KSMM_OK) return rc;
+    if (!x || !w || !y) return KSMM_ERR_NULL_POINTER;
+    const int64_t xbytes = (int64_t)a * c * d * batch * (int64_t)dtype_size(x_dtype);
+    const int64_t ybytes = (int64_t)a * b * d * batch * (int64_t)dtype_size(y_dtype);
+    if (overlaps(x, xbytes, y, ybytes)) return KSMM_ERR_ALIAS;
+    Problem p{x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last ? 1 : 0, scale,
+              (hipStream_t)stream};
+    if (ep) {
+        p.bias = ep->bias;
+        p.act = ep->act;
+    }
+    // Every kernel but the one-thread-per-output one moves 16-byte vectors: tensors that do not
+    // start on a 16-byte boundary run on that kernel (a forced family refuses them).
+    if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) != 0) {
+        if (algo != KSMM_ALGO_AUTO && !(algo == KSMM_ALGO_GENERIC && variant <= 0)) return KSMM_ERR_BAD_ALGO;
+        return generic_run(p, 0, true, nullptr);
+    }
+    return dispatch(p, algo, variant, true, nullptr);
+}
+
+int factor_forward_ws_impl(const void *x, const void *w, void *y, int64_t batch, int a, int b, int c, int d,
+                           int x_dtype, int w_dtype, int y_dtype, int bs_last, float scale,
+                           const ksmm_epilogue *ep, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    const int64_t need = ksmm_factor_workspace(batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last);
+    if (need < 0) return (int)need;
+    if (need == 0)
+        return factor_forward_impl(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale,
+                                   KSMM_ALGO_AUTO, -1, ep, stream);
+    if (!x || !w || !y) return KSMM_ERR_NULL_POINTER;
+    if (!workspace || workspace_bytes < need) return KSMM_ERR_WORKSPACE;
+    const int64_t in_size = (int64_t)a * c * d, out_size = (int64_t)a * b * d;
+    const int64_t xbytes = in_size * batch * (int64_t)dtype_size(x_dtype);
+    const int64_t ybytes = out_size * batch * (int64_t)dtype_size(y_dtype);
+    if (overlaps(x, xbytes, y, ybytes) || overlaps(workspace, need, x, xbytes) || overlaps(workspace, need, y, ybytes))
+        return KSMM_ERR_ALIAS;
+    if (((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
+    char *xt = (char *)workspace;
+    char *yt = xt + align256(xbytes);
+    int rc = transpose_run(x, xt, batch, in_size, (int)dtype_size(x_dtype), (hipStream_t)stream);
+    if (rc != KSMM_OK) return rc;
+    rc = factor_forward_impl(xt, w, yt, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, 1, scale, KSMM_ALGO_AUTO, -1,
+                             ep, stream);
+    if (rc != KSMM_OK) return rc;
+    return transpose_run(yt, y, out_size, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+}
+
+int check_chain(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype)
+{
+    if (!f) return KSMM_ERR_NULL_POINTER;
+    if (n < 1 || n > KSMM_MAX_FACTORS) return KSMM_ERR_BAD_CHAIN;
+    for (int i = 0; i < n; ++i) {
+        // the first factor reads x_dtype, later ones read the intermediate type y_dtype
+        int rc = check_shape(batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
+                             f[i].w_dtype, y_dtype);
+        if (rc != KSMM_OK) return rc;
+        if (i > 0 && (int64_t)f[i].a * f[i].c * f[i].d != (int64_t)f[i - 1].a * f[i - 1].b * f[i - 1].d)
+            return KSMM_ERR_CHAIN_MISMATCH;
+    }
+    return KSMM_OK;
+}
+
+// batch-size-first chain with at least one factor that needs the transposed route
+bool chain_wants_transposed(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype,
+                            int bs_last)
+{
+    if (bs_last) return false;
+    for (int i = 0; i < n; ++i) {
+        Problem p{nullptr, nullptr, nullptr, batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
+                  f[i].w_dtype, y_dtype, 0, 1.f, nullptr};
+        if (wants_transposed(p)) return true;
+    }
+    return false;
+}
+
+// The chain launcher behind ksmm_chain_forward and ksmm_chain_forward_ep: `ep` (may be null)
+// belongs to the last factor.
+int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y, void *workspace,
+                       int64_t workspace_bytes, int64_t batch, int x_dtype, int y_dtype, int bs_last, int fuse,
+                       const ksmm_epilogue *ep, void *stream)
+{
+    int rc = check_chain(factors, n_factors, batch, x_dtype, y_dtype);
+    if (rc != KSMM_OK) return rc;
+    if ((rc = check_epilogue(ep)) != KSMM_OK) return rc;
+    if (!x || !y) return KSMM_ERR_NULL_POINTER;
+    for (int i = 0; i < n_factors; ++i)
+        if (!factors[i].w) return KSMM_ERR_NULL_POINTER;
+    const ksmm_factor_desc &last = factors[n_factors - 1];
+    const int64_t in0 = (int64_t)factors[0].a * factors[0].c * factors[0].d;
+    const int64_t out_n = (int64_t)last.a * last.b * last.d;
+    const int64_t xbytes = in0 * batch * (int64_t)dtype_size(x_dtype);
+    const int64_t ybytes = out_n * batch * (int64_t)dtype_size(y_dtype);
+    if (overlaps(x, xbytes, y, ybytes)) return KSMM_ERR_ALIAS;
+    if (workspace && workspace_bytes > 0) {
+        if (overlaps(workspace, workspace_bytes, x, xbytes) || overlaps(workspace, workspace_bytes, y, ybytes))
+            return KSMM_ERR_ALIAS;
+        if (((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
+    }
+    auto ep_of = [&](int i) { return i == n_factors - 1 ? ep : nullptr; };
+    if (chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
+        // transpose once, run the whole chain in batch-size-last layout, transpose back
+        const int64_t need_t = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 0);
+        if (workspace && workspace_bytes >= need_t) {
+            const int64_t xt_bytes = align256(xbytes);
+            char *xt = (char *)workspace;
+            char *pp = xt + xt_bytes;
+            const int64_t one = (need_t - xt_bytes) / 2;
+            rc = transpose_run(x, xt, batch, in0, (int)dtype_size(x_dtype), (hipStream_t)stream);
+            if (rc != KSMM_OK) return rc;
+            const void *cur = xt;
+            int cur_dtype = x_dtype;
+            rc = KSMM_ERR_BAD_ALGO;
+            if (fuse)
+                rc = chain16_run(factors, n_factors, xt, pp, batch, x_dtype, y_dtype, 1, true, (hipStream_t)stream, ep);
+            if (rc == KSMM_OK) {
+                cur = pp;
+            } else if (rc != KSMM_ERR_BAD_ALGO) {
+                return rc;
+            } else {
+                for (int i = 0; i < n_factors; ++i) {
+                    void *dst = pp + (i & 1) * one;
+                    rc = factor_forward_impl(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b, factors[i].c,
+                                             factors[i].d, cur_dtype, factors[i].w_dtype, y_dtype, 1, factors[i].scale,
+                                             KSMM_ALGO_AUTO, -1, ep_of(i), stream);
+                    if (rc != KSMM_OK) return rc;
+                    cur = dst;
+                    cur_dtype = y_dtype;
+                }
+            }
+            return transpose_run(cur, y, out_n, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+        }
+    }
+    if (fuse) {
+        // chains whose intermediates fit LDS run as one kernel (no workspace traffic)
+        rc = chain16_run(factors, n_factors, x, y, batch, x_dtype, y_dtype, bs_last ? 1 : 0, true,
+                         (hipStream_t)stream, ep);
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
+    }
+    const int64_t need = ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
+    if (n_factors > 1 && (!workspace || workspace_bytes < need)) return KSMM_ERR_WORKSPACE;
+    char *buf[2] = {(char *)workspace, (char *)workspace + need / 2};
+    const void *cur = x;
+    int cur_dtype = x_dtype;
+    for (int i = 0; i < n_factors; ++i) {
+        void *dst = (i == n_factors - 1) ? y : (void *)buf[i & 1];
+        rc = factor_forward_impl(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b, factors[i].c,
+                                 factors[i].d, cur_dtype, factors[i].w_dtype, y_dtype, bs_last, factors[i].scale,
+                                 KSMM_ALGO_AUTO, -1, ep_of(i), stream);
+        if (rc != KSMM_OK) return rc;
+        cur = dst;
+        cur_dtype = y_dtype;
+    }
+    return KSMM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -142,7 +352,8 @@ const char *ksmm_strerror(int status)
     case KSMM_ERR_CHAIN_MISMATCH: return "consecutive factors have incompatible sizes";
     case KSMM_ERR_WORKSPACE: return "workspace missing or too small";
     case KSMM_ERR_BAD_CHAIN: return "bad number of factors";
-    case KSMM_ERR_ALIAS: return "output overlaps input";
+    case KSMM_ERR_ALIAS: return "output, input or workspace overlap";
+    case KSMM_ERR_BAD_EPILOGUE: return "unknown activation in the epilogue";
     default: return "unknown ksmm status";
     }
 }
@@ -194,24 +405,16 @@ int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batc
                              int b, int c, int d, int x_dtype, int w_dtype, int y_dtype,
                              int bs_last, float scale, int algo, int variant, void *stream)
 {
-    int rc = check_shape(batch, a, b, c, d, x_dtype, w_dtype, y_dtype);
-    if (rc != KSMM_OK) return rc;
-    if (!x || !w || !y) return KSMM_ERR_NULL_POINTER;
-    const char *xb = (const char *)x, *yb = (const char *)y;
-    const int64_t xbytes = (int64_t)a * c * d * batch * (int64_t)dtype_size(x_dtype);
-    const int64_t ybytes = (int64_t)a * b * d * batch * (int64_t)dtype_size(y_dtype);
-    if (xb < yb + ybytes && yb < xb + xbytes) return KSMM_ERR_ALIAS;
-    Problem p{x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last ? 1 : 0, scale,
-              (hipStream_t)stream};
-    return dispatch(p, algo, variant, true, nullptr);
+    return factor_forward_impl(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale, algo,
+                               variant, nullptr, stream);
 }
 
 int ksmm_factor_forward(const void *x, const void *w, void *y, int64_t batch, int a, int b,
                         int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
                         float scale, void *stream)
 {
-    return ksmm_factor_forward_algo(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last,
-                                    scale, KSMM_ALGO_AUTO, -1, stream);
+    return factor_forward_impl(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale,
+                               KSMM_ALGO_AUTO, -1, nullptr, stream);
 }
 
 int64_t ksmm_factor_workspace(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
@@ -230,35 +433,17 @@ int ksmm_factor_forward_ws(const void *x, const void *w, void *y, int64_t batch,
                            int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
                            float scale, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    const int64_t need = ksmm_factor_workspace(batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last);
-    if (need < 0) return (int)need;
-    if (need == 0)
-        return ksmm_factor_forward(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale, stream);
-    if (!x || !w || !y) return KSMM_ERR_NULL_POINTER;
-    if (!workspace || workspace_bytes < need) return KSMM_ERR_WORKSPACE;
-    const int64_t in_size = (int64_t)a * c * d, out_size = (int64_t)a * b * d;
-    char *xt = (char *)workspace;
-    char *yt = xt + align256(in_size * batch * (int64_t)dtype_size(x_dtype));
-    int rc = transpose_run(x, xt, batch, in_size, (int)dtype_size(x_dtype), (hipStream_t)stream);
-    if (rc != KSMM_OK) return rc;
-    rc = ksmm_factor_forward(xt, w, yt, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, 1, scale, stream);
-    if (rc != KSMM_OK) return rc;
-    return transpose_run(yt, y, out_size, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+    return factor_forward_ws_impl(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale, nullptr,
+                                  workspace, workspace_bytes, stream);
 }
 
-static int check_chain(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype)
+int ksmm_factor_forward_ep(const void *x, const void *w, void *y, int64_t batch, int a, int b,
+                           int c, int d, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                           float scale, const ksmm_epilogue *epilogue, void *workspace,
+                           int64_t workspace_bytes, void *stream)
 {
-    if (!f) return KSMM_ERR_NULL_POINTER;
-    if (n < 1 || n > KSMM_MAX_FACTORS) return KSMM_ERR_BAD_CHAIN;
-    for (int i = 0; i < n; ++i) {
-        // the first factor reads x_dtype, later ones read the intermediate type y_dtype
-        int rc = check_shape(batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
-                             f[i].w_dtype, y_dtype);
-        if (rc != KSMM_OK) return rc;
-        if (i > 0 && (int64_t)f[i].a * f[i].c * f[i].d != (int64_t)f[i - 1].a * f[i - 1].b * f[i - 1].d)
-            return KSMM_ERR_CHAIN_MISMATCH;
-    }
-    return KSMM_OK;
+    return factor_forward_ws_impl(x, w, y, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, bs_last, scale, epilogue,
+                                  workspace, workspace_bytes, stream);
 }
 
 int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
@@ -277,19 +462,6 @@ int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int
     // two buffers, each rounded up to 256 bytes so that both stay 256-byte aligned
     int64_t one = (widest * batch * (int64_t)dtype_size(y_dtype) + 255) / 256 * 256;
     return n_factors > 1 ? 2 * one : 0;
-}
-
-// batch-size-first chain with at least one factor that needs the transposed route
-static bool chain_wants_transposed(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype,
-                                   int bs_last)
-{
-    if (bs_last) return false;
-    for (int i = 0; i < n; ++i) {
-        Problem p{nullptr, nullptr, nullptr, batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
-                  f[i].w_dtype, y_dtype, 0, 1.f, nullptr};
-        if (wants_transposed(p)) return true;
-    }
-    return false;
 }
 
 int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
@@ -313,67 +485,17 @@ int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const voi
                        void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
                        int y_dtype, int bs_last, int fuse, void *stream)
 {
-    int rc = check_chain(factors, n_factors, batch, x_dtype, y_dtype);
-    if (rc != KSMM_OK) return rc;
-    if (!x || !y) return KSMM_ERR_NULL_POINTER;
-    for (int i = 0; i < n_factors; ++i)
-        if (!factors[i].w) return KSMM_ERR_NULL_POINTER;
-    if (chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
-        // transpose once, run the whole chain in batch-size-last layout, transpose back
-        const int64_t need_t = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 0);
-        if (workspace && workspace_bytes >= need_t) {
-            const int64_t in0 = (int64_t)factors[0].a * factors[0].c * factors[0].d;
-            const int64_t out_n = (int64_t)factors[n_factors - 1].a * factors[n_factors - 1].b * factors[n_factors - 1].d;
-            const int64_t xt_bytes = align256(in0 * batch * (int64_t)dtype_size(x_dtype));
-            char *xt = (char *)workspace;
-            char *pp = xt + xt_bytes;
-            const int64_t one = (need_t - xt_bytes) / 2;
-            rc = transpose_run(x, xt, batch, in0, (int)dtype_size(x_dtype), (hipStream_t)stream);
-            if (rc != KSMM_OK) return rc;
-            const void *cur = xt;
-            int cur_dtype = x_dtype;
-            rc = KSMM_ERR_BAD_ALGO;
-            if (fuse)
-                rc = chain16_run(factors, n_factors, xt, pp, batch, x_dtype, y_dtype, 1, true, (hipStream_t)stream);
-            if (rc == KSMM_OK) {
-                cur = pp;
-            } else if (rc != KSMM_ERR_BAD_ALGO) {
-                return rc;
-            } else {
-                for (int i = 0; i < n_factors; ++i) {
-                    void *dst = pp + (i & 1) * one;
-                    rc = ksmm_factor_forward_algo(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b,
-                                                  factors[i].c, factors[i].d, cur_dtype, factors[i].w_dtype,
-                                                  y_dtype, 1, factors[i].scale, KSMM_ALGO_AUTO, -1, stream);
-                    if (rc != KSMM_OK) return rc;
-                    cur = dst;
-                    cur_dtype = y_dtype;
-                }
-            }
-            return transpose_run(cur, y, out_n, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
-        }
-    }
-    if (fuse) {
-        // chains whose intermediates fit LDS run as one kernel (no workspace traffic)
-        rc = chain16_run(factors, n_factors, x, y, batch, x_dtype, y_dtype, bs_last ? 1 : 0, true,
-                         (hipStream_t)stream);
-        if (rc != KSMM_ERR_BAD_ALGO) return rc;
-    }
-    const int64_t need = ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
-    if (n_factors > 1 && (!workspace || workspace_bytes < need)) return KSMM_ERR_WORKSPACE;
-    char *buf[2] = {(char *)workspace, (char *)workspace + need / 2};
-    const void *cur = x;
-    int cur_dtype = x_dtype;
-    for (int i = 0; i < n_factors; ++i) {
-        void *dst = (i == n_factors - 1) ? y : (void *)buf[i & 1];
-        rc = ksmm_factor_forward_algo(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b,
-                                      factors[i].c, factors[i].d, cur_dtype, factors[i].w_dtype,
-                                      y_dtype, bs_last, factors[i].scale, KSMM_ALGO_AUTO, -1, stream);
-        if (rc != KSMM_OK) return rc;
-        cur = dst;
-        cur_dtype = y_dtype;
-    }
-    return KSMM_OK;
+    return chain_forward_impl(factors, n_factors, x, y, workspace, workspace_bytes, batch, x_dtype, y_dtype,
+                              bs_last, fuse, nullptr, stream);
+}
+
+int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
+                          void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
+                          int y_dtype, int bs_last, int fuse, const ksmm_epilogue *epilogue,
+                          void *stream)
+{
+    return chain_forward_impl(factors, n_factors, x, y, workspace, workspace_bytes, batch, x_dtype, y_dtype,
+                              bs_last, fuse, epilogue, stream);
 }
 
 }  // extern "C"

@@ -29,17 +29,6 @@
 // round trip of the intermediate per factor.
 #include "ksmm_mfma.h"
 
-#ifdef KSMM_PROFILE
-// Phase timestamps of wave 0 of every workgroup (standalone profiling builds only).
-__device__ unsigned long long ksmm_cprof[256][64];
-#define KC_STAMP(slot)                                                                    \
-    do {                                                                                  \
-        if (threadIdx.x == 0 && blockIdx.x < 256 && (slot) < 64)                          \
-            ksmm_cprof[blockIdx.x][(slot)] = __builtin_amdgcn_s_memtime();                \
-    } while (0)
-#else
-#define KC_STAMP(slot) do { } while (0)
-#endif
 
 namespace ksmm {
 
@@ -47,6 +36,8 @@ struct Chain16Args {
     const void *w[4];
     int log2d[4];
     float scale[4];
+    const void *bias;  // of the last factor's outputs (fp16), or none
+    int act;
 };
 
 namespace {
@@ -94,8 +85,6 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
     if (c_begin >= c_end) return;
     const int c_last = c_begin + ((c_end - 1 - c_begin) / c_step) * c_step;  // this workgroup's last chunk
     const int n_blocks = n_feat / 16;  // blocks per factor
-    KC_STAMP(0);
-    int chunk_no = 0;
     constexpr int MAXB = 64 / CH_WAVES;  // blocks per wave and factor (n_feat <= 1024)
 
     // ---- input staging: each thread carries 16-byte pieces of the next chunk in registers ----
@@ -163,7 +152,6 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         __builtin_amdgcn_sched_barrier(0);
         gload(c_begin, true);
         __builtin_amdgcn_sched_barrier(0);
-        KC_STAMP(10);
 #pragma unroll
         for (int f = 0; f < NF; ++f)
 #pragma unroll
@@ -180,9 +168,7 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                 }
             }
     }
-    KC_STAMP(11);
     __syncthreads();
-    KC_STAMP(12);
     half4_t wreg[NF][MAXB];
 #pragma unroll
     for (int f = 0; f < NF; ++f)
@@ -201,12 +187,10 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         v_out[f] = lds_piece(r << args.log2d[f], 0, q);
     }
     __syncthreads();
-    KC_STAMP(1);
 
     for (int n0 = c_begin; n0 < c_end; n0 += c_step) {
         lstore();
         __syncthreads();
-        KC_STAMP(4 + 8 * chunk_no);
         if (FULL)
             gload(min(n0 + c_step, c_last), n0 + c_step < c_end);  // after the last chunk: a dummy request
         else if (n0 + c_step < c_end)
@@ -243,11 +227,21 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                                                                    float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 // D^T: lane (r = output m, q) holds the 4 columns of piece q of slot s
                 half4_t o[4];
-#pragma unroll
-                for (int s = 0; s < 4; ++s)
-                    o[s] = half4_t{(half_t)(acc[s][0] * scale), (half_t)(acc[s][1] * scale),
-                                   (half_t)(acc[s][2] * scale), (half_t)(acc[s][3] * scale)};
                 const int row0 = block_row0(g);
+                if (f + 1 == NF && (args.bias != nullptr || args.act != KSMM_ACT_NONE)) {
+                    // the chain's epilogue: the lane's output row is row0 + r * d
+                    const Epi ep{scale, args.act, args.bias};
+                    const float bv = epi_bias<half_t>(ep, (size_t)(row0 + (r << ld)));
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        o[s] = half4_t{(half_t)epi_finish(ep, acc[s][0], bv), (half_t)epi_finish(ep, acc[s][1], bv),
+                                       (half_t)epi_finish(ep, acc[s][2], bv), (half_t)epi_finish(ep, acc[s][3], bv)};
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        o[s] = half4_t{(half_t)(acc[s][0] * scale), (half_t)(acc[s][1] * scale),
+                                       (half_t)(acc[s][2] * scale), (half_t)(acc[s][3] * scale)};
+                }
                 if (f + 1 < NF) {
                     // all inputs of the block are in registers: write its 16 output rows in place
                     const int obase = lds_piece(row0, 0, 0) ^ v_out[f];
@@ -264,11 +258,8 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                 }
             }
             __syncthreads();
-            KC_STAMP(5 + 8 * chunk_no + f);
         }
-        ++chunk_no;
     }
-    KC_STAMP(2);
 }
 
 template <typename TX, typename TW> const void *chain16_fn(int nf, bool full)
@@ -285,7 +276,7 @@ template <typename TX, typename TW> const void *chain16_fn(int nf, bool full)
 
 // Returns KSMM_ERR_BAD_ALGO when the chain is not a radix-16 butterfly this kernel takes.
 int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_t batch, int x_dtype,
-                int y_dtype, int bs_last, bool launch, hipStream_t stream)
+                int y_dtype, int bs_last, bool launch, hipStream_t stream, const ksmm_epilogue *ep)
 {
     if (!bs_last || n < 2 || n > 4 || y_dtype != KSMM_F16) return KSMM_ERR_BAD_ALGO;
     if (x_dtype != KSMM_FP8_E4M3 && x_dtype != KSMM_F16) return KSMM_ERR_BAD_ALGO;
@@ -319,14 +310,13 @@ int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_
         args.log2d[i] = __builtin_ctz((unsigned)f[j].d);
         args.scale[i] = f[j].scale;
     }
+    args.bias = ep ? ep->bias : nullptr;
+    args.act = ep ? ep->act : KSMM_ACT_NONE;
     // one persistent workgroup per CU, chunks dealt round-robin
     const int64_t n_chunks = (batch + CH_TN - 1) / CH_TN;
     const int64_t wgs = n_chunks < 256 ? n_chunks : 256;
     const int lds = (int)n_feat * CH_ROW;
-    if (lds > 64 * 1024) {
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (ensure_dynamic_lds(fn, lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)batch, n_feat_i = (int)n_feat;
     void *kargs[] = {(void *)&x, (void *)&y, (void *)&args, &batch_i, &n_feat_i};
     hipError_t e = hipLaunchKernel(fn, dim3((unsigned)wgs), dim3(CH_THREADS), kargs, lds, stream);

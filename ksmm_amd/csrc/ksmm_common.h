@@ -74,7 +74,43 @@ struct Problem {
     int bs_last;
     float scale;
     hipStream_t stream;
+    const void *bias = nullptr;  // one value of y's type per output feature, or none
+    int act = KSMM_ACT_NONE;
 };
+
+// What a kernel does to an fp32 accumulator before rounding it to the output type:
+// v = act(acc * scale + bias[output feature]).  Passed to the kernels by value.
+struct Epi {
+    float scale;
+    int act;
+    const void *bias;
+};
+static inline Epi epi_of(const Problem &p) { return Epi{p.scale, p.act, p.bias}; }
+
+// GELU, erf form: x * Phi(x).  erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7, branch-free:
+// one reciprocal, one exponential, a degree-5 polynomial), far inside fp32 storage rounding of
+// the result for the value range of activations.
+__device__ __forceinline__ float gelu_erf(float x)
+{
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float poly = fmaf(1.061405429f, t, -1.453152027f);
+    poly = fmaf(poly, t, 1.421413741f);
+    poly = fmaf(poly, t, -0.284496736f);
+    poly = fmaf(poly, t, 0.254829592f);
+    const float tail = 0.5f * poly * t * __builtin_amdgcn_exp2f(-z * z * 1.44269504088896341f);  // 0.5 * erfc(z)
+    return x * (x >= 0.f ? 1.0f - tail : tail);
+}
+
+template <typename TY> __device__ __forceinline__ float epi_bias(const Epi &e, size_t feature)
+{
+    return e.bias ? (float)((const TY *)e.bias)[feature] : 0.f;
+}
+__device__ __forceinline__ float epi_finish(const Epi &e, float acc, float bias_value)
+{
+    const float v = fmaf(acc, e.scale, bias_value);
+    return e.act == KSMM_ACT_GELU ? gelu_erf(v) : v;
+}
 
 // dtype combination index: 0 f32, 1 f16, 2 fp8*fp8->f16, 3 f16*fp8->f16, -1 unsupported
 static inline int combo_of(int xd, int wd, int yd)
@@ -85,6 +121,11 @@ static inline int combo_of(int xd, int wd, int yd)
     if (xd == KSMM_F16 && wd == KSMM_FP8_E4M3 && yd == KSMM_F16) return 3;
     return -1;
 }
+
+// Kernels that use more than 64 KB of dynamic LDS need their limit raised before the first
+// launch.  Done once per (kernel, device): later calls only look the pair up.  Returns
+// KSMM_OK or KSMM_ERR_LAUNCH.
+int ensure_dynamic_lds(const void *fn, int bytes);
 
 // Launchers, one per kernel family.  Each fills `tile` and, when `launch` is true, enqueues
 // the kernel on p.stream.  They return KSMM_ERR_BAD_ALGO when the family (or the requested
@@ -100,6 +141,6 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  /
 // Fused radix-16 chain (intermediates in LDS); KSMM_ERR_BAD_ALGO when the chain does not qualify.
 int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream);
 int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_t batch, int x_dtype,
-                int y_dtype, int bs_last, bool launch, hipStream_t stream);
+                int y_dtype, int bs_last, bool launch, hipStream_t stream, const ksmm_epilogue *ep);
 
 }  // namespace ksmm

@@ -27,17 +27,6 @@
 //  template_kernels_half.cuh:103-1092).
 #include "ksmm_mfma.h"
 
-#ifdef KSMM_PROFILE
-// Phase timestamps of wave 0 of the first workgroups (standalone profiling builds only).
-__device__ unsigned long long ksmm_gprof[256][64];
-#define KG_STAMP(slot)                                                                    \
-    do {                                                                                  \
-        if (threadIdx.x == 0 && blockIdx.x < 256 && (slot) < 64)                          \
-            ksmm_gprof[blockIdx.x][(slot)] = __builtin_amdgcn_s_memtime();                \
-    } while (0)
-#else
-#define KG_STAMP(slot) do { } while (0)
-#endif
 
 namespace ksmm {
 
@@ -47,26 +36,16 @@ constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | (((n >
 
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr)
 {
-#ifdef KSMM_GABL_NODMA
-    if (lds_addr != 0xffffffffu) return;
-#endif
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(gptr), "s"(lds_addr)
                  : "memory", "m0");
 }
 
-#ifdef KSMM_GABL_NOMFMA
-__device__ __forceinline__ float abl_first(float v) { return v; }
-__device__ __forceinline__ float abl_first(half8_t v) { return (float)v[0] + (float)v[7]; }
-#endif
 
 // the same with a uniform 64-bit base (SGPR pair) and a 32-bit per-lane byte offset
 __device__ __forceinline__ void dma16s(const void *sbase, uint32_t voff, uint32_t lds_addr)
 {
-#ifdef KSMM_GABL_NODMA
-    if (lds_addr != 0xffffffffu) return;
-#endif
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(sbase), "s"(lds_addr)
@@ -180,9 +159,11 @@ template <typename CT, typename TY, bool BS_LAST, int DD, int TM, int TN, int TK
 __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__restrict__ x,
                                                               const CT *__restrict__ w,
                                                               TY *__restrict__ y, int batch, int a,
-                                                              int b, int c, int d, float scale,
+                                                              int b, int c, int d, Epi ep,
                                                               int m_tiles, int n_tiles, int blocks, int pf_dist)
 {
+    const float scale = ep.scale;
+    const bool has_epi = ep.bias != nullptr || ep.act != KSMM_ACT_NONE;  // uniform
     typedef GemmCfg<CT, BS_LAST, DD, TM, TN, TK, WM, WN, ST> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     // XCD-aware id: TM-tiles of one input tile get consecutive logical ids on one XCD
@@ -291,7 +272,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = 0.f;
 
-    KG_STAMP(0);
     // L2 prefetch for the workgroup that will take this one's place: the input tile of logical
     // id lid + pf_dist (same XCD, pf_dist = workgroups resident per XCD), this workgroup's
     // share of its rows (the TM-tiles of one input tile split it).  One 4-byte load per
@@ -328,15 +308,11 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     }
 #pragma unroll
     for (int p = 0; p < ST - 1; ++p) issue(min(p, steps - 1), p);
-    KG_STAMP(1);
 
     // MFMA operands of sub-step k0 of the slab whose operand addresses are wa[] / xa[]
     typedef typename frag<CT>::type frag_t;
     auto load_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[DD][C::MT],
                           frag_t(&fx)[DD][C::NT]) {
-#ifdef KSMM_GABL_NOFRAG
-        if (batch != -12345) return;
-#endif
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
@@ -422,16 +398,13 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
             if (kk + 1 < K0) {
                 load_frags(wa, xa, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], fx[(kk + 1) & 1]);
             } else {
-                KG_STAMP(4 + 4 * it);
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
                 if (KT && it + 2 == steps && rem < TK) clear_tail((it + 1) % ST);
                 __syncthreads();  // slab it+1 landed for every wave, and everyone left slab it
-                KG_STAMP(5 + 4 * it);
                 if (it + 1 < steps) {
                     stage_addrs((it + 1) % ST);
                     load_frags(wa, xa, 0, fw[0], fx[0]);
                 }
-                KG_STAMP(6 + 4 * it);
             }
 #pragma unroll
             for (int dd = 0; dd < DD; ++dd)
@@ -439,12 +412,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
                 for (int i = 0; i < C::MT; ++i)
 #pragma unroll
                     for (int j = 0; j < C::NT; ++j) {
-#ifdef KSMM_GABL_NOMFMA
-                        acc[dd][i][j][0] += abl_first(fw[kk & 1][dd][i]) + abl_first(fx[kk & 1][dd][j]);
-#else
                         acc[dd][i][j] = BS_LAST ? frag<CT>::mfma(fx[kk & 1][dd][j], fw[kk & 1][dd][i], acc[dd][i][j])
                                                 : frag<CT>::mfma(fw[kk & 1][dd][i], fx[kk & 1][dd][j], acc[dd][i][j]);
-#endif
                         const int m = kk * PER_K0 + (dd * C::MT + i) * C::NT + j;  // MFMA index in the slab
                         if (kk + 1 < K0 && (m + 1) % STRIDE == 0 && m / STRIDE < C::L) {
                             issue_one(m / STRIDE);
@@ -458,7 +427,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
             }
         }
     }
-    KG_STAMP(2);
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // repeats of the last slab must land before LDS is released
 
     __syncthreads();  // every wave is done with the operand ring: LDS becomes the output tile
@@ -479,6 +447,41 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
         static_assert(RPP >= 32, "output pass");
         TY *const out = (TY *)smem;
         const int l32 = lane & 31, lq = lane >> 5;
+        // bias and activation act on the accumulators in place, before the tile is written out;
+        // the passes below then store them as they are
+        float st_scale = scale;
+        if (has_epi) {
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j) {
+                    const int mb = (wm * C::MT + i) * 32, nb = (wn * C::NT + j) * 32;
+                    // bs_last: the lane's row is one output feature; bs_first: element u of group eg
+                    // is output m0 + mb + 4*lq + 8*eg + u (x DD interleaved d_i)
+                    const size_t f0 = BS_LAST ? ((size_t)a_i * b + m0 + mb + l32) * d + d_i
+                                              : ((size_t)a_i * b + m0 + mb + 4 * lq) * DD;
+                    const float bl = BS_LAST ? epi_bias<TY>(ep, f0) : 0.f;
+                    (void)nb;
+#pragma unroll
+                    for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const float bv = BS_LAST ? bl : epi_bias<TY>(ep, f0 + (size_t)(8 * (e >> 2) + (e & 3)) * DD + dd);
+                            acc[dd][i][j][e] = fmaf(acc[dd][i][j][e], scale, bv);
+                        }
+                }
+            if (ep.act == KSMM_ACT_GELU) {
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+                    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                        for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = gelu_erf(acc[dd][i][j][e]);
+            }
+            st_scale = 1.f;
+        }
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
             if (pass > 0) __syncthreads();
@@ -494,19 +497,19 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
                     for (int eg = 0; eg < 4; ++eg) {
                         if constexpr (sizeof(TY) == 4) {
-                            float4_t v = {acc[0][i][j][4 * eg] * scale, acc[0][i][j][4 * eg + 1] * scale,
-                                          acc[0][i][j][4 * eg + 2] * scale, acc[0][i][j][4 * eg + 3] * scale};
+                            float4_t v = {acc[0][i][j][4 * eg] * st_scale, acc[0][i][j][4 * eg + 1] * st_scale,
+                                          acc[0][i][j][4 * eg + 2] * st_scale, acc[0][i][j][4 * eg + 3] * st_scale};
                             *(float4_t *)(dst + rcol + 8 * eg) = v;
                         } else if constexpr (DD == 1) {
-                            half4_t v = {(half_t)(acc[0][i][j][4 * eg] * scale), (half_t)(acc[0][i][j][4 * eg + 1] * scale),
-                                         (half_t)(acc[0][i][j][4 * eg + 2] * scale), (half_t)(acc[0][i][j][4 * eg + 3] * scale)};
+                            half4_t v = {(half_t)(acc[0][i][j][4 * eg] * st_scale), (half_t)(acc[0][i][j][4 * eg + 1] * st_scale),
+                                         (half_t)(acc[0][i][j][4 * eg + 2] * st_scale), (half_t)(acc[0][i][j][4 * eg + 3] * st_scale)};
                             *(half4_t *)(dst + rcol + 8 * eg) = v;
                         } else {
                             half8_t v;
 #pragma unroll
                             for (int u = 0; u < 4; ++u) {
-                                v[2 * u] = (half_t)(acc[0][i][j][4 * eg + u] * scale);
-                                v[2 * u + 1] = (half_t)(acc[DD - 1][i][j][4 * eg + u] * scale);
+                                v[2 * u] = (half_t)(acc[0][i][j][4 * eg + u] * st_scale);
+                                v[2 * u + 1] = (half_t)(acc[DD - 1][i][j][4 * eg + u] * st_scale);
                             }
                             *(half8_t *)(dst + (rcol + 8 * eg) * DD) = v;
                         }
@@ -531,7 +534,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
             }
         }
     }
-    KG_STAMP(3);
 }
 
 struct GemmInst {
@@ -673,10 +675,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (t.lds > 64 * 1024) {
-        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
     // L2 prefetch for the successor workgroup (bs_last): when the TM-tiles of an input tile can
     // cover it with PF lines per thread; distance = workgroups resident on an XCD (32 CUs)
@@ -688,8 +687,9 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         const int64_t in_l2 = 2 * (int64_t)p.c * t.tn * es * ((resident + m_tiles - 1) / m_tiles);
         if (lines <= (int64_t)GEMM_PF * t.threads && in_l2 <= (5 << 19)) pf_dist = resident;
     }
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i, &pf_dist};
+                    (void *)&p.c, (void *)&p.d, &ep, &m_tiles_i, &n_tiles_i, &blocks_i, &pf_dist};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

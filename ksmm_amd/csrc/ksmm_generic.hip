@@ -23,7 +23,7 @@ template <typename TX, typename TW, typename TY, bool BS_LAST>
 __global__ __launch_bounds__(256) void ks_generic_kernel(const TX *__restrict__ x,
                                                          const TW *__restrict__ w,
                                                          TY *__restrict__ y, int64_t batch, int a,
-                                                         int b, int c, int d, float scale)
+                                                         int b, int c, int d, Epi ep)
 {
     const int64_t in_size = (int64_t)a * c * d;
     const int64_t out_size = (int64_t)a * b * d;
@@ -47,11 +47,11 @@ __global__ __launch_bounds__(256) void ks_generic_kernel(const TX *__restrict__ 
         const TX *xp = x + ((int64_t)a_i * c * d + d_i) * batch + n;
         const int64_t xs = (int64_t)d * batch;
         for (int k = 0; k < c; ++k) acc += elem<TW>::load(wp + (int64_t)k * b) * elem<TX>::load(xp + k * xs);
-        elem<TY>::store(y + j * batch + n, acc * scale);
+        elem<TY>::store(y + j * batch + n, epi_finish(ep, acc, epi_bias<TY>(ep, (size_t)j)));
     } else {
         const TX *xp = x + n * in_size + (int64_t)a_i * c * d + d_i;
         for (int k = 0; k < c; ++k) acc += elem<TW>::load(wp + (int64_t)k * b) * elem<TX>::load(xp + (int64_t)k * d);
-        elem<TY>::store(y + n * out_size + j, acc * scale);
+        elem<TY>::store(y + n * out_size + j, epi_finish(ep, acc, epi_bias<TY>(ep, (size_t)j)));
     }
 }
 
@@ -100,7 +100,7 @@ template <> struct vec16<fp8_t> {
 template <typename TX, typename TW, typename TY, int BT>
 __global__ __launch_bounds__(256) void ks_small_bl_kernel(const TX *__restrict__ x, const TW *__restrict__ w,
                                                           TY *__restrict__ y, int64_t batch, int a, int b, int c,
-                                                          int d, float scale, int n_blocks, int b_chunks)
+                                                          int d, Epi ep, int n_blocks, int b_chunks)
 {
     constexpr int V = vec16<TX>::N;
     const int bc = blockIdx.x % b_chunks;
@@ -132,15 +132,18 @@ __global__ __launch_bounds__(256) void ks_small_bl_kernel(const TX *__restrict__
 #pragma unroll
     for (int j = 0; j < BT; ++j) {
         if (b0 + j >= b) break;
-        TY *yp = y + ((int64_t)(a_i * b + b0 + j) * d + d_i) * batch + n0;
+        const int64_t feature = (int64_t)(a_i * b + b0 + j) * d + d_i;
+        TY *yp = y + feature * batch + n0;
+        const float bv = epi_bias<TY>(ep, (size_t)feature);
         if constexpr (sizeof(TY) == 4) {
-            *(float4_t *)yp = float4_t{acc[j][0] * scale, acc[j][1] * scale, acc[j][2] * scale, acc[j][3] * scale};
+            *(float4_t *)yp = float4_t{epi_finish(ep, acc[j][0], bv), epi_finish(ep, acc[j][1], bv),
+                                       epi_finish(ep, acc[j][2], bv), epi_finish(ep, acc[j][3], bv)};
         } else {
 #pragma unroll
             for (int h = 0; h < V / 8; ++h) {
                 half8_t o;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = (half_t)(acc[j][8 * h + e] * scale);
+                for (int e = 0; e < 8; ++e) o[e] = (half_t)epi_finish(ep, acc[j][8 * h + e], bv);
                 *(half8_t *)(yp + 8 * h) = o;
             }
         }
@@ -151,7 +154,7 @@ template <typename TX, typename TW, typename TY>
 static void launch_small(const Problem &p, int64_t grid, int n_blocks, int b_chunks)
 {
     hipLaunchKernelGGL((ks_small_bl_kernel<TX, TW, TY, 8>), dim3((unsigned)grid), dim3(256), 0, p.stream,
-                       (const TX *)p.x, (const TW *)p.w, (TY *)p.y, p.batch, p.a, p.b, p.c, p.d, p.scale, n_blocks,
+                       (const TX *)p.x, (const TW *)p.w, (TY *)p.y, p.batch, p.a, p.b, p.c, p.d, epi_of(p), n_blocks,
                        b_chunks);
 }
 
@@ -161,11 +164,11 @@ static void launch_generic(const Problem &p, dim3 grid, dim3 block)
     if (p.bs_last)
         hipLaunchKernelGGL((ks_generic_kernel<TX, TW, TY, true>), grid, block, 0, p.stream,
                            (const TX *)p.x, (const TW *)p.w, (TY *)p.y, p.batch, p.a, p.b, p.c, p.d,
-                           p.scale);
+                           epi_of(p));
     else
         hipLaunchKernelGGL((ks_generic_kernel<TX, TW, TY, false>), grid, block, 0, p.stream,
                            (const TX *)p.x, (const TW *)p.w, (TY *)p.y, p.batch, p.a, p.b, p.c, p.d,
-                           p.scale);
+                           epi_of(p));
 }
 
 // variant 0: one thread per output; 1: the vector form (batch-size-last, batch a multiple of the

@@ -43,7 +43,7 @@ template <int BB, int CC, int DD, int TN, bool NT_STORE>
 __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a,
-                                                            int d, float scale, int wgs_per_a, int n_tiles)
+                                                            int d, Epi ep, int wgs_per_a, int n_tiles)
 {
     typedef RowCfg<BB, CC, DD, TN> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -69,6 +69,12 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
 #pragma unroll
             for (int mt = 0; mt < C::MT; ++mt) wreg[mt][ks] = wg[(4 * ks + q) * BB + 16 * mt + r];
     }
+    float bv[C::MT][4];  // bias of the outputs this lane holds: m = 16*mt + 4*q + i of d_i = d0 + dd
+#pragma unroll
+    for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * BB + 16 * mt + 4 * q + i) * d + d0 + dd);
 
     // element e of a tile row (e = k * DD + j) lives at k * d + j behind the group's origin
     const float *xg = x + (size_t)a_i * CC * d + d0;
@@ -128,7 +134,7 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = acc[mt][nt][i] * scale;
+                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -184,7 +190,7 @@ __device__ __forceinline__ half_t row_to_half(fp8_t v) { return fp8_to_half(v.bi
 template <typename TX, int BB, int CC, int DD, int TN>
 __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restrict__ x, const TX *__restrict__ w,
                                                               half_t *__restrict__ y, int batch, int a, int d,
-                                                              float scale, int wgs_per_a, int n_tiles)
+                                                              Epi ep, int wgs_per_a, int n_tiles)
 {
     typedef RowCfgH<TX, BB, CC, DD, TN> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -212,6 +218,12 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
 #pragma unroll
                 for (int j = 0; j < 4; ++j) wreg[mt][ks][j] = row_to_half(wg[(16 * ks + 4 * q + j) * BB + 16 * mt + r]);
     }
+    float bv[C::MT][4];  // bias of the outputs this lane holds: m = 16*mt + 4*q + i of d_i = d0 + dd
+#pragma unroll
+    for (int mt = 0; mt < C::MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            bv[mt][i] = epi_bias<half_t>(ep, ((size_t)a_i * BB + 16 * mt + 4 * q + i) * d + d0 + dd);
 
     const TX *xg = x + (size_t)a_i * CC * d + d0;
     half_t *yg = y + (size_t)a_i * BB * d + d0;
@@ -270,7 +282,7 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = (half_t)(acc[mt][nt][i] * scale);
+                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = (half_t)epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -351,19 +363,22 @@ const RowInst row_insts[] = {
     ROW_SET_16B(ROW_INST_Q),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
+constexpr int ROW_INST_BITS = 10, ROW_INST_ANY = (1 << ROW_INST_BITS) - 1;
+static_assert(N_ROW_INSTS < ROW_INST_ANY, "the variant's instance field must hold every index");
 
 }  // namespace
 
-// variant: bits 0-6 instance (0x7f: first that fits), bits 7.. workgroups per a_i (0: heuristic)
+// variant: bits 0-9 instance (all ones: first that fits), bits 10.. workgroups per a_i (0: heuristic)
 int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     if (p.bs_last || combo < 0 || combo > 2) return KSMM_ERR_BAD_ALGO;
-    const int want = variant < 0 ? 0x7f : (variant & 0x7f);
-    int64_t wgs = variant < 0 ? 0 : (variant >> 7);
+    const int want = variant < 0 ? ROW_INST_ANY : (variant & ROW_INST_ANY);
+    int64_t wgs = variant < 0 ? 0 : (variant >> ROW_INST_BITS);
+    if (want != ROW_INST_ANY && want >= N_ROW_INSTS) return KSMM_ERR_BAD_ALGO;
     int pick = -1;
     for (int i = 0; i < N_ROW_INSTS; ++i) {
-        if (want != 0x7f && want != i) continue;
+        if (want != ROW_INST_ANY && want != i) continue;
         const RowInst &t = row_insts[i];
         if (t.combo != combo || t.bb != p.b || t.cc != p.c) continue;
         // row segments start on 16-byte boundaries (output vectors: 4 floats / 8 halves)
@@ -372,7 +387,7 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         // all d blocks in one workgroup, or groups of dd whose runs keep the 16-byte alignment
         const bool grouped_ok = t.dd % t.vec == 0 && t.dd % ovec == 0 && p.d % t.dd == 0;
         const int run_bytes = t.dd * (combo == 0 ? 4 : 2);  // output run of a group
-        if (want != 0x7f) {
+        if (want != ROW_INST_ANY) {
             if (t.dd == p.d || grouped_ok) pick = i;
             break;
         }
@@ -411,13 +426,11 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (t.lds > 64 * 1024) {
-        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, wgs_i = (int)wgs, n_tiles_i = (int)n_tiles;
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
-                    (void *)&p.scale, &wgs_i, &n_tiles_i};
+                    &ep, &wgs_i, &n_tiles_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(64 * t.dd), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

@@ -29,17 +29,6 @@
 //  template_kernels_half.cuh:103-1092).
 #include "ksmm_mfma.h"
 
-#ifdef KSMM_PROFILE
-// Phase timestamps of wave 0 of every workgroup (standalone profiling builds only).
-__device__ unsigned long long ksmm_prof[512][64];
-#define KS_STAMP(slot)                                                                         \
-    do {                                                                                       \
-        if (threadIdx.x == 0 && blockIdx.x < 512 && (slot) < 64)                               \
-            ksmm_prof[blockIdx.x][(slot)] = ((slot) == 0 || (slot) == 3) ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); \
-    } while (0)
-#else
-#define KS_STAMP(slot) do { } while (0)
-#endif
 
 namespace ksmm {
 
@@ -82,7 +71,10 @@ struct StreamCfg {
     // overlap the weight staging area, so the first input tiles are requested before the
     // weights are staged
     static constexpr int HEAD_BYTES = ((W_BYTES > O_BYTES ? W_BYTES : O_BYTES) + 1023) / 1024 * 1024;
-    static constexpr int LDS_BYTES = HEAD_BYTES + ST * X_STAGE_BYTES;
+    // behind the stages: the bias of the block's BB outputs as floats (zeros without a bias)
+    static constexpr int BIAS_OFF = HEAD_BYTES + ST * X_STAGE_BYTES;
+    static constexpr int LDS_BYTES = BIAS_OFF + BB * 4;
+    static_assert(BB <= THREADS, "one bias value per thread");
     // vector-memory instructions issued after the loads of the tile being waited for
     static constexpr int N_SAFE = (ST - 1) * L;             // while fewer than ST-1 tiles were stored
     static constexpr int N_FULL = (ST - 1) * (L + S);       // steady state
@@ -146,8 +138,10 @@ template <typename CT, typename TW, typename TY, bool BS_LAST, int BB, int CC, i
 __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__restrict__ x,
                                                                 const TW *__restrict__ w,
                                                                 TY *__restrict__ y, int batch, int a,
-                                                                int d, float scale, int wgs_per_group)
+                                                                int d, Epi ep, int wgs_per_group)
 {
+    const float scale = ep.scale;
+    const bool has_epi = ep.bias != nullptr || ep.act != KSMM_ACT_NONE;  // uniform
     typedef StreamCfg<CT, TW, BS_LAST, BB, CC, TN, WM, WN, ST> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int g = blockIdx.x / wgs_per_group;  // a_i * d + d_i
@@ -163,7 +157,6 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
-    KS_STAMP(0);
 
     // ---- direct-to-LDS loads of one input tile ---------------------------------------------
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -216,9 +209,10 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
             const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
             r[i].load(wg + (size_t)(v / (BB / C::W_EPV)) * BB + (v % (BB / C::W_EPV)) * C::W_EPV);
         }
+        const float bias_v = tid < BB ? epi_bias<TY>(ep, ((size_t)a_i * BB + tid) * d + d_i) : 0.f;
 #pragma unroll
         for (int p = 0; p < ST - 1; ++p) issue(c_begin + min(p, n_iters - 1) * step, p);
-        KS_STAMP(1);
+        if (tid < BB) ((float *)(smem + C::BIAS_OFF))[tid] = bias_v;
 #pragma unroll
         for (int i = 0; i < W_PER_T; ++i) {
             const int v = min(tid + i * C::THREADS, C::W_VECS - 1);
@@ -233,7 +227,6 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
         for (int ks = 0; ks < C::KS; ++ks)
             wreg[i][ks] = frag<CT>::k_outer((const CT *)smem, C::LDW, (wm * C::MT + i) * 32, ks * C::KSTEP, lane);
     __syncthreads();  // the staging area becomes the output tile from here on
-    KS_STAMP(2);
 
 
     for (int it = 0; it < n_iters; ++it) {
@@ -245,7 +238,6 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
         else
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_SAFE));
         __syncthreads();  // tile `it` has landed for every wave
-        KS_STAMP(4 + 4 * it);
 
         const CT *xb = (const CT *)(smem + C::HEAD_BYTES + (it % ST) * C::X_STAGE_BYTES);
         float16_t acc[C::MT][C::NT];
@@ -271,7 +263,6 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
                 for (int j = 0; j < C::NT; ++j)
                     acc[i][j] = BS_LAST ? frag<CT>::mfma(fx[ks][j], wreg[i][ks], acc[i][j])
                                         : frag<CT>::mfma(wreg[i][ks], fx[ks][j], acc[i][j]);
-        KS_STAMP(5 + 4 * it);
         // ---- accumulators -> LDS output tile: out[lane index][4 consecutive row indices] ----
 #pragma unroll
         for (int i = 0; i < C::MT; ++i)
@@ -285,7 +276,18 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
 #pragma unroll
                 for (int eg = 0; eg < 4; ++eg) {
                     CT *dst = out + orow * C::O_LD + ocol0 + 8 * eg;
-                    if constexpr (sizeof(CT) == 2) {
+                    if (has_epi) {
+                        // output index of element u: bs_last the lane's row, bs_first 4 consecutive ones
+                        const float *bs = (const float *)(smem + C::BIAS_OFF);
+                        float v[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            v[u] = epi_finish(ep, acc[i][j][4 * eg + u], BS_LAST ? bs[orow] : bs[ocol0 + 8 * eg + u]);
+                        if constexpr (sizeof(CT) == 2)
+                            *(half4_t *)dst = half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                        else
+                            *(float4_t *)dst = float4_t{v[0], v[1], v[2], v[3]};
+                    } else if constexpr (sizeof(CT) == 2) {
                         half4_t hv = {(half_t)(acc[i][j][4 * eg] * scale), (half_t)(acc[i][j][4 * eg + 1] * scale),
                                       (half_t)(acc[i][j][4 * eg + 2] * scale), (half_t)(acc[i][j][4 * eg + 3] * scale)};
                         *(half4_t *)dst = hv;
@@ -297,7 +299,6 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
                 }
             }
         __syncthreads();
-        KS_STAMP(6 + 4 * it);
         // ---- LDS output tile -> global, 16 bytes per lane along the contiguous axis --------
 #pragma unroll
         for (int i = 0; i < C::S; ++i) {
@@ -317,9 +318,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
                 if (n < n_stop) __builtin_nontemporal_store(v, (uint4_t *)dst);
             }
         }
-        KS_STAMP(7 + 4 * it);
     }
-    KS_STAMP(3);
     // direct-to-LDS loads of the repeated last tile may still be in flight: they must land
     // before this workgroup's LDS is handed to another one
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -382,6 +381,8 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     const int want = variant < 0 ? 0x7f : (variant & 0x7f);
     int64_t wgs = variant < 0 ? 0 : (variant >> 7);
+    static_assert(N_STREAM_INSTS < 0x7f, "the variant's instance field must hold every index");
+    if (want != 0x7f && want >= N_STREAM_INSTS) return KSMM_ERR_BAD_ALGO;
     int pick = -1;
     for (int i = 0; i < N_STREAM_INSTS; ++i) {
         if (want != 0x7f && want != i) continue;
@@ -416,13 +417,11 @@ int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (t.lds > 64 * 1024) {
-        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, wgs_i = (int)wgs;
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
-                    (void *)&p.scale, &wgs_i};
+                    &ep, &wgs_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

@@ -59,7 +59,7 @@ template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int 
 __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restrict__ x,
                                                               const TW *__restrict__ w,
                                                               TY *__restrict__ y, int batch, int a,
-                                                              int b, int c, int d, float scale,
+                                                              int b, int c, int d, Epi ep,
                                                               int m_tiles, int n_tiles, int blocks)
 {
     typedef TileCfg<CT, TX, TW, TY, BS_LAST, TM, TN, TK, WM, WN> C;
@@ -228,16 +228,17 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
                     const int lrow = (wm * C::MT + i) * 32 + l32, rcol = (wn * C::NT + j) * 32 + 4 * lq;
                     if (lrow / RPP != pass) continue;  // uniform per wave (32-row tiles)
                     TY *dst = out + (lrow - pass * RPP) * RC + rcol;
+                    // the lane's output feature (clamped: rows behind b are not stored)
+                    const float bv = epi_bias<TY>(ep, ((size_t)a_i * b + min(m0 + lrow, b - 1)) * d + d_i);
 #pragma unroll
                     for (int eg = 0; eg < 4; ++eg) {
-                        if constexpr (sizeof(TY) == 4) {
-                            *(float4_t *)(dst + 8 * eg) = float4_t{acc[i][j][4 * eg] * scale, acc[i][j][4 * eg + 1] * scale,
-                                                                   acc[i][j][4 * eg + 2] * scale, acc[i][j][4 * eg + 3] * scale};
-                        } else {
-                            *(half4_t *)(dst + 8 * eg) =
-                                half4_t{(half_t)(acc[i][j][4 * eg] * scale), (half_t)(acc[i][j][4 * eg + 1] * scale),
-                                        (half_t)(acc[i][j][4 * eg + 2] * scale), (half_t)(acc[i][j][4 * eg + 3] * scale)};
-                        }
+                        float v[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] = epi_finish(ep, acc[i][j][4 * eg + u], bv);
+                        if constexpr (sizeof(TY) == 4)
+                            *(float4_t *)(dst + 8 * eg) = float4_t{v[0], v[1], v[2], v[3]};
+                        else
+                            *(half4_t *)(dst + 8 * eg) = half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
                     }
                 }
             __syncthreads();
@@ -256,10 +257,11 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_kernel(const TX *__restr
 #pragma unroll
             for (int j = 0; j < C::NT; ++j) {
                 const int mb = m0 + (wm * C::MT + i) * 32, nb = n0 + (wn * C::NT + j) * 32;
+                const float bv = epi_bias<TY>(ep, (size_t)a_i * b + min(mb + l32, b - 1));  // d == 1 in this layout
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int rr = 8 * (e >> 2) + 4 * lq + (e & 3);
-                    const float v = acc[i][j][e] * scale;
+                    const float v = epi_finish(ep, acc[i][j][e], bv);
                     const int n = nb + rr, m = mb + l32;
                     if (n < batch && (!RB || m < b)) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * b + m, v);
                 }
@@ -302,7 +304,7 @@ template <typename CT, typename TX, typename TW, typename TY, bool BS_LAST, int 
 __global__ __launch_bounds__(64 * WM * WN) void ks_ws_kernel(const TX *__restrict__ x,
                                                             const TW *__restrict__ w,
                                                             TY *__restrict__ y, int batch, int a,
-                                                            int d, float scale, int wgs_per_group,
+                                                            int d, Epi ep, int wgs_per_group,
                                                             int n_tiles)
 {
     typedef WsCfg<CT, TX, TW, TY, BS_LAST, BB, CC, TN, WM, WN> C;
@@ -420,14 +422,16 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_ws_kernel(const TX *__restric
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int rr = 8 * (e >> 2) + 4 * lq + (e & 3);
-                    const float v = acc[i][j][e] * scale;
                     if (BS_LAST) {
                         const int m = mb + rr, n = nb + l32;
-                        if (n < batch)
-                            elem<TY>::store(y + ((size_t)(a_i * BB + m) * d + d_i) * batch + n, v);
+                        const size_t feature = (size_t)(a_i * BB + m) * d + d_i;
+                        const float v = epi_finish(ep, acc[i][j][e], epi_bias<TY>(ep, feature));
+                        if (n < batch) elem<TY>::store(y + feature * batch + n, v);
                     } else {
                         const int n = nb + rr, m = mb + l32;
-                        if (n < batch) elem<TY>::store(y + (size_t)n * out_size + (size_t)a_i * BB + m, v);
+                        const size_t feature = (size_t)a_i * BB + m;  // d == 1 in this layout
+                        const float v = epi_finish(ep, acc[i][j][e], epi_bias<TY>(ep, feature));
+                        if (n < batch) elem<TY>::store(y + (size_t)n * out_size + feature, v);
                     }
                 }
             }
@@ -516,13 +520,11 @@ int ws_run(const Problem &p, int variant, int wgs_hint, bool launch, ksmm_tile *
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (t.lds > 64 * 1024) {
-        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, wgs_i = (int)wgs, n_tiles_i = (int)n_tiles;
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
-                    (void *)&p.scale, &wgs_i, &n_tiles_i};
+                    &ep, &wgs_i, &n_tiles_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
@@ -675,15 +677,11 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (t.lds > 64 * 1024) {
-        // opt in to more than 64 KB of dynamic LDS: a per-function attribute, set on every
-        // launch that needs it (idempotent, so there is no state to keep)
-        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (t.lds > 64 * 1024 && ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i};
+                    (void *)&p.c, (void *)&p.d, &ep, &m_tiles_i, &n_tiles_i, &blocks_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

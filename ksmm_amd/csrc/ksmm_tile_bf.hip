@@ -47,7 +47,7 @@ template <typename CT, typename TW, typename TY, int DD, int TM, int TN, int TK,
 __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__restrict__ x,
                                                                  const TW *__restrict__ w,
                                                                  TY *__restrict__ y, int batch, int a,
-                                                                 int b, int c, float scale,
+                                                                 int b, int c, Epi ep,
                                                                  int m_tiles, int n_tiles, int blocks)
 {
     typedef BfCfg<CT, TW, DD, TM, TN, TK, WM, WN> C;
@@ -174,12 +174,15 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
         for (int j = 0; j < C::NT; ++j) {
             const int m = m0 + (wm * C::MT + i) * 32 + l32;
             const int nb = n0 + (wn * C::NT + j) * 32;
+            float bv[DD];  // bias of the lane's DD adjacent outputs
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) bv[dd] = epi_bias<TY>(ep, ((size_t)a_i * b + m) * DD + dd);
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int n = nb + 8 * (e >> 2) + 4 * lq + (e & 3);
                 pack_t<TY, DD> o;
 #pragma unroll
-                for (int dd = 0; dd < DD; ++dd) o.e[dd] = (TY)(acc[dd][i][j][e] * scale);
+                for (int dd = 0; dd < DD; ++dd) o.e[dd] = (TY)epi_finish(ep, acc[dd][i][j][e], bv[dd]);
                 if (n < batch)
                     *(pack_t<TY, DD> *)(y + (size_t)n * out_size + ((size_t)a_i * b + m) * DD) = o;
             }
@@ -262,13 +265,11 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (t.lds > 64 * 1024) {
-        if (hipFuncSetAttribute(t.fn, hipFuncAttributeMaxDynamicSharedMemorySize, t.lds) != hipSuccess)
-            return KSMM_ERR_LAUNCH;
-    }
+    if (ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, (void *)&p.scale, &m_tiles_i, &n_tiles_i, &blocks_i};
+                    (void *)&p.c, &ep, &m_tiles_i, &n_tiles_i, &blocks_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

@@ -26,18 +26,6 @@
 
 #include "ksmm_common.h"
 
-#ifdef KSMM_PROFILE
-// Phase timestamps of wave 0 of every workgroup (standalone profiling builds only).
-__device__ unsigned long long ksmm_wprof[2048][40];
-#define KW_STAMP(slot)                                                                           \
-    do {                                                                                         \
-        if (threadIdx.x == 0 && blockIdx.x < 2048 && (slot) < 40)                                \
-            ksmm_wprof[blockIdx.x][(slot)] = ((slot) < 2) ? __builtin_amdgcn_s_memrealtime()     \
-                                                          : __builtin_amdgcn_s_memtime();        \
-    } while (0)
-#else
-#define KW_STAMP(slot) do { } while (0)
-#endif
 
 namespace ksmm {
 
@@ -115,13 +103,16 @@ template <> struct mfma16<8> {
 // fp32: v_mfma_f32_16x16x4_f32, VEC = 4 (16-byte loads and stores)
 // MT = b / 16, KS = c / 4.  Each wave iteration covers 64 batch columns.
 // ------------------------------------------------------------------------------------------
-template <int MT, int KS, int OCC, bool ROLL>
+// EPI: the instance that also adds a bias and/or applies the activation (kept apart so that
+// the plain instance's registers and loop body stay as they are).
+template <int MT, int KS, int OCC, bool ROLL, bool EPI>
 __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restrict__ x,
                                                      const float *__restrict__ w,
                                                      float *__restrict__ y, int batch, int a, int b,
-                                                     int c, int d, float scale, int n_slabs,
+                                                     int c, int d, Epi ep, int n_slabs,
                                                      int iters, int rr)
 {
+    const float scale = ep.scale;
     constexpr int VEC = 4, TN = 16 * VEC;
     const int lane = threadIdx.x & 63;
     const int q = lane >> 4, r = lane & 15;
@@ -130,8 +121,6 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     if (g >= a * d) return;
     const int slab = wave - g * n_slabs;
     const int a_i = g / d, d_i = g - a_i * d;
-    KW_STAMP(0);
-    KW_STAMP(2);
 
     // weights -> A operands, once per wave
     float areg[MT][KS];
@@ -141,12 +130,6 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = wg[(4 * ks + q) * b + 16 * mt + r];
-#ifdef KSMM_ABL_NOW
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = (float)(ks + mt + lane);
-#endif
     }
     // Addressing: uniform (scalar) row base + one 32-bit per-lane byte offset, so that the
     // loads and stores need no per-row vector address registers.  The host checks that the
@@ -176,11 +159,18 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
         for (int ks = 0; ks < KS; ++ks)
             xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + off);
     }
+    // bias of the output rows this lane holds (16*mt + 4*q + i), once per wave
+    float bv[EPI ? MT : 1][4];
+    if constexpr (EPI) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * b + 16 * mt + 4 * q + i) * d + d_i);
+    }
     // Everything issued so far (weights, first tile) is complete before the loop, so that the
     // waits inside the loop only ever count that loop's own loads and stores.
     __builtin_amdgcn_s_waitcnt(0);
-    KW_STAMP(3);
-    int kw_slot = 4;
     const int n_last = n_first + ((n_end - n_first - 1) / stride) * stride;  // first column of the last tile
     // FULL tiles store without a predicate, which keeps the loop body free of branches; a
     // ragged last tile (batch not a multiple of the tile) runs once more with the predicate.
@@ -194,25 +184,17 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
             for (int v = 0; v < VEC; ++v) acc[mt][v] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-#ifdef KSMM_ABL_NOMFMA
-#pragma unroll
-            for (int v = 0; v < VEC; ++v)
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt][v][ks & 3] += areg[mt][ks] + xc[ks][v];
-#else
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     acc[mt][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[mt][ks], xc[ks][v],
                                                                       acc[mt][v], 0, 0, 0);
-#endif
             if constexpr (ROLL) {
                 xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + next_off);
                 __builtin_amdgcn_sched_barrier(0);  // keep the refill between the MFMA groups
             }
         }
-        KW_STAMP(kw_slot);
         const int col = n0 + VEC * r;
         if (decltype(full)::value || col < batch) {
             const uint32_t off = y_lane + (uint32_t)col * 4u;
@@ -220,32 +202,33 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float4_t o = {acc[mt][0][i] * scale, acc[mt][1][i] * scale,
-                                  acc[mt][2][i] * scale, acc[mt][3][i] * scale};
+                    float4_t o;
+                    if constexpr (EPI)
+                        o = float4_t{epi_finish(ep, acc[mt][0][i], bv[mt][i]), epi_finish(ep, acc[mt][1][i], bv[mt][i]),
+                                     epi_finish(ep, acc[mt][2][i], bv[mt][i]), epi_finish(ep, acc[mt][3][i], bv[mt][i])};
+                    else
+                        o = float4_t{acc[mt][0][i] * scale, acc[mt][1][i] * scale, acc[mt][2][i] * scale,
+                                     acc[mt][3][i] * scale};
                     *(float4_t *)(yg + (size_t)(16 * mt + i) * row_stride * 4 + off) = o;
                 }
         }
-        KW_STAMP(kw_slot + 1);
-#ifdef KSMM_PROFILE
-        kw_slot += 2;
-#endif
     };
     int n0 = n_first;
     for (; n0 + TN <= n_end; n0 += stride) do_tile(n0, std::true_type{});
     if (n0 < n_end) do_tile(n0, std::false_type{});
-    KW_STAMP(1);
 }
 
 // ------------------------------------------------------------------------------------------
 // 16-bit MFMA path: x is fp16 or e4m3fn (decoded to fp16, exact), w is fp16 or e4m3fn,
 // y is fp16.  MT = b / 16, KS = c / (4 * KL).  Each wave iteration covers 16 * VEC columns.
 // ------------------------------------------------------------------------------------------
-template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC, bool ROLL>
+template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC, bool ROLL, bool EPI>
 __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ x,
                                                    const TW *__restrict__ w,
                                                    half_t *__restrict__ y, int batch, int a, int b,
-                                                   int c, int d, float scale, int n_slabs, int iters, int rr)
+                                                   int c, int d, Epi ep, int n_slabs, int iters, int rr)
 {
+    const float scale = ep.scale;
     constexpr int TN = 16 * VEC, KSTEP = 4 * KL;
     typedef typename hvec<KL>::type frag_t;
     const int lane = threadIdx.x & 63;
@@ -292,6 +275,14 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
             for (int jj = 0; jj < KL; ++jj)
                 io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + off),
                          raw[ks][jj]);
+    }
+    float bv[EPI ? MT : 1][4];  // bias of the output rows this lane holds
+    if constexpr (EPI) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                bv[mt][i] = epi_bias<half_t>(ep, ((size_t)a_i * b + 16 * mt + 4 * q + i) * d + d_i);
     }
     __builtin_amdgcn_s_waitcnt(0);
     const int n_last = n_first + ((n_end - n_first - 1) / stride) * stride;
@@ -344,7 +335,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
                     for (int v0 = 0; v0 < VEC; v0 += W) {
                         typename hvec<W>::type o;
 #pragma unroll
-                        for (int v = 0; v < W; ++v) o[v] = (half_t)(acc[mt][v0 + v][i] * scale);
+                        for (int v = 0; v < W; ++v) {
+                            if constexpr (EPI)
+                                o[v] = (half_t)epi_finish(ep, acc[mt][v0 + v][i], bv[mt][i]);
+                            else
+                                o[v] = (half_t)(acc[mt][v0 + v][i] * scale);
+                        }
                         *(typename hvec<W>::type *)(dst + v0) = o;
                     }
                 }
@@ -358,27 +354,31 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
 // ---- instance table ---------------------------------------------------------------------
 struct WaveInst {
     int b, c, vec, kl, occ;
-    const void *fn;       // several tiles per wave, rolling register pipeline
-    const void *fn_once;  // one tile per wave: nothing is reloaded
+    // [0]: several tiles per wave, rolling register pipeline; [1]: one tile per wave (nothing is
+    // reloaded); [2], [3]: the same with bias / activation
+    const void *fn[4];
 };
 
-typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, float, int, int, int);
+typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, Epi, int, int, int);
 template <typename TX, typename TW>
-using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int, float, int, int, int);
+using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int, Epi, int, int, int);
 
 // OCC_ = minimum waves per SIMD the register allocation must allow
+#define F32_FN(B_, C_, OCC_, ROLL_, EPI_) (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_, ROLL_, EPI_>
 #define F32_INST(B_, C_, OCC_) \
-    {B_, C_, 4, 1, OCC_, (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_, true>, \
-     (const void *)(f32_fn)ks_wave_bl_f32<B_ / 16, C_ / 4, OCC_, false>}
+    {B_, C_, 4, 1, OCC_, {F32_FN(B_, C_, OCC_, true, false), F32_FN(B_, C_, OCC_, false, false), \
+                          F32_FN(B_, C_, OCC_, true, true), F32_FN(B_, C_, OCC_, false, true)}}
 const WaveInst f32_insts[] = {
     F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
     F32_INST(16, 16, 4), F32_INST(32, 32, 3), F32_INST(48, 192, 1),
 };
 
-#define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_)                           \
-    {B_, C_, VEC_, KL_, OCC_,                                               \
-     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, true>, \
-     (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, false>}
+#define H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, ROLL_, EPI_) \
+    (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, ROLL_, EPI_>
+#define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_)                                                          \
+    {B_, C_, VEC_, KL_, OCC_,                                                                              \
+     {H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, true, false), H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false, false), \
+      H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, true, true), H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false, true)}}
 #define H_SET(TX_, TW_)                                                                      \
     H_INST(TX_, TW_, 64, 64, 8, 4, 2), H_INST(TX_, TW_, 64, 64, 8, 8, 2),                    \
         H_INST(TX_, TW_, 64, 64, 8, 8, 1), H_INST(TX_, TW_, 48, 48, 4, 4, 3),                \
@@ -427,8 +427,15 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
     const WaveInst &in = insts[pick];
-    // per-lane byte offsets (up to 4*KL rows of d*batch elements plus one row) must fit in 32 bits
-    if ((int64_t)(4 * in.kl + 1) * p.d * p.batch * 4 >= 0xffffffffLL) return KSMM_ERR_BAD_ALGO;
+    // The per-lane byte offsets must fit in 32 bits.  The largest ones formed are row 3*KL of a
+    // k-step plus one row of columns on the input side and row 12 of a 16-row output tile plus
+    // one row of columns on the output side (rows are d*batch elements apart).
+    {
+        const int64_t db = (int64_t)p.d * p.batch;
+        const int64_t x_max = (3 * in.kl * db + p.batch) * (int64_t)dtype_size(p.x_dtype);
+        const int64_t y_max = (12 * db + p.batch) * (int64_t)dtype_size(p.y_dtype);
+        if ((x_max > y_max ? x_max : y_max) >= 0xffffffffLL) return KSMM_ERR_BAD_ALGO;
+    }
     const int tn = 16 * in.vec;
     const int64_t n_tiles = (p.batch + tn - 1) / tn;
     // Tiles per wave.  Small blocks (16x16, 32x32) have little matrix work per byte: one tile
@@ -460,13 +467,14 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = blocks;
     }
     if (!launch) return KSMM_OK;
+    Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, nullptr, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, (void *)&p.d, (void *)&p.scale, nullptr, nullptr, &rr};
+                    (void *)&p.c, (void *)&p.d, &ep, nullptr, nullptr, &rr};
     int batch_i = (int)p.batch, n_slabs_i = (int)n_slabs;
     args[3] = &batch_i;
     args[9] = &n_slabs_i;
     args[10] = &iters;
-    const void *fn = iters == 1 ? in.fn_once : in.fn;
+    const void *fn = in.fn[(iters == 1 ? 1 : 0) + (p.bias || p.act ? 2 : 0)];
     hipError_t e = hipLaunchKernel(fn, dim3((unsigned)blocks), dim3(64 * wpb), args, 0, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

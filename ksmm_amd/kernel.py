@@ -39,12 +39,35 @@ def _stream_ptr(t):
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
+_ACTS = {None: _lib.ACT_NONE, "none": _lib.ACT_NONE, "gelu": _lib.ACT_GELU}
+
+
+def _epilogue(bias, act, out_size, out_dtype, device):
+    """ctypes epilogue (or None) for a bias vector of ``out_size`` values and an activation name."""
+    if act not in _ACTS:
+        raise ValueError("act must be one of %s" % sorted(k for k in _ACTS if k))
+    if bias is None and _ACTS[act] == _lib.ACT_NONE:
+        return None, None
+    ep = _lib.KsmmEpilogue()
+    ep.act = _ACTS[act]
+    keep = None
+    if bias is not None:
+        keep = bias.detach().reshape(-1)
+        assert keep.numel() == out_size, "bias must hold one value per output feature"
+        if keep.dtype != out_dtype or keep.device != device or not keep.is_contiguous():
+            keep = keep.to(device=device, dtype=out_dtype).contiguous()
+        ep.bias = keep.data_ptr()
+    else:
+        ep.bias = None
+    return ep, keep
+
+
 class Kernel:
     """Namespace with the reference's static-method calling convention (forward only)."""
 
     @staticmethod
     def forward(input, factor, bs_last, a, b, c, d, dtype=None, vsize=4, scale=1.0,
-                algo=_lib.ALGO_AUTO, variant=-1, out=None, workspace=None):
+                algo=_lib.ALGO_AUTO, variant=-1, out=None, workspace=None, bias=None, act=None):
         """y = K x for one factor.
 
         ``input``: (a*c*d, batch) if ``bs_last`` else (batch, a*c*d); ``factor``: kernel
@@ -53,7 +76,9 @@ class Kernel:
         are part of the tile table).  fp8 inputs/weights produce an fp16 result scaled by
         ``scale``.  Batch-size-first factors with d > 1 that have no kernel of their own run
         in batch-size-last layout between two transposes; the scratch tensor for that is
-        allocated here unless ``workspace`` (uint8, large enough) is passed.
+        allocated here unless ``workspace`` (uint8, large enough) is passed.  ``bias`` (one
+        value per output feature) and ``act`` ("gelu") are applied to the fp32 accumulator
+        inside the kernel: y = act(scale * acc + bias).
         """
         lib = _lib.load()
         _check_input(input, "input")
@@ -75,6 +100,9 @@ class Kernel:
         else:
             assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
         yd = dtype_code(out_dtype)
+        ep, _keep = _epilogue(bias, act, out_size, out_dtype, input.device)
+        if ep is not None and not (algo == _lib.ALGO_AUTO and variant == -1):
+            raise ValueError("bias/act go with the automatic kernel choice")
         with torch.cuda.device(input.device):
             if algo == _lib.ALGO_AUTO and variant == -1:
                 need = lib.ksmm_factor_workspace(batch, a, b, c, d, xd, wd, yd, int(bs_last))
@@ -82,9 +110,10 @@ class Kernel:
                     _lib.check(int(need))
                 if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
                     workspace = torch.empty(need, dtype=torch.uint8, device=input.device)
-                rc = lib.ksmm_factor_forward_ws(
+                rc = lib.ksmm_factor_forward_ep(
                     input.data_ptr(), factor.data_ptr(), out.data_ptr(), batch, a, b, c, d, xd, wd, yd,
-                    int(bs_last), float(scale), workspace.data_ptr() if need > 0 else None,
+                    int(bs_last), float(scale), ctypes.byref(ep) if ep is not None else None,
+                    workspace.data_ptr() if need > 0 else None,
                     workspace.numel() * workspace.element_size() if need > 0 else 0, _stream_ptr(input))
             else:
                 rc = lib.ksmm_factor_forward_algo(
@@ -94,8 +123,10 @@ class Kernel:
         return out
 
     @staticmethod
-    def chain_forward(input, factors, patterns, bs_last, scales=None, fuse=True, workspace=None):
-        """All factors of a KSLinear in one call (factor-chain launcher)."""
+    def chain_forward(input, factors, patterns, bs_last, scales=None, fuse=True, workspace=None,
+                      bias=None, act=None, out=None):
+        """All factors of a KSLinear in one call (factor-chain launcher).  ``bias``/``act`` are
+        applied by the last factor's kernel."""
         lib = _lib.load()
         _check_input(input, "input")
         n = len(factors)
@@ -118,8 +149,13 @@ class Kernel:
         batch = input.size(1 if bs_last else 0)
         out_dtype = torch.float16 if any_fp8 else input.dtype
         out_size = al * bl * dl
-        out = torch.empty((out_size, batch) if bs_last else (batch, out_size), dtype=out_dtype,
-                          device=input.device)
+        shape = (out_size, batch) if bs_last else (batch, out_size)
+        if out is None:
+            out = torch.empty(shape, dtype=out_dtype, device=input.device)
+        else:
+            assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
+        ep, _keep = _epilogue(bias, act, out_size, out_dtype, input.device)
+        ep_ref = ctypes.byref(ep) if ep is not None else None
         need = lib.ksmm_chain_workspace_layout(descs, n, batch, dtype_code(input.dtype),
                                                dtype_code(out_dtype), int(bs_last))
         if need < 0:
@@ -129,9 +165,9 @@ class Kernel:
         ws_ptr = workspace.data_ptr() if need > 0 else None
         ws_bytes = workspace.numel() * workspace.element_size() if need > 0 else 0
         with torch.cuda.device(input.device):
-            rc = lib.ksmm_chain_forward(descs, n, input.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes,
-                                        batch, dtype_code(input.dtype), dtype_code(out_dtype),
-                                        int(bs_last), int(bool(fuse)), _stream_ptr(input))
+            rc = lib.ksmm_chain_forward_ep(descs, n, input.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes,
+                                           batch, dtype_code(input.dtype), dtype_code(out_dtype),
+                                           int(bs_last), int(bool(fuse)), ep_ref, _stream_ptr(input))
         _lib.check(rc)
         return out
 

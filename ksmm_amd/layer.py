@@ -104,6 +104,13 @@ class KSLinear(nn.Module):
     """Drop-in for the reference's ``KSLinear`` on the ``kernel``/``dense``/``bmm``/``einsum``
     algorithms.
 
+    Beyond the reference's signature: ``fuse`` lets the chain launcher keep intermediates in
+    LDS where it has a kernel for the chain, and ``act='gelu'`` applies GELU (erf form) after
+    the bias, as the feed-forward block of the reference's ViT does between its two
+    projections (src/ksmm_py/model/vit.py:416-431).  With ``algo='kernel'`` the bias and the
+    activation are applied to the fp32 accumulator inside the last factor's kernel instead of
+    in a pass of their own (interface.py:457-466).
+
     ``dtype=torch.float8_e4m3fn`` (kernel only on the device): weights are quantised per
     tensor to e4m3fn with an fp32 scale, the input is quantised on entry unless it already
     is e4m3fn (then pass ``x_scale``), accumulation is fp32 and the result is fp16.  With
@@ -112,8 +119,10 @@ class KSLinear(nn.Module):
     """
 
     def __init__(self, patterns, weights=None, bias=True, algo="dense", dtype=torch.float16,
-                 bs_last=False, vsize=4, device="cpu", fuse=True):
+                 bs_last=False, vsize=4, device="cpu", fuse=True, act=None):
         super().__init__()
+        assert act in (None, "gelu"), "act must be None or 'gelu'"
+        self.act = act
         assert algo in ("sparse", "bsr") + ALGOS
         if algo in ("sparse", "bsr"):
             raise NotImplementedError("algo=%r is outside the kernel path provided here" % algo)
@@ -174,10 +183,10 @@ class KSLinear(nn.Module):
             scales[0] *= 1.0 if x_scale is None else float(x_scale)
         if self.fuse or self.num_mat > 1:
             return Kernel.chain_forward(x, list(self.factors), self.patterns, self.bs_last,
-                                        scales=scales, fuse=self.fuse)
+                                        scales=scales, fuse=self.fuse, bias=self.bias, act=self.act)
         a, b, c, d = self.patterns[0]
         return Kernel.forward(x, self.factors[0], self.bs_last, a, b, c, d, dtype=self.dtype,
-                              vsize=self.vsize, scale=scales[0])
+                              vsize=self.vsize, scale=scales[0], bias=self.bias, act=self.act)
 
     def forward_bs_first(self, output, x_scale=None):
         if self.algo == "kernel":
@@ -250,9 +259,13 @@ class KSLinear(nn.Module):
         return tensor.view(-1, tensor.size(-1))
 
     def post_process(self, tensor, output):
-        """interface.py:451-467: bias, then restore the caller's batch axes."""
-        if self.bias is not None:
-            output = output + self.bias
+        """interface.py:451-467: bias, then restore the caller's batch axes.  The kernel path
+        has added the bias (and applied the activation) in its last factor already."""
+        if self.algo != "kernel":
+            if self.bias is not None:
+                output = output + self.bias
+            if self.act == "gelu":
+                output = F.gelu(output)
         if self.bs_last:
             return output.view(self.out_size, *tensor.shape[1:])
         return output.view(*tensor.shape[:-1], self.out_size)

@@ -1,6 +1,6 @@
 """GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same
-seeded inputs.  Tolerances are relative Frobenius errors: fp32 1e-5, fp16 2e-3, fp8 5e-2
-(fp8: oracle on the dequantised operands)."""
+seeded inputs.  Tolerances are relative Frobenius errors: fp32 1e-5, fp16 2e-3, fp8 5e-3
+(fp8: oracle on the dequantised operands; the contract allows 5e-2)."""
 import numpy as np
 import pytest
 import torch
@@ -70,8 +70,11 @@ def test_factor_small(prec, bs_last, algo):
             err = O.rel_fro_error(y, z)
             assert y.shape == z.shape
             assert err <= TOL[prec], (pattern, batch, prec, bs_last, algo, err)
-    if ran == 0:
-        pytest.skip("family %s takes none of the small problems for %s" % (algo, prec))
+    print("test_factor_small", prec, bs_last, algo, "ran", ran, flush=True)
+    # a family that starts refusing the shapes it is built for must not pass silently
+    total = len(SMALL_PATTERNS) * len(BATCHES)
+    floor = {"generic": total, "auto": total, "wave": 20 if bs_last else 10, "tile": 20 if bs_last else 8}[algo]
+    assert ran >= floor, (prec, bs_last, algo, ran, floor)
 
 
 def test_gemm_kernels_forced():
@@ -495,3 +498,89 @@ def test_current_stream_is_used():
     s.synchronize()
     z = O.ks_apply_einsum(w4.double().numpy(), x.double().cpu().numpy(), True)
     assert O.rel_fro_error(y.cpu().numpy(), z) <= 1e-5
+
+
+def _gelu64(v):
+    from scipy.special import erf
+
+    return 0.5 * v * (1.0 + erf(v / np.sqrt(2.0)))
+
+
+EPILOGUE_CASES = [
+    # pattern, batch: chosen so that the automatic choice visits every kernel family
+    ((1, 48, 48, 16), 1040), ((6, 64, 64, 1), 520), ((2, 192, 192, 1), 520), ((1, 256, 64, 2), 520),
+    ((2, 3, 5, 4), 203), ((1, 96, 48, 2), 520), ((3, 16, 16, 4), 528), ((1, 192, 192, 16), 264),
+    ((2, 128, 70, 1), 520), ((1, 2, 4, 112), 64), ((2, 77, 64, 1), 520), ((1, 128, 128, 1), 1024),
+]
+
+
+@pytest.mark.parametrize("bs_last", [True, False])
+@pytest.mark.parametrize("prec", ["fp32", "fp16", "fp8"])
+def test_bias_and_gelu_in_the_kernel_epilogue(prec, bs_last):
+    """y = gelu(scale * K x + bias) computed inside the kernels against the float64 oracle
+    (bias and GELU applied to the oracle's product), bias only and bias + GELU; the families the
+    automatic choice used are collected and must include every one that exists for the layout."""
+    from ksmm_amd import Kernel, generate_factor
+    from ksmm_amd.kernel import query_tile
+
+    dt = TORCH_DTYPE[prec]
+    out_dt = torch.float16 if prec == "fp8" else dt
+    seen = set()
+    for pattern, batch in EPILOGUE_CASES:
+        a, b, c, d = pattern
+        (w4,) = seeded_weights([pattern], seed=61)
+        x = seeded_input(a * c * d, batch, bs_last, seed=62)
+        g = torch.Generator().manual_seed(63)
+        bias = (torch.rand(a * b * d, generator=g) - 0.5).to(out_dt)
+        wr, wq, ws = round_to(w4, prec)
+        xr, xq, xs = round_to(x, prec)
+        if prec == "fp8":
+            fac = generate_factor(a, b, c, d, "kernel", wq.to(torch.float32), dt, "cuda")
+            xin, scale = xq.cuda(), ws * xs
+        else:
+            fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+            xin, scale = x.to(dt).cuda(), 1.0
+        t = query_tile(batch, pattern, dt, None, bs_last)
+        seen.add((t["algo"], t["variant"] >> 24 if t["algo"] == 3 else (t["variant"] >= 1000 if t["algo"] == 2 else t["variant"])))
+        z = O.ks_apply_einsum(wr, xr, bs_last)
+        bz = bias.double().numpy()
+        zb = z + (bz[:, None] if bs_last else bz[None, :])
+        for act, want in ((None, zb), ("gelu", _gelu64(zb))):
+            y = Kernel.forward(xin, fac, bs_last, a, b, c, d, scale=scale, bias=bias.cuda(), act=act)
+            err = O.rel_fro_error(y.float().cpu().numpy(), want)
+            assert err <= TOL[prec], (pattern, batch, prec, bs_last, act, t, err)
+        # activation without a bias
+        y = Kernel.forward(xin, fac, bs_last, a, b, c, d, scale=scale, act="gelu")
+        assert O.rel_fro_error(y.float().cpu().numpy(), _gelu64(z)) <= TOL[prec], (pattern, prec, bs_last)
+    print("families seen", prec, bs_last, sorted(seen), flush=True)
+    assert len(seen) >= (4 if bs_last else 3), seen
+
+
+@pytest.mark.parametrize("prec", ["fp16", "fp8"])
+def test_kslinear_bias_gelu_chain(prec):
+    """KSLinear(bias=True, act='gelu', algo='kernel') against the same layer with algo='dense' (which
+    adds the bias and applies F.gelu in PyTorch) and against the float64 oracle: the two-factor
+    ViT up-projection shape in batch-size-first layout and the fused radix-16 chain."""
+    from ksmm_amd import KSLinear
+
+    for patterns, bs_last, batch in [([(12, 64, 64, 1), (1, 1536, 384, 2)], False, 392),
+                                     ([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], True, 1008),
+                                     ([(6, 64, 64, 1), (1, 768, 192, 2)], True, 520)]:
+        if prec == "fp8" and patterns[0][1] == 64 and not bs_last:
+            continue  # e4m3 batch-size-first with d = 2 runs on the transposed route: covered above
+        ws4 = seeded_weights(patterns, seed=71, bound=0.25 if patterns[0][1] == 16 else None)
+        n_in = patterns[0][0] * patterns[0][2] * patterns[0][3]
+        x = seeded_input(n_in, batch, bs_last, seed=72)
+        dt = TORCH_DTYPE[prec]
+        kk = KSLinear(patterns, weights=ws4, bias=True, algo="kernel", dtype=dt, bs_last=bs_last, device="cuda",
+                      act="gelu")
+        bz = kk.bias.detach().double().cpu().numpy().reshape(-1)
+        if prec == "fp8":
+            xr, xq, xs = round_to(x, prec)
+            y = kk(xq.cuda(), x_scale=xs).float().cpu().numpy()
+        else:
+            xr = round_to(x, prec)[0]
+            y = kk(x.to(dt).cuda()).float().cpu().numpy()
+        z = oracle_chain([round_to(w, prec)[0] for w in ws4], xr, bs_last)
+        want = _gelu64(z + (bz[:, None] if bs_last else bz[None, :]))
+        assert O.rel_fro_error(y, want) <= TOL[prec], (patterns, prec)

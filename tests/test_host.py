@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.ksmm_version() == 1
+    assert lib.ksmm_version() == 2
 
 
 def test_struct_layout_matches_header():
@@ -93,10 +93,19 @@ def test_chain_argument_checks(lib):
     assert need == 2 * ((24 * 100 * 4 + 255) // 256 * 256)
     assert lib.ksmm_chain_workspace(d, 1, 100, 0) == 0
     assert lib.ksmm_chain_workspace(d, 0, 100, 0) == -10
-    assert lib.ksmm_chain_forward(d, 2, 4096, 8192, None, 0, 100, 0, 0, 1, 1, None) == -9
+    # (fake, non-overlapping device addresses: every check below fails before anything is launched)
+    x, y, ws = 1 << 20, 2 << 20, 3 << 20
+    assert lib.ksmm_chain_forward(d, 2, x, y, None, 0, 100, 0, 0, 1, 1, None) == -9
+    # overlapping tensors are refused: y inside x, workspace inside y, misaligned workspace
+    assert lib.ksmm_chain_forward(d, 2, x, x + 256, ws, need, 100, 0, 0, 1, 1, None) == -11
+    assert lib.ksmm_chain_forward(d, 2, x, y, y + 512, need, 100, 0, 0, 1, 1, None) == -11
+    assert lib.ksmm_chain_forward(d, 2, x, y, ws + 4, need, 100, 0, 0, 1, 1, None) == -9
+    ep = _lib.KsmmEpilogue(None, 7)
+    import ctypes
+    assert lib.ksmm_chain_forward_ep(d, 2, x, y, ws, need, 100, 0, 0, 1, 1, ctypes.byref(ep), None) == -12
     d[1].c = 5  # 3*5*2 = 30 != 24
-    assert lib.ksmm_chain_forward(d, 2, 4096, 8192, 1 << 20, need, 100, 0, 0, 1, 1, None) == -8
-    assert lib.ksmm_chain_forward(d, 17, 4096, 8192, 1 << 20, need, 100, 0, 0, 1, 1, None) == -10
+    assert lib.ksmm_chain_forward(d, 2, x, y, ws, need, 100, 0, 0, 1, 1, None) == -8
+    assert lib.ksmm_chain_forward(d, 17, x, y, ws, need, 100, 0, 0, 1, 1, None) == -10
 
 
 def test_kslinear_constructor_contract():

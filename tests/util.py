@@ -6,7 +6,11 @@ import torch
 
 from oracle import ks_oracle as O
 
-TOL = {"fp32": 1e-5, "fp16": 2e-3, "fp8": 5e-2}  # relative Frobenius error vs the oracle
+# Relative Frobenius error vs the oracle.  The contract asks for 1e-5 / 2e-3 / 5e-2; the e4m3 path
+# multiplies exactly decoded operands with fp32 accumulation and rounds once to fp16, so its real
+# error is that of fp16 storage (a few 1e-4) and the tests hold it to 5e-3: one wrong output row
+# or column in a thousand would not pass.
+TOL = {"fp32": 1e-5, "fp16": 2e-3, "fp8": 5e-3}
 TORCH_DTYPE = {"fp32": torch.float32, "fp16": torch.float16, "fp8": torch.float8_e4m3fn}
 
 
