@@ -130,11 +130,21 @@ int ksmm_query_tile_variant(int64_t batch, int a, int b, int c, int d, int x_dty
 /* The measured table KSMM_ALGO_AUTO consults for batches of 8192 and more: the counterpart
  * of the reference's tuned `*.best` files and the if-chains generated from them
  * (src/ksmm_py/layer/kronecker_sparse/kernel.py:151-257).  Row i is
- * {a, b, c, d, combo, bs_last, algo, variant}, combo 0 = fp32, 1 = fp16, 2 = e4m3 -> fp16;
- * rows are sorted by (a, b, c, d, combo, bs_last).  Patterns without a row use the
- * heuristic order of kernel families. */
+ * {a, b, c, d, combo, bs_last, algo, instance id, parameter, variant}, combo 0 = fp32,
+ * 1 = fp16, 2 = e4m3 -> fp16; rows are sorted by (a, b, c, d, combo, bs_last).  The table
+ * stores (instance id, parameter): the id is a hash of the instance's own parameters, so rows
+ * keep naming the same kernel when instances are added or reordered; `variant` is what that
+ * resolves to in this build (-1: the instance no longer exists, the heuristics take over).
+ * Patterns without a row use the heuristic order of kernel families. */
 int ksmm_tuned_count(void);
-int ksmm_tuned_row(int index, int row[8]);
+int ksmm_tuned_row(int index, int row[10]);
+
+/* The stable name of the instance a (family, variant) pair selects for these element types
+ * and layout, and back.  The tuner writes ids; forcing a kernel still takes a variant. */
+int ksmm_variant_id(int algo, int variant, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                    uint32_t *id, int *param);
+int ksmm_variant_from_id(int algo, uint32_t id, int param, int x_dtype, int w_dtype, int y_dtype,
+                         int bs_last, int *variant);
 
 /* One factor.  Replaces `kernel.forward(input, factor, bs_last, a, b, c, d, dtype, vsize)`
  * (src/ksmm_py/layer/kronecker_sparse/kernel.cpp:25-45 -> kernel.cu:40-127); the caller

@@ -48,7 +48,11 @@ SIGNATURES = {
     "ksmm_query_tile_variant": (c_int, [c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                         c_int, ctypes.POINTER(KsmmTile)]),
     "ksmm_tuned_count": (c_int, []),
-    "ksmm_tuned_row": (c_int, [c_int, ctypes.POINTER(c_int * 8)]),
+    "ksmm_tuned_row": (c_int, [c_int, ctypes.POINTER(c_int * 10)]),
+    "ksmm_variant_id": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(ctypes.c_uint32),
+                                ctypes.POINTER(c_int)]),
+    "ksmm_variant_from_id": (c_int, [c_int, ctypes.c_uint32, c_int, c_int, c_int, c_int, c_int,
+                                     ctypes.POINTER(c_int)]),
     "ksmm_factor_forward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, ctypes.c_float, c_vp]),
     "ksmm_factor_forward_algo": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int,

@@ -70,13 +70,95 @@ int check_shape(int64_t batch, int a, int b, int c, int d, int xd, int wd, int y
 
 // Measured choices for known patterns (the counterpart of the reference's *.best tables,
 // src/ksmm_py/layer/kronecker_sparse/kernel.py:151-239): rows sorted by key.
+// A row names its kernel by family, stable instance id (inst_hash of the instance's parameters)
+// and a family-specific launch parameter, never by a position in an instance table.
 struct TunedRow {
-    int a, b, c, d, combo, bs_last, algo, variant;
+    int a, b, c, d, combo, bs_last, algo;
+    uint32_t id;
+    int param;
 };
 const TunedRow tuned_rows[] = {
 #include "ksmm_tuned.inc"
-    {0, 0, 0, 0, 0, 0, 0, 0},  // sentinel: keeps the array non-empty
+    {0, 0, 0, 0, 0, 0, 0, 0, 0},  // sentinel: keeps the array non-empty
 };
+
+// (family, variant) <-> (family, instance id, parameter).  Variant layouts are those of
+// ksmm_factor_forward_algo; `param` keeps what is not the instance: tiles per wave and tile
+// order (wave), workgroups per a_i (row kernels), workgroups per block (stream, weight-stationary).
+bool describe_variant(int algo, int variant, int combo, int bs_last, uint32_t *id, int *param)
+{
+    *param = 0;
+    if (algo == KSMM_ALGO_GENERIC) {
+        const int v[1] = {variant};
+        *id = inst_hash('X', v, 1);
+        return variant == 0 || variant == 1;
+    }
+    if (algo == KSMM_ALGO_WAVE) {
+        if (bs_last) {
+            if (variant < 0) return false;
+            *id = wave_inst_id(combo, variant & 0xff);
+            *param = variant >> 8;
+        } else {
+            if (variant < 1000) return false;
+            *id = rows_inst_id((variant - 1000) & 0x3ff);
+            *param = (variant - 1000) >> 10;
+        }
+        return *id != 0;
+    }
+    if (algo == KSMM_ALGO_TILE) {
+        if (variant < 0) return false;
+        const int sub = (variant >> 24) & 15, inst = variant & 0xff;
+        *param = (variant >> 8) & 0xffff;
+        switch (sub) {
+        case 0: *id = ktile_inst_id(inst); break;
+        case 1: *id = ws_inst_id(inst); break;
+        case 2: *id = stream_inst_id(inst); break;
+        case 3: *id = bf_inst_id(inst); break;
+        case 4: *id = gemm_inst_id(inst); break;
+        default: *id = 0;
+        }
+        return *id != 0;
+    }
+    return false;
+}
+
+template <typename F> int find_id(int n, uint32_t id, F id_of)
+{
+    for (int i = 0; i < n; ++i)
+        if (id_of(i) == id) return i;
+    return -1;
+}
+
+bool resolve_variant(int algo, uint32_t id, int param, int combo, int bs_last, int *variant)
+{
+    if (algo == KSMM_ALGO_GENERIC) {
+        for (int v = 0; v <= 1; ++v) {
+            const int a[1] = {v};
+            if (inst_hash('X', a, 1) == id) return *variant = v, true;
+        }
+        return false;
+    }
+    if (algo == KSMM_ALGO_WAVE) {
+        if (bs_last) {
+            const int i = find_id(wave_inst_count(combo), id, [&](int k) { return wave_inst_id(combo, k); });
+            return i >= 0 ? (*variant = i | (param << 8), true) : false;
+        }
+        const int i = find_id(rows_inst_count(), id, rows_inst_id);
+        return i >= 0 ? (*variant = 1000 + (i | (param << 10)), true) : false;
+    }
+    if (algo == KSMM_ALGO_TILE) {
+        int i, sub = 0;
+        if ((i = find_id(ktile_inst_count(), id, ktile_inst_id)) >= 0) sub = 0;
+        else if ((i = find_id(ws_inst_count(), id, ws_inst_id)) >= 0) sub = 1;
+        else if ((i = find_id(stream_inst_count(), id, stream_inst_id)) >= 0) sub = 2;
+        else if ((i = find_id(bf_inst_count(), id, bf_inst_id)) >= 0) sub = 3;
+        else if ((i = find_id(gemm_inst_count(), id, gemm_inst_id)) >= 0) sub = 4;
+        else return false;
+        *variant = (sub << 24) | ((param & 0xffff) << 8) | i;
+        return true;
+    }
+    return false;
+}
 constexpr int N_TUNED = (int)(sizeof(tuned_rows) / sizeof(TunedRow)) - 1;
 constexpr int64_t TUNED_MIN_BATCH = 8192;  // the table was measured at batch 25088
 
@@ -117,8 +199,10 @@ int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *ti
         // variant -3: heuristics only (what the tuner compares against)
         if (variant == -1 && p.batch >= TUNED_MIN_BATCH) {
             const TunedRow *row = tuned_lookup(p);
-            if (row && row->algo != KSMM_ALGO_AUTO) {
-                const int rc = dispatch(p, row->algo, row->variant, launch, tile);
+            int row_variant;
+            if (row && row->algo != KSMM_ALGO_AUTO &&
+                resolve_variant(row->algo, row->id, row->param, row->combo, row->bs_last, &row_variant)) {
+                const int rc = dispatch(p, row->algo, row_variant, launch, tile);
                 if (rc != KSMM_ERR_BAD_ALGO) return rc;
             }
         }
@@ -391,14 +475,34 @@ int ksmm_query_tile_variant(int64_t batch, int a, int b, int c, int d, int x_dty
 
 int ksmm_tuned_count(void) { return N_TUNED; }
 
-int ksmm_tuned_row(int index, int row[8])
+int ksmm_tuned_row(int index, int row[10])
 {
     if (!row) return KSMM_ERR_NULL_POINTER;
     if (index < 0 || index >= N_TUNED) return KSMM_ERR_BAD_ALGO;
     const TunedRow &r = tuned_rows[index];
-    const int v[8] = {r.a, r.b, r.c, r.d, r.combo, r.bs_last, r.algo, r.variant};
-    for (int i = 0; i < 8; ++i) row[i] = v[i];
+    int variant = -1;  // the row's instance is gone from the library: the heuristics serve the pattern
+    if (!resolve_variant(r.algo, r.id, r.param, r.combo, r.bs_last, &variant)) variant = -1;
+    const int v[10] = {r.a, r.b, r.c, r.d, r.combo, r.bs_last, r.algo, (int)r.id, r.param, variant};
+    for (int i = 0; i < 10; ++i) row[i] = v[i];
     return KSMM_OK;
+}
+
+int ksmm_variant_id(int algo, int variant, int x_dtype, int w_dtype, int y_dtype, int bs_last,
+                    uint32_t *id, int *param)
+{
+    if (!id || !param) return KSMM_ERR_NULL_POINTER;
+    const int combo = combo_of(x_dtype, w_dtype, y_dtype);
+    if (combo < 0) return KSMM_ERR_BAD_DTYPE;
+    return describe_variant(algo, variant, combo, bs_last ? 1 : 0, id, param) ? KSMM_OK : KSMM_ERR_BAD_ALGO;
+}
+
+int ksmm_variant_from_id(int algo, uint32_t id, int param, int x_dtype, int w_dtype, int y_dtype,
+                         int bs_last, int *variant)
+{
+    if (!variant) return KSMM_ERR_NULL_POINTER;
+    const int combo = combo_of(x_dtype, w_dtype, y_dtype);
+    if (combo < 0) return KSMM_ERR_BAD_DTYPE;
+    return resolve_variant(algo, id, param, combo, bs_last ? 1 : 0, variant) ? KSMM_OK : KSMM_ERR_BAD_ALGO;
 }
 
 int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batch, int a,

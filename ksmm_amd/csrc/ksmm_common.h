@@ -127,6 +127,35 @@ static inline int combo_of(int xd, int wd, int yd)
 // KSMM_OK or KSMM_ERR_LAUNCH.
 int ensure_dynamic_lds(const void *fn, int bytes);
 
+// Stable identity of a kernel instance: a hash of the numbers that describe it (family tag and
+// template parameters), not of its position in an instance table.  The measured table names
+// instances by these, so inserting or reordering instances cannot re-target its rows.
+static inline uint32_t inst_hash(uint32_t tag, const int *v, int n)
+{
+    uint32_t h = 2166136261u ^ tag;
+    for (int i = 0; i < n; ++i) {
+        h ^= (uint32_t)v[i];
+        h *= 16777619u;
+        h ^= h >> 15;
+    }
+    return (h & 0x7fffffffu) | 1u;  // positive and never 0
+}
+// per (sub-)family: number of instances and the id of instance i (0 when i is out of range)
+int wave_inst_count(int combo);
+uint32_t wave_inst_id(int combo, int i);
+int rows_inst_count();
+uint32_t rows_inst_id(int i);
+int stream_inst_count();
+uint32_t stream_inst_id(int i);
+int ktile_inst_count();
+uint32_t ktile_inst_id(int i);
+int ws_inst_count();
+uint32_t ws_inst_id(int i);
+int bf_inst_count();
+uint32_t bf_inst_id(int i);
+int gemm_inst_count();
+uint32_t gemm_inst_id(int i);
+
 // Launchers, one per kernel family.  Each fills `tile` and, when `launch` is true, enqueues
 // the kernel on p.stream.  They return KSMM_ERR_BAD_ALGO when the family (or the requested
 // variant) cannot run the problem.

@@ -539,6 +539,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 struct GemmInst {
     int combo, bs_last, dd, tm, tn, tk, threads, lds, epc;
     int ktail;  // takes c that is not a multiple of tk
+    int wm;     // waves along the TM side
     const void *fn;
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
@@ -547,7 +548,7 @@ struct GemmInst {
     {COMBO_, BL_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES,                                 \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::EPC,                                       \
-     KT_, (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_>}
+     KT_, WM_, (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_>}
 #define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
     GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
@@ -599,6 +600,9 @@ const GemmInst gemm_insts[] = {
     // e4m3, b a multiple of 64 only
     GEMM_INST_T(2, fp8_t, half_t, true, 1, 64, 256, 64, 1, 4, 3, 2),
     GEMM_INST_K(2, fp8_t, half_t, true, 1, 64, 256, 64, 1, 4, 3, 2, true),
+    // fp16, bs_first, d == 2: 16 waves on the 256 x 128 tile (4 per SIMD: more to issue from while
+    // others wait at the slab barrier)
+    GEMM_INST(1, half_t, false, 2, 256, 128, 32, 4, 4, 3),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
@@ -625,6 +629,17 @@ bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
 }
 
 }  // namespace
+
+int gemm_inst_count() { return N_GEMM_INSTS; }
+
+uint32_t gemm_inst_id(int i)
+{
+    if (i < 0 || i >= N_GEMM_INSTS) return 0;
+    const GemmInst &t = gemm_insts[i];
+    // threads and the LDS footprint stand for the wave grid and the ring depth
+    const int v[10] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm};
+    return inst_hash('G', v, 10);
+}
 
 // variant: index into the instance table; -1: first that fits with enough workgroups to fill
 // the chip (TM = 64 tiles only where nothing better exists); -4: the TM = 64 tiles, same

@@ -314,15 +314,16 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
 struct RowInst {
     int combo, bb, cc, dd, tn, lds;
     int vec;  // elements per 16-byte vector of the input
+    int nt;   // streaming (nontemporal) output stores
     const void *fn;
 };
 #define ROW_INST(BB_, CC_, DD_, TN_, NT_) \
-    {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, 4, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
+    {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, 4, NT_, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
 #define ROW_INST_H(BB_, CC_, DD_, TN_)                                                                      \
-    {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 8,                             \
+    {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 8, 1,                          \
      (const void *)ks_rows_bf_h_kernel<half_t, BB_, CC_, DD_, TN_>}
 #define ROW_INST_Q(BB_, CC_, DD_, TN_)                                                                      \
-    {2, BB_, CC_, DD_, TN_, RowCfgH<fp8_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 16,                             \
+    {2, BB_, CC_, DD_, TN_, RowCfgH<fp8_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 16, 1,                          \
      (const void *)ks_rows_bf_h_kernel<fp8_t, BB_, CC_, DD_, TN_>}
 #define ROW_SET_16(M) \
     M(48, 48, 16, 16), M(48, 48, 8, 32), M(48, 48, 4, 64), M(48, 48, 12, 32), \
@@ -367,6 +368,16 @@ constexpr int ROW_INST_BITS = 10, ROW_INST_ANY = (1 << ROW_INST_BITS) - 1;
 static_assert(N_ROW_INSTS < ROW_INST_ANY, "the variant's instance field must hold every index");
 
 }  // namespace
+
+int rows_inst_count() { return N_ROW_INSTS; }
+
+uint32_t rows_inst_id(int i)
+{
+    if (i < 0 || i >= N_ROW_INSTS) return 0;
+    const RowInst &t = row_insts[i];
+    const int v[6] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt};
+    return inst_hash('R', v, 6);
+}
 
 // variant: bits 0-9 instance (all ones: first that fits), bits 10.. workgroups per a_i (0: heuristic)
 int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)

@@ -327,12 +327,13 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_stream_kernel(const CT *__res
 struct StreamInst {
     int combo, bs_last, bb, cc, tn, threads, lds, epc;
     int per_cu;  // persistent workgroups per CU the heuristic launches; 0: only when forced
+    int wm;      // waves along the output side
     const void *fn;
 };
 #define STREAM_INST(COMBO_, CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_, PER_CU_)                     \
     {COMBO_, BL_, BB_, CC_, TN_, 64 * WM_ * WN_,                                                     \
      StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::LDS_BYTES,                               \
-     StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::EPC, PER_CU_,                            \
+     StreamCfg<CT_, TW_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>::EPC, PER_CU_, WM_,                       \
      (const void *)ks_stream_kernel<CT_, TW_, CT_, BL_, BB_, CC_, TN_, WM_, WN_, ST_>}
 // The first instance that fits a problem is the default; the order and the workgroups-per-CU
 // column come from sweeps at batch 25088 on MI355X.
@@ -374,6 +375,17 @@ bool stream_fits(const StreamInst &t, const Problem &p, int combo)
 }
 
 }  // namespace
+
+int stream_inst_count() { return N_STREAM_INSTS; }
+
+uint32_t stream_inst_id(int i)
+{
+    if (i < 0 || i >= N_STREAM_INSTS) return 0;
+    const StreamInst &t = stream_insts[i];
+    // threads and the LDS footprint stand for the wave grid and the number of stages
+    const int v[8] = {t.combo, t.bs_last, t.bb, t.cc, t.tn, t.threads, t.lds, t.wm};
+    return inst_hash('S', v, 8);
+}
 
 // variant: bits 0-6 instance (0x7f: first that fits), bits 7.. workgroups per group (0: heuristic)
 int stream_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)

@@ -441,12 +441,12 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_ws_kernel(const TX *__restric
 }
 
 struct WsInst {
-    int combo, bs_last, bb, cc, tn, threads, lds;
+    int combo, bs_last, bb, cc, tn, threads, lds, wm;
     const void *fn;
 };
 #define WS_INST(COMBO_, CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_)                            \
     {COMBO_, BL_, BB_, CC_, TN_, 64 * WM_ * WN_,                                                    \
-     WsCfg<CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_>::LDS_BYTES,                             \
+     WsCfg<CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_>::LDS_BYTES, WM_,                        \
      (const void *)ks_ws_kernel<CT_, TX_, TW_, TY_, BL_, BB_, CC_, TN_, WM_, WN_>}
 #define WS_SET_H(COMBO_, TX_, TW_, BL_)                                                             \
     WS_INST(COMBO_, half_t, TX_, TW_, half_t, BL_, 192, 192, 64, 2, 2),                             \
@@ -533,12 +533,13 @@ int ws_run(const Problem &p, int variant, int wgs_hint, bool launch, ksmm_tile *
 struct TileInst {
     int combo, bs_last, tm, tn, tk, threads, lds;
     int ragged_b;
+    int wm;
     const void *fn;
 };
 
 #define TILE_INST_R(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_, RB_)                    \
     {COMBO_, BL_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                    \
-     TileCfg<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, RB_,                      \
+     TileCfg<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, RB_, WM_,                 \
      (const void *)ks_tile_kernel<CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_, RB_>}
 #define TILE_INST(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_)                          \
     TILE_INST_R(COMBO_, CT_, TX_, TW_, TY_, BL_, TM_, TN_, TK_, WM_, WN_, false)
@@ -612,6 +613,26 @@ bool tile_fits(const TileInst &t, const Problem &p, int combo)
 }
 
 }  // namespace
+
+int ktile_inst_count() { return N_TILE_INSTS; }
+
+uint32_t ktile_inst_id(int i)
+{
+    if (i < 0 || i >= N_TILE_INSTS) return 0;
+    const TileInst &t = tile_insts[i];
+    const int v[8] = {t.combo, t.bs_last, t.tm, t.tn, t.tk, t.threads, t.ragged_b, t.wm};
+    return inst_hash('K', v, 8);
+}
+
+int ws_inst_count() { return N_WS_INSTS; }
+
+uint32_t ws_inst_id(int i)
+{
+    if (i < 0 || i >= N_WS_INSTS) return 0;
+    const WsInst &t = ws_insts[i];
+    const int v[7] = {t.combo, t.bs_last, t.bb, t.cc, t.tn, t.threads, t.wm};
+    return inst_hash('V', v, 7);
+}
 
 int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {

@@ -190,11 +190,11 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
 }
 
 struct BfInst {
-    int combo, dd, tm, tn, tk, threads, lds;
+    int combo, dd, tm, tn, tk, threads, lds, wm;
     const void *fn;
 };
 #define BF_INST(COMBO_, CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_)                                  \
-    {COMBO_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, BfCfg<CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, \
+    {COMBO_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, BfCfg<CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, WM_, \
      (const void *)ks_tile_bf_kernel<CT_, TW_, CT_, DD_, TM_, TN_, TK_, WM_, WN_>}
 #define BF_SET_H(COMBO_, TW_)                                                                    \
     BF_INST(COMBO_, half_t, TW_, 2, 128, 128, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 2, 256, 128, 32, 2, 2), \
@@ -224,6 +224,17 @@ bool bf_fits(const BfInst &t, const Problem &p, int combo)
 }
 
 }  // namespace
+
+int bf_inst_count() { return N_BF_INSTS; }
+
+uint32_t bf_inst_id(int i)
+{
+    if (i < 0 || i >= N_BF_INSTS) return 0;
+    const BfInst &t = bf_insts[i];
+    const int v[7] = {t.combo, t.dd, t.tm, t.tn, t.tk, t.threads, t.wm};
+    return inst_hash('B', v, 7);
+}
+
 
 // variant: index into the instance table (-1: heuristic)
 int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)

@@ -395,22 +395,43 @@ const WaveInst q_insts[] = {
     H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),  H_INST(fp8_t, fp8_t, 48, 192, 8, 8, 1),
 };
 
+const WaveInst *wave_table(int combo, int *n)
+{
+    switch (combo) {
+    case 0: *n = sizeof(f32_insts) / sizeof(WaveInst); return f32_insts;
+    case 1: *n = sizeof(h_insts) / sizeof(WaveInst); return h_insts;
+    case 2: *n = sizeof(q_insts) / sizeof(WaveInst); return q_insts;
+    case 3: *n = sizeof(hq_insts) / sizeof(WaveInst); return hq_insts;
+    default: *n = 0; return nullptr;
+    }
+}
+
 }  // namespace
+
+int wave_inst_count(int combo)
+{
+    int n;
+    wave_table(combo, &n);
+    return n;
+}
+
+uint32_t wave_inst_id(int combo, int i)
+{
+    int n;
+    const WaveInst *t = wave_table(combo, &n);
+    if (i < 0 || i >= n) return 0;
+    const int v[6] = {combo, t[i].b, t[i].c, t[i].vec, t[i].kl, t[i].occ};
+    return inst_hash('W', v, 6);
+}
 
 int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     // batch-size-first: the register-stationary row kernel (variants >= 1000), d > 1 only
     if (!p.bs_last) return rows_bf_run(p, variant >= 1000 ? variant - 1000 : -1, launch, tile);
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
-    const WaveInst *insts;
     int n_insts;
-    switch (combo) {
-    case 0: insts = f32_insts; n_insts = sizeof(f32_insts) / sizeof(WaveInst); break;
-    case 1: insts = h_insts; n_insts = sizeof(h_insts) / sizeof(WaveInst); break;
-    case 2: insts = q_insts; n_insts = sizeof(q_insts) / sizeof(WaveInst); break;
-    case 3: insts = hq_insts; n_insts = sizeof(hq_insts) / sizeof(WaveInst); break;
-    default: return KSMM_ERR_BAD_DTYPE;
-    }
+    const WaveInst *insts = wave_table(combo, &n_insts);
+    if (!insts) return KSMM_ERR_BAD_DTYPE;
     // vector loads along the batch axis need every row start aligned to the vector
     // variant: bits 0-7 instance index (0xff: first that fits), bits 8-15 wave iterations
     // (0: heuristic); -1: everything automatic

@@ -186,13 +186,40 @@ def query_tile(batch, pattern, x_dtype, w_dtype=None, bs_last=True, algo=_lib.AL
     return t.as_dict()
 
 
-def tuned_table():
+def tuned_table(full=False):
     """Rows (a, b, c, d, combo, bs_last, algo, variant) of the measured table compiled into the
-    library (combo 0 = fp32, 1 = fp16, 2 = e4m3 -> fp16)."""
+    library (combo 0 = fp32, 1 = fp16, 2 = e4m3 -> fp16); ``variant`` is what the row's stable
+    instance id resolves to in this build.  ``full=True`` returns the id and the parameter too:
+    (a, b, c, d, combo, bs_last, algo, id, param, variant)."""
     lib = _lib.load()
     rows = []
-    buf = (ctypes.c_int * 8)()
+    buf = (ctypes.c_int * 10)()
     for i in range(lib.ksmm_tuned_count()):
         _lib.check(lib.ksmm_tuned_row(i, ctypes.byref(buf)))
-        rows.append(tuple(buf))
+        r = tuple(buf)
+        rows.append(r if full else r[:7] + (r[9],))
     return rows
+
+
+_COMBO_DTYPES = {0: (_lib.KSMM_F32,) * 3, 1: (_lib.KSMM_F16,) * 3,
+                 2: (_lib.KSMM_FP8_E4M3, _lib.KSMM_FP8_E4M3, _lib.KSMM_F16),
+                 3: (_lib.KSMM_F16, _lib.KSMM_FP8_E4M3, _lib.KSMM_F16)}
+
+
+def variant_id(algo, variant, combo, bs_last):
+    """(instance id, parameter) of a forced (family, variant) for an element-type combination."""
+    lib = _lib.load()
+    iid, par = ctypes.c_uint32(), ctypes.c_int()
+    xd, wd, yd = _COMBO_DTYPES[combo]
+    _lib.check(lib.ksmm_variant_id(int(algo), int(variant), xd, wd, yd, int(bool(bs_last)), ctypes.byref(iid),
+                                   ctypes.byref(par)))
+    return iid.value, par.value
+
+
+def variant_from_id(algo, iid, param, combo, bs_last):
+    lib = _lib.load()
+    v = ctypes.c_int()
+    xd, wd, yd = _COMBO_DTYPES[combo]
+    _lib.check(lib.ksmm_variant_from_id(int(algo), int(iid), int(param), xd, wd, yd, int(bool(bs_last)),
+                                        ctypes.byref(v)))
+    return v.value

@@ -6,15 +6,20 @@ winners in ``*.best`` files that are turned into ``best_kernel_*`` if-chains
 (src/ksmm_py/layer/kronecker_sparse/kernel.py:151-257,
 kernel_bs_first_float.cuh:8-21).  Here the candidates are the instances of the kernel families
 (wave, stream, weight-stationary, GEMM, k-loop tiles), each forced through
-``ksmm_factor_forward_algo``; the fastest one per (pattern, element types, layout) goes into
-``ksmm_amd/csrc/ksmm_tuned.inc``, which is compiled into the library.
+``ksmm_factor_forward_algo`` and checked against the CPU oracle on sampled batch columns; the
+fastest one per (pattern, element types, layout) goes into ``ksmm_amd/csrc/ksmm_tuned.inc``,
+which is compiled into the library, named by its stable instance id.
 
     python -m ksmm_amd.tune --patterns FILE [--dtypes fp32,fp16,fp8] [--layouts last,first]
                             [--batch 25088] [--json OUT.json] [--merge A.json B.json ...]
-                            [--emit ksmm_amd/csrc/ksmm_tuned.inc]
+                            [--emit ksmm_amd/csrc/ksmm_tuned.inc] [--emit-best ksmm_amd/tuned]
 
 ``FILE`` holds one ``a,b,c,d`` per line (the reference's patterns.in has that format).  Several
 runs (e.g. one per element type) can be merged with ``--merge`` before ``--emit``.
+``--emit-best DIR`` writes ``kernel_bs_{first,last}_{float,half,fp8e4m3}.best``: one line per
+pattern, ``batch a b c d <kernel> ms std mse`` as in the reference's files of that name
+(kernel_bs_last_float.best:9), with the kernel named by family, instance id, parameter and
+tile shape instead of the CUDA hyper-parameters.
 """
 import argparse
 import json
@@ -23,6 +28,7 @@ import os
 import sys
 import time
 
+import numpy as np
 import torch
 
 DT = {"fp32": torch.float32, "fp16": torch.float16, "fp8": torch.float8_e4m3fn}
@@ -52,36 +58,54 @@ def _time_graph(fn, n_sets, steps):
     return t0.elapsed_time(t1) / 1e3 / steps
 
 
-def candidates(bs_last=True):
+def _count(algo, make_variant, combo, bs_last, limit=1024):
+    """Number of instances of a (sub-)family: indices are dense, the first one without an id ends it."""
+    from . import _lib
+    from .kernel import variant_id
+
+    n = 0
+    while n < limit:
+        try:
+            variant_id(algo, make_variant(n), combo, bs_last)
+        except _lib.KsmmError:
+            break
+        n += 1
+    return n
+
+
+def candidates(bs_last=True, combo=1):
     """(algo, variant) pairs worth trying; the library refuses those that do not fit."""
     out = []
     if bs_last:
-        for inst in range(16):                   # wave family: instance x tiles per wave
+        for inst in range(_count(2, lambda i: i, combo, True, 255)):   # wave family: instance x tiles per wave
             for it in (0, 1, 2, 4, 8):
                 out.append((2, inst | (it << 8)))
             for it in (0, 2, 4):                 # the same with tiles dealt round-robin
                 out.append((2, inst | (it << 8) | (1 << 16)))
     else:
-        for inst in range(150):                  # batch-size-first row kernel
+        for inst in range(_count(2, lambda i: 1000 + i, combo, False)):   # batch-size-first row kernel
             out.append((2, 1000 + inst))
-    for inst in range(28):                       # stream
-        out.append((3, (2 << 24) | inst))
-    for inst in range(40):                       # direct-to-LDS GEMM
-        out.append((3, (4 << 24) | inst))
-    for inst in range(64):                       # weight-stationary
-        out.append((3, (1 << 24) | inst))
-    for inst in range(16):                       # batch-size-first d > 1 tiles
-        out.append((3, (3 << 24) | inst))
+    for sub in (2, 4, 1, 3):                     # stream, direct-to-LDS GEMM, weight-stationary, d > 1 tiles
+        for inst in range(_count(3, lambda i, sub=sub: (sub << 24) | i, combo, bs_last, 255)):
+            out.append((3, (sub << 24) | inst))
     return out
 
 
-KLOOP = [(3, inst) for inst in range(80)]        # k-loop tiles: only when nothing else fits
+def kloop_candidates(combo, bs_last):
+    """k-loop tiles: only when nothing else fits."""
+    return [(3, inst) for inst in range(_count(3, lambda i: i, combo, bs_last, 255))]
+
+
+def _sample_cols(batch, n=48):
+    idx = set(range(min(4, batch))) | set(range(max(0, batch - 4), batch))
+    idx |= set(range(0, batch, max(1, batch // n)))
+    return np.array(sorted(idx))
 
 
 def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
     from . import Kernel, generate_factor, quantize_fp8
-
-    from .kernel import query_tile
+    from .kernel import query_tile, variant_id
+    from .layer import from_kernel_format_to_abcd
 
     a, b, c, d = pattern
     dt = DT[prec]
@@ -89,7 +113,7 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
     if query_tile(batch, pattern, dt, dt, bs_last)["algo"] == 1:
         # only the generic kernel (or the transposed route, which uses the batch-size-last
         # table) takes it in this layout: nothing to tune
-        return {"pattern": list(pattern), "prec": prec, "bs_last": bool(bs_last), "auto_us": None,
+        return {"pattern": list(pattern), "prec": prec, "bs_last": bool(bs_last), "batch": batch, "auto_us": None,
                 "best_us": None, "algo": 0, "variant": -1, "n_candidates": 0}
     es_in = 1 if prec == "fp8" else (2 if prec == "fp16" else 4)
     es_out = 2 if prec != "fp32" else 4
@@ -112,14 +136,29 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
     def run(algo, variant, j=0):
         return Kernel.forward(xs[j], fac, bs_last, a, b, c, d, out=ys[j], algo=algo, variant=variant)
 
+    # the checker: float64 oracle on sampled batch columns of the first input set (columns are
+    # independent), on the values the device holds (rounded / dequantised operands)
+    from oracle import ks_oracle as O
+
+    cols = _sample_cols(batch)
+    cols_t = torch.from_numpy(cols).cuda()
+    xsub = (xs[0][:, cols_t] if bs_last else xs[0][cols_t, :]).to(torch.float32).double().cpu().numpy()
+    wr = from_kernel_format_to_abcd(fac.to(torch.float32).cpu(), pattern).double().numpy()
+    z = O.ks_apply_einsum(wr, xsub, bs_last)
+    tol = {"fp32": 1e-5, "fp16": 2e-3, "fp8": 5e-3}[prec]
+
+    def check(y):
+        ysub = (y[:, cols_t] if bs_last else y[cols_t, :]).to(torch.float32).double().cpu().numpy()
+        return O.rel_fro_error(ysub, z), float(np.mean((ysub - z) ** 2))
+
+    combo = COMBO[prec]
     # what the heuristics pick, without the tuned table (variant -3)
-    ref = run(0, -3).clone()
+    auto_err, auto_mse = check(run(0, -3))
     t_auto = _time_graph(lambda j: run(0, -3, j), n_sets, 6)
     steps = int(min(40, max(6, 1.5e-3 / max(t_auto, 1e-6))))
     results = []
-    cands = candidates(bs_last)
     tried_any = False
-    for pool in (cands, KLOOP):
+    for pool in (candidates(bs_last, combo), kloop_candidates(combo, bs_last)):
         for algo, variant in pool:
             try:
                 y = run(algo, variant)
@@ -128,28 +167,46 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
                     continue
                 raise
             tried_any = True
-            err = ((y.float() - ref.float()).norm() / ref.float().norm().clamp_min(1e-30)).item()
-            if not err <= (1e-5 if prec == "fp32" else 5e-3):
+            err, mse = check(y)
+            if not err <= tol:
                 print("  MISMATCH", pattern, prec, bs_last, algo, hex(variant), err, flush=True)
                 continue
             t = _time_graph(lambda j: run(algo, variant, j), n_sets, steps)
-            results.append((t, algo, variant))
+            results.append((t, algo, variant, err, mse))
         if tried_any:
             break  # k-loop tiles only when no other family took the problem
     results.sort()
     best = results[0] if results else None
+    t_a, t_b = [t_auto], [best[0]] if best else []
     if best:
-        # confirm: heuristic choice and winner timed alternately, best of three each
-        t_a, t_b = [t_auto], [best[0]]
+        # confirm: heuristic choice and winner timed alternately, three runs each
         for _ in range(2):
             t_a.append(_time_graph(lambda j: run(0, -3, j), n_sets, steps))
             t_b.append(_time_graph(lambda j: run(best[1], best[2], j), n_sets, steps))
-        t_auto, best = min(t_a), (min(t_b), best[1], best[2])
-    # roofline bound of the factor: HBM at 8 TB/s against dense MFMA (fp32 157.3, fp16 2500 TFLOP/s)
-    bound = max(per_set / 8e12, 2.0 * batch * a * b * c * d / (157.3e12 if prec == "fp32" else 2.5e15))
-    return {"pattern": list(pattern), "prec": prec, "bs_last": bool(bs_last), "auto_us": t_auto * 1e6,
-            "bound_us": bound * 1e6, "best_us": best[0] * 1e6 if best else None, "algo": best[1] if best else 0,
-            "variant": best[2] if best else -1, "n_candidates": len(results)}
+    # roofline bound of the factor: HBM at 8 TB/s against the dense MFMA peak of the type the
+    # kernels multiply in (fp32 157.3, fp16 2516.6, e4m3 GEMM tiles 5033.2 TFLOP/s)
+    peak = {"fp32": 157.3e12, "fp16": 2516.6e12, "fp8": 5033.2e12}[prec]
+    bound = max(per_set / 8e12, 2.0 * batch * a * b * c * d / peak)
+    entry = {"pattern": list(pattern), "prec": prec, "bs_last": bool(bs_last), "batch": batch,
+             "auto_us": min(t_a) * 1e6, "auto_mean_us": float(np.mean(t_a)) * 1e6, "auto_std_us": float(np.std(t_a)) * 1e6,
+             "auto_rel_err": auto_err, "auto_mse": auto_mse, "auto_tile": query_tile(batch, pattern, dt, dt, bs_last, 0, -3),
+             "bound_us": bound * 1e6, "best_us": None, "algo": 0, "variant": -1, "n_candidates": len(results)}
+    if best:
+        iid, par = variant_id(best[1], best[2], combo, bs_last)
+        entry.update({"best_us": min(t_b) * 1e6, "best_mean_us": float(np.mean(t_b)) * 1e6,
+                      "best_std_us": float(np.std(t_b)) * 1e6, "algo": best[1], "variant": best[2], "id": iid,
+                      "param": par, "rel_err": best[3], "mse": best[4],
+                      "tile": query_tile(batch, pattern, dt, dt, bs_last, best[1], best[2])})
+    return entry
+
+
+def _entry_id(e):
+    """(instance id, parameter) of an entry; entries of older runs carry only the variant."""
+    if "id" in e:
+        return e["id"], e["param"]
+    from .kernel import variant_id
+
+    return variant_id(e["algo"], e["variant"], COMBO[e["prec"]], e["bs_last"])
 
 
 def emit(entries, path, batch):
@@ -161,18 +218,63 @@ def emit(entries, path, batch):
         if not e["best_us"] < 0.97 * e["auto_us"]:
             continue
         a, b, c, d = e["pattern"]
-        rows.append((a, b, c, d, COMBO[e["prec"]], 1 if e["bs_last"] else 0, e["algo"], e["variant"],
+        iid, par = _entry_id(e)
+        rows.append((a, b, c, d, COMBO[e["prec"]], 1 if e["bs_last"] else 0, e["algo"], iid, par,
                      e["best_us"], e["auto_us"]))
-    rows.sort(key=lambda r: (r[:6], r[8]))  # by key, fastest first
+    rows.sort(key=lambda r: (r[:6], r[9]))  # by key, fastest first
     rows = [r for i, r in enumerate(rows) if i == 0 or r[:6] != rows[i - 1][:6]]  # one row per key
     with open(path, "w") as f:
         f.write("// Generated by `python -m ksmm_amd.tune` on MI355X (gfx950) at batch %d: fastest measured\n" % batch)
-        f.write("// (family, variant) per (a, b, c, d, element-type combination, layout), kept only where it\n")
-        f.write("// beats the heuristic choice by more than 3 %.  Sorted by key for binary search.\n")
-        f.write("// {a, b, c, d, combo, bs_last, algo, variant},  // tuned us (heuristic us)\n")
+        f.write("// (family, instance id, parameter) per (a, b, c, d, element-type combination, layout), kept only\n")
+        f.write("// where it beats the heuristic choice by more than 3 %.  Sorted by key for binary search.\n")
+        f.write("// {a, b, c, d, combo, bs_last, algo, instance id, parameter},  // tuned us (heuristic us)\n")
         for r in rows:
-            f.write("{%d, %d, %d, %d, %d, %d, %d, %d},  // %.1f (%.1f)\n" % r)
+            f.write("{%d, %d, %d, %d, %d, %d, %d, %du, %d},  // %.1f (%.1f)\n" % r)
     return len(rows)
+
+
+BEST_NAME = {"fp32": "float", "fp16": "half", "fp8": "fp8e4m3"}
+FAMILY = {0: "auto", 1: "generic", 2: "wave", 3: "tile"}
+
+
+def emit_best(entries, directory):
+    """Per element type and layout, one ``*.best`` text file in the reference's spirit
+    (kernel_bs_last_float.best: ``batch a b c d TILEX TILEK TILEY TX TY VSIZE ms std mse``):
+    ``batch a b c d family instance_id parameter tile_m tile_n tile_k tile_d threads ms std mse``
+    for the fastest measured kernel, followed by the heuristic choice's ``ms std`` and the
+    factor's roofline floor.  Times are milliseconds per launch (mean and standard deviation of
+    the repeated HIP-graph timings), mse is the mean squared error against the float64 oracle on
+    the sampled batch columns."""
+    os.makedirs(directory, exist_ok=True)
+    written = {}
+    for prec in ("fp32", "fp16", "fp8"):
+        for bs_last in (False, True):
+            sel = [e for e in entries if e["prec"] == prec and e["bs_last"] == bs_last and e.get("auto_us")]
+            if not sel:
+                continue
+            sel.sort(key=lambda e: e["pattern"])
+            name = "kernel_bs_%s_%s.best" % ("last" if bs_last else "first", BEST_NAME[prec])
+            with open(os.path.join(directory, name), "w") as f:
+                f.write("# batch a b c d family instance_id parameter tile_m tile_n tile_k tile_d threads ms std mse "
+                        "| heuristic_ms heuristic_std roofline_floor_ms\n")
+                for e in sel:
+                    a, b, c, d = e["pattern"]
+                    use_best = e.get("best_us") is not None and e["algo"] != 0 and e["best_us"] <= e["auto_us"]
+                    if use_best and "id" in e:
+                        t = e.get("tile", {})
+                        fam, iid, par = FAMILY[e["algo"]], e["id"], e["param"]
+                        ms, std, mse = e.get("best_mean_us", e["best_us"]) / 1e3, e.get("best_std_us", 0.0) / 1e3, e.get("mse", float("nan"))
+                    else:
+                        t = e.get("auto_tile", {})
+                        fam, iid, par = FAMILY.get(t.get("algo", 0), "auto"), 0, 0
+                        ms, std, mse = e.get("auto_mean_us", e["auto_us"]) / 1e3, e.get("auto_std_us", 0.0) / 1e3, e.get("auto_mse", float("nan"))
+                    f.write("%d %d %d %d %d %s %d %d %d %d %d %d %d %.6f %.6f %.3e | %.6f %.6f %.6f\n" % (
+                        e.get("batch", 25088), a, b, c, d, fam, iid, par, t.get("tile_m", 0), t.get("tile_n", 0),
+                        t.get("tile_k", 0), t.get("tile_d", 0), t.get("threads", 0), ms, std, mse,
+                        e.get("auto_mean_us", e["auto_us"]) / 1e3, e.get("auto_std_us", 0.0) / 1e3,
+                        e.get("bound_us", 0.0) / 1e3))
+            written[name] = len(sel)
+    return written
 
 
 def main():
@@ -184,6 +286,7 @@ def main():
     ap.add_argument("--json")
     ap.add_argument("--merge", nargs="*", default=[])
     ap.add_argument("--emit")
+    ap.add_argument("--emit-best", help="directory for the kernel_bs_*_*.best text files")
     ap.add_argument("--shard", default="0/1", help="i/n: take every n-th pattern starting at i")
     ap.add_argument("--time-limit", type=float, default=1e9, help="stop (and save) after this many seconds")
     args = ap.parse_args()
@@ -229,6 +332,9 @@ def main():
     if args.emit:
         n = emit(entries, args.emit, args.batch)
         print("wrote %d rows to %s" % (n, args.emit))
+    if args.emit_best:
+        for name, n in emit_best(entries, args.emit_best).items():
+            print("wrote %d patterns to %s" % (n, os.path.join(args.emit_best, name)))
 
 
 if __name__ == "__main__":

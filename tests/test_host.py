@@ -5,6 +5,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -286,5 +287,138 @@ def test_tuner_emit_keeps_one_sorted_row_per_key_above_the_threshold(tmp_path):
     path = tmp_path / "t.inc"
     assert emit(entries, str(path), 25088) == 2
     rows = [l for l in path.read_text().splitlines() if l.startswith("{")]
-    assert rows[0].startswith("{1, 48, 48, 16, 0, 0, 2, 1000}")
-    assert rows[1].startswith("{2, 64, 64, 1, 1, 1, 3, 7}")
+    # rows name the kernel by stable instance id and parameter, not by table position
+    from ksmm_amd.kernel import variant_id
+
+    assert rows[0].startswith("{1, 48, 48, 16, 0, 0, 2, %du, %d}" % variant_id(2, 1000, 0, False))
+    assert rows[1].startswith("{2, 64, 64, 1, 1, 1, 3, %du, %d}" % variant_id(3, 7, 1, True))
+
+
+def test_tuner_best_files_have_the_reference_columns(tmp_path):
+    """ksmm_amd.tune.emit_best: `batch a b c d <kernel> ms std mse` per pattern, one file per
+    element type and layout, named like the reference's *.best files."""
+    from ksmm_amd.tune import emit_best
+
+    e = {"pattern": [1, 48, 48, 16], "prec": "fp32", "bs_last": True, "batch": 25088, "auto_us": 35.0,
+         "auto_mean_us": 35.5, "auto_std_us": 0.2, "auto_mse": 1e-14, "bound_us": 19.3, "best_us": 34.0,
+         "best_mean_us": 34.2, "best_std_us": 0.1, "algo": 2, "variant": 0x700, "id": 12345, "param": 7,
+         "mse": 2e-14, "tile": {"tile_m": 48, "tile_n": 64, "tile_k": 48, "tile_d": 1, "threads": 256},
+         "auto_tile": {"algo": 2, "tile_m": 48, "tile_n": 64, "tile_k": 48, "tile_d": 1, "threads": 256}}
+    slow = dict(e, pattern=[2, 64, 64, 1], best_us=40.0)      # the heuristic choice is the faster one
+    written = emit_best([e, slow], str(tmp_path))
+    assert written == {"kernel_bs_last_float.best": 2}
+    lines = (tmp_path / "kernel_bs_last_float.best").read_text().splitlines()
+    assert lines[0].startswith("# batch a b c d family instance_id parameter")
+    f = lines[1].split()
+    assert f[:8] == ["25088", "1", "48", "48", "16", "wave", "12345", "7"]
+    assert float(f[13]) == pytest.approx(0.0342) and float(f[14]) == pytest.approx(0.0001) and float(f[15]) == 2e-14
+    g = lines[2].split()
+    assert g[:8] == ["25088", "2", "64", "64", "1", "wave", "0", "0"] and float(g[13]) == pytest.approx(0.0355)
+
+
+def test_instance_ids_are_unique_and_round_trip(lib):
+    """Every instance of every family has its own id inside the set a table row is resolved in
+    (family x element types x layout), and (id, parameter) -> variant -> (id, parameter) is the
+    identity; every row of the compiled table still names an instance of this build."""
+    from ksmm_amd import _lib
+    from ksmm_amd.kernel import tuned_table, variant_from_id, variant_id
+    from ksmm_amd.tune import candidates, kloop_candidates
+
+    for combo in (0, 1, 2, 3):
+        for bs_last in (True, False):
+            seen = {}
+            for algo, variant in candidates(bs_last, combo) + kloop_candidates(combo, bs_last) + [(1, 0), (1, 1)]:
+                iid, par = variant_id(algo, variant, combo, bs_last)
+                assert variant_from_id(algo, iid, par, combo, bs_last) == variant, (combo, bs_last, algo, hex(variant))
+                key = (algo, iid)
+                inst = variant & 0xff if algo != 2 or bs_last else (variant - 1000) & 0x3ff
+                sub = (variant >> 24) if algo == 3 else 0
+                assert seen.setdefault(key, (sub, inst)) == (sub, inst), ("id collision", combo, bs_last, key)
+    rows = tuned_table(full=True)
+    assert len(rows) >= 700
+    assert all(r[9] >= 0 for r in rows), [r for r in rows if r[9] < 0][:3]
+    with pytest.raises(_lib.KsmmError):
+        variant_from_id(3, 12345, 0, 1, True)
+
+
+def test_kernel_format_converters_match_oracle():
+    """from_kernel_format_to_dense / from_bmm_format_to_dense / from_abcd_to_dense on asymmetric
+    patterns against the oracle's dense form (interface.py:75-113)."""
+    from ksmm_amd.layer import (from_abcd_to_dense, from_bmm_format_to_dense, from_kernel_format_to_abcd,
+                                from_kernel_format_to_dense, generate_factor)
+
+    for pattern in [(2, 3, 5, 4), (3, 2, 2, 1), (1, 4, 3, 2), (2, 6, 4, 3)]:
+        a, b, c, d = pattern
+        w4 = torch.arange(a * b * c * d, dtype=torch.float64).reshape(a, b, c, d) + 1
+        dense = O.ks_dense(w4.numpy())
+        fk = generate_factor(a, b, c, d, "kernel", w4, torch.float64, "cpu")
+        assert fk.shape == (a * d * c, b)
+        assert torch.equal(from_kernel_format_to_abcd(fk, pattern), w4)
+        assert np.array_equal(from_kernel_format_to_dense(fk, pattern).numpy(), dense)
+        fb = generate_factor(a, b, c, d, "bmm", w4, torch.float64, "cpu")
+        assert np.array_equal(from_bmm_format_to_dense(fb, pattern).numpy(), dense)
+        assert np.array_equal(from_abcd_to_dense(w4).numpy(), dense)
+
+
+def test_get_dense_product_of_a_kernel_format_layer_on_cpu_tensors():
+    """get_dense_product() reads the kernel-format parameters: build the layer's parameters by
+    hand (algo='kernel' itself needs a device) and compare with the oracle's chain product."""
+    from ksmm_amd import KSLinear, generate_factor
+
+    patterns = [(2, 3, 5, 4), (3, 6, 4, 2)]
+    ws4 = seeded_weights(patterns, seed=9)
+    ksl = KSLinear(patterns, weights=ws4, bias=False, algo="einsum", dtype=torch.float64)
+    # swap in kernel-format storage: the dense product must not change
+    want = O.chain_dense([w.double().numpy() for w in ws4])
+    assert np.allclose(ksl.get_dense_product().numpy(), want, rtol=0, atol=1e-12)
+    ksl.algo = "kernel"
+    for i, (p, w) in enumerate(zip(patterns, ws4)):
+        ksl.factors[i] = torch.nn.Parameter(generate_factor(*p, "kernel", w, torch.float64, "cpu"))
+    assert np.allclose(ksl.get_dense_product().numpy(), want, rtol=0, atol=1e-12)
+
+
+def test_wave_family_refuses_offsets_beyond_32_bits(lib):
+    """The wave kernels address rows with 32-bit per-lane byte offsets; the largest one formed
+    on the output side is (12*d*B + B) elements.  (1,16,16,4096) fp32 at B = 25088 passes the
+    shape check but would wrap: the family must refuse it (another family takes it)."""
+    from ksmm_amd.kernel import query_tile
+    from ksmm_amd import _lib
+
+    assert lib.ksmm_validate(25088, 1, 16, 16, 4096, 0, 0, 0, 1) == 0
+    with pytest.raises(_lib.KsmmError) as e:
+        query_tile(25088, (1, 16, 16, 4096), torch.float32, None, True, algo=_lib.ALGO_WAVE)
+    assert e.value.status == -6
+    assert query_tile(25088, (1, 16, 16, 4096), torch.float32, None, True)["algo"] != _lib.ALGO_WAVE
+    # just below the limit the family still takes the shape: 12*d*B*4 + 4*B < 2^32
+    assert query_tile(25088, (1, 16, 16, 3500), torch.float32, None, True, algo=_lib.ALGO_WAVE)["algo"] == 2
+    # 16-bit outputs: 24*d*B + 2*B bytes stays below 2^32 for every shape the 2^31-element limit lets in
+    assert query_tile(25088, (1, 16, 16, 5300), torch.float16, None, True, algo=_lib.ALGO_WAVE)["algo"] == 2
+
+
+def test_row_kernel_variants_round_trip(lib):
+    """What ksmm_query_tile reports for the batch-size-first row kernels can be forced back to
+    the same tile, for every element type (the instance field holds every index)."""
+    from ksmm_amd.kernel import query_tile
+    from ksmm_amd import _lib
+
+    seen = set()
+    for dt in (torch.float32, torch.float16, torch.float8_e4m3fn):
+        for pattern in [(1, 48, 48, 8), (1, 48, 48, 16), (2, 64, 64, 4), (1, 96, 96, 4), (1, 192, 48, 3),
+                        (1, 48, 192, 4), (1, 64, 64, 16), (1, 48, 48, 2)]:
+            t = query_tile(25088, pattern, dt, None, False, algo=_lib.ALGO_WAVE)
+            assert t["variant"] >= 1000
+            again = query_tile(25088, pattern, dt, None, False, algo=_lib.ALGO_WAVE, variant=t["variant"])
+            assert again == t, (dt, pattern, t, again)
+            seen.add(t["variant"] - 1000)
+    assert max(seen) >= 128  # instances beyond the old 7-bit field are reachable
+    # an index outside the table is refused, not aliased to another instance
+    with pytest.raises(_lib.KsmmError):
+        query_tile(25088, (1, 48, 48, 8), torch.float32, None, False, algo=_lib.ALGO_WAVE, variant=1000 + 1000)
+
+
+def test_unaligned_tensors_are_refused_by_forced_families(lib):
+    """Pointer checks happen before any launch: a forced vector family refuses tensors that do
+    not start on a 16-byte boundary (the automatic choice would run the scalar kernel)."""
+    f = lib.ksmm_factor_forward_algo
+    assert f(4096 + 4, 1 << 20, 2 << 20, 64, 1, 16, 16, 1, 0, 0, 0, 1, 1.0, 2, -1, None) == -6
+    assert f(4096, (1 << 20) + 8, 2 << 20, 64, 1, 16, 16, 1, 0, 0, 0, 1, 1.0, 3, -1, None) == -6

@@ -209,3 +209,43 @@ def test_torch_bmm_restatement_matches():
             wb = torch.from_numpy(O.pack_bmm_format(w4))
             y = O.torch_bmm_forward(wb, torch.from_numpy(xin), p, bs_last).numpy()
             np.testing.assert_array_equal(y, O.ks_apply_loops(w4, xin, bs_last))
+
+
+def test_rel_fro_error_closed_forms():
+    """The metric every parity assertion rests on, on values that can be worked out by hand."""
+    z = np.array([[3.0, 4.0], [0.0, 0.0]])                 # ||z|| = 5
+    assert O.rel_fro_error(z, z) == 0.0
+    assert O.rel_fro_error(z + np.array([[0.0, 0.0], [0.3, 0.4]]), z) == pytest.approx(0.1, rel=1e-12)
+    assert O.rel_fro_error(1.01 * z, z) == pytest.approx(0.01, rel=1e-9)      # relative: scale-free
+    assert O.rel_fro_error(np.zeros_like(z), z) == pytest.approx(1.0, rel=1e-12)
+    # not symmetric: the second argument is the reference
+    assert O.rel_fro_error(z, 2 * z) == pytest.approx(0.5, rel=1e-12)
+    assert O.rel_fro_error(2 * z, z) == pytest.approx(1.0, rel=1e-12)
+
+
+@pytest.mark.parametrize("tol_name", ["fp32", "fp16", "fp8"])
+def test_checker_fails_on_plausible_mistakes(tol_name):
+    """Negative controls: the mistakes a kernel is likely to make must exceed every tolerance
+    class, i.e. the parity tests can fail.  One swapped pair of weight blocks, one transposed
+    block, one wrong d index, one dropped k term, one stale output row."""
+    from tests.util import TOL
+
+    tol = TOL[tol_name]
+    pattern = (2, 48, 48, 16)
+    a, b, c, d = pattern
+    w4, x = _rand(pattern, 64, seed=5)
+    z = O.ks_apply_einsum(w4, x, True)
+    bad = {}
+    w = w4.copy(); w[[0, 1]] = w[[1, 0]]; bad["swapped a blocks"] = O.ks_apply_einsum(w, x, True)
+    w = w4.copy(); w[0, :, :, 3] = w4[0, :, :, 3].T; bad["one transposed block"] = O.ks_apply_einsum(w, x, True)
+    w = w4.copy(); w[:, :, :, 5] = w4[:, :, :, 6]; bad["wrong d index"] = O.ks_apply_einsum(w, x, True)
+    w = w4.copy(); w[:, :, c - 1, :] = 0; bad["dropped last k term"] = O.ks_apply_einsum(w, x, True)
+    y = z.copy(); y[17] = 0; bad["one of 1536 output rows missing"] = y
+    y = z.copy(); y[:, 63] = z[:, 62]; bad["one of 64 columns stale"] = y
+    for name, y in bad.items():
+        assert O.rel_fro_error(y, z) > tol, (name, O.rel_fro_error(y, z), tol)
+    # and rounding of the size the storage types produce stays inside
+    noise = {"fp32": 2.0 ** -24, "fp16": 2.0 ** -11, "fp8": 2.0 ** -11}[tol_name]
+    rng = np.random.default_rng(0)
+    y = z * (1 + noise * rng.uniform(-1, 1, z.shape))
+    assert O.rel_fro_error(y, z) <= tol
