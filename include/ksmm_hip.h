@@ -23,7 +23,8 @@
  * type only.  Workspaces must be 16-byte aligned.
  *
  * The library never allocates device memory and keeps no caller-visible mutable state (it
- * only remembers which kernels had their LDS limit raised).  All launches go to the stream the caller passes (a
+ * remembers which kernels had their LDS limit raised, and ksmm_chain_forward_static owns one
+ * fixed device buffer per GPU).  All launches go to the stream the caller passes (a
  * hipStream_t cast to void*; NULL is the legacy default stream).  Every entry point returns
  * KSMM_OK or a negative error code; ksmm_strerror() names it.  Only ksmm_factor_forward*,
  * ksmm_chain_forward* and ksmm_factor_backward* touch the GPU.
@@ -216,6 +217,20 @@ int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const 
                           void *workspace, int64_t workspace_bytes, int64_t batch, int x_dtype,
                           int y_dtype, int bs_last, int fuse, const ksmm_epilogue *epilogue,
                           void *stream);
+
+/* ksmm_chain_forward_ep for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the ping-pong intermediates
+ * and the transposed-route buffers live in a fixed device array inside the library,
+ * ksmm_static_scratch_bytes() = 32 MiB per GPU, instead of a caller's workspace.  It has no
+ * counterpart in the reference (whose Python loop lets torch allocate every intermediate,
+ * interface.py:269-291).  Chains whose ksmm_chain_workspace_layout() exceeds the array return
+ * KSMM_ERR_WORKSPACE.  Allocates nothing and frees nothing.  All calls on one GPU share the
+ * array (every intermediate is fully written before it is read, so nothing has to be cleared
+ * between calls): calls that overlap in time on one GPU race. */
+int64_t ksmm_static_scratch_bytes(void);
+int ksmm_chain_forward_static(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
+                              int64_t batch, int x_dtype, int y_dtype, int bs_last, int fuse,
+                              const ksmm_epilogue *epilogue, void *stream);
 
 #ifdef __cplusplus
 }

@@ -40,6 +40,12 @@ int ensure_dynamic_lds(const void *fn, int bytes)
 
 }  // namespace ksmm
 
+// Scratch memory of ksmm_chain_forward_static: one fixed device array per GPU (each GPU that
+// runs the library holds its own copy until the process ends).  In host code the name is only
+// a handle for hipGetSymbolAddress (static_scratch below), never a device address.
+constexpr int64_t KSMM_STATIC_SCRATCH_BYTES = 32ll << 20;
+static __device__ __align__(256) unsigned char scratch[KSMM_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 bool dtype_known(int dt) { return dt == KSMM_F32 || dt == KSMM_F16 || dt == KSMM_FP8_E4M3; }
@@ -336,8 +342,8 @@ bool chain_wants_transposed(const ksmm_factor_desc *f, int n, int64_t batch, int
     return false;
 }
 
-// The chain launcher behind ksmm_chain_forward and ksmm_chain_forward_ep: `ep` (may be null)
-// belongs to the last factor.
+// The chain launcher behind ksmm_chain_forward, ksmm_chain_forward_ep and
+// ksmm_chain_forward_static: `ep` (may be null) belongs to the last factor.
 int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y, void *workspace,
                        int64_t workspace_bytes, int64_t batch, int x_dtype, int y_dtype, int bs_last, int fuse,
                        const ksmm_epilogue *ep, void *stream)
@@ -413,6 +419,25 @@ int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const voi
         cur = dst;
         cur_dtype = y_dtype;
     }
+    return KSMM_OK;
+}
+
+// ---- scratch of ksmm_chain_forward_static ---------------------------------------------------
+// The device address of the array is asked for once per device, with that device current, and
+// kept; kernels and copies only ever see that address.
+constexpr int MAX_DEVICES = 64;
+std::atomic<void *> scratch_ptr[MAX_DEVICES];
+
+int static_scratch(void **out)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return KSMM_ERR_LAUNCH;
+    void *ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return KSMM_ERR_LAUNCH;
+        scratch_ptr[dev].store(ptr, std::memory_order_release);  // racing callers store the same address
+    }
+    *out = ptr;
     return KSMM_OK;
 }
 
@@ -600,6 +625,25 @@ int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const 
 {
     return chain_forward_impl(factors, n_factors, x, y, workspace, workspace_bytes, batch, x_dtype, y_dtype,
                               bs_last, fuse, epilogue, stream);
+}
+
+int64_t ksmm_static_scratch_bytes(void) { return KSMM_STATIC_SCRATCH_BYTES; }
+
+int ksmm_chain_forward_static(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
+                              int64_t batch, int x_dtype, int y_dtype, int bs_last, int fuse,
+                              const ksmm_epilogue *epilogue, void *stream)
+{
+    // what the chain would ask a caller to lend (0 when it needs no scratch at all)
+    const int64_t need = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, bs_last);
+    if (need < 0) return (int)need;
+    if (need > KSMM_STATIC_SCRATCH_BYTES) return KSMM_ERR_WORKSPACE;
+    void *buf = nullptr;
+    if (need > 0) {
+        const int rc = static_scratch(&buf);
+        if (rc != KSMM_OK) return rc;
+    }
+    return chain_forward_impl(factors, n_factors, x, y, buf, need > 0 ? KSMM_STATIC_SCRATCH_BYTES : 0, batch,
+                              x_dtype, y_dtype, bs_last, fuse, epilogue, stream);
 }
 
 }  // extern "C"

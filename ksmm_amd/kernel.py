@@ -124,9 +124,11 @@ class Kernel:
 
     @staticmethod
     def chain_forward(input, factors, patterns, bs_last, scales=None, fuse=True, workspace=None,
-                      bias=None, act=None, out=None):
+                      bias=None, act=None, static_scratch=False, out=None):
         """All factors of a KSLinear in one call (factor-chain launcher).  ``bias``/``act`` are
-        applied by the last factor's kernel."""
+        applied by the last factor's kernel.  ``static_scratch=True`` uses the library's fixed
+        32 MiB scratch array instead of a workspace tensor (no device allocation besides the
+        output, which ``out`` can supply)."""
         lib = _lib.load()
         _check_input(input, "input")
         n = len(factors)
@@ -156,6 +158,13 @@ class Kernel:
             assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
         ep, _keep = _epilogue(bias, act, out_size, out_dtype, input.device)
         ep_ref = ctypes.byref(ep) if ep is not None else None
+        if static_scratch:
+            with torch.cuda.device(input.device):
+                rc = lib.ksmm_chain_forward_static(descs, n, input.data_ptr(), out.data_ptr(), batch,
+                                                   dtype_code(input.dtype), dtype_code(out_dtype), int(bs_last),
+                                                   int(bool(fuse)), ep_ref, _stream_ptr(input))
+            _lib.check(rc)
+            return out
         need = lib.ksmm_chain_workspace_layout(descs, n, batch, dtype_code(input.dtype),
                                                dtype_code(out_dtype), int(bs_last))
         if need < 0:

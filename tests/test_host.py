@@ -104,6 +104,10 @@ def test_chain_argument_checks(lib):
     ep = _lib.KsmmEpilogue(None, 7)
     import ctypes
     assert lib.ksmm_chain_forward_ep(d, 2, x, y, ws, need, 100, 0, 0, 1, 1, ctypes.byref(ep), None) == -12
+    # the static-scratch entry point refuses chains that need more than its fixed array
+    assert lib.ksmm_static_scratch_bytes() == 32 << 20
+    assert lib.ksmm_chain_workspace_layout(d, 2, 1 << 20, 0, 0, 1) > lib.ksmm_static_scratch_bytes()
+    assert lib.ksmm_chain_forward_static(d, 2, x, 1 << 40, 1 << 20, 0, 0, 1, 1, None, None) == -9
     d[1].c = 5  # 3*5*2 = 30 != 24
     assert lib.ksmm_chain_forward(d, 2, x, y, ws, need, 100, 0, 0, 1, 1, None) == -8
     assert lib.ksmm_chain_forward(d, 17, x, y, ws, need, 100, 0, 0, 1, 1, None) == -10

@@ -1,0 +1,89 @@
+"""The entry point that allocates nothing (ksmm_chain_forward_static): its result must equal
+ksmm_chain_forward_ep's, which takes a caller's workspace, on two calls in a row, the second
+with a smaller input (the library's scratch array keeps the first call's contents)."""
+import ctypes
+
+import pytest
+import torch
+
+from tests.util import TORCH_DTYPE, round_to, seeded_input, seeded_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _descs(patterns, facs, scales):
+    from ksmm_amd import _lib
+    from ksmm_amd.kernel import dtype_code
+
+    d = (_lib.KsmmFactorDesc * len(patterns))()
+    for i, (p, f) in enumerate(zip(patterns, facs)):
+        d[i].w = f.data_ptr()
+        d[i].a, d[i].b, d[i].c, d[i].d = p
+        d[i].w_dtype = dtype_code(f.dtype)
+        d[i].scale = scales[i]
+    return d
+
+
+@pytest.mark.parametrize("case", [
+    # patterns, precision, bs_last, fuse, first batch, second (smaller) batch
+    ([(6, 64, 64, 1), (1, 768, 192, 2)], "fp32", True, 0, 1024, 264),       # ping-pong intermediates
+    ([(12, 64, 64, 1), (1, 1536, 384, 2)], "fp16", False, 0, 1000, 203),    # batch-size-first chain
+    ([(2, 64, 64, 8), (16, 64, 64, 1)], "fp16", False, 1, 520, 264),        # transposed route
+    ([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], "fp8", True, 0, 1008, 528),
+])
+def test_static_scratch_entry_point_matches_the_workspace_one(case):
+    from ksmm_amd import _lib, generate_factor, quantize_fp8
+    from ksmm_amd.kernel import dtype_code
+
+    lib = _lib.load()
+    patterns, prec, bs_last, fuse, batch1, batch2 = case
+    dt = TORCH_DTYPE[prec]
+    out_dt = torch.float16 if prec == "fp8" else dt
+    ws4 = seeded_weights(patterns, seed=81, bound=0.25 if prec == "fp8" else None)
+    facs, scales = [], []
+    for p, w4 in zip(patterns, ws4):
+        if prec == "fp8":
+            q, s = quantize_fp8(w4)
+            facs.append(generate_factor(*p, "kernel", q.float(), dt, "cuda"))
+            scales.append(float(s))
+        else:
+            facs.append(generate_factor(*p, "kernel", w4, dt, "cuda"))
+            scales.append(1.0)
+    n_in = patterns[0][0] * patterns[0][2] * patterns[0][3]
+    n_out = patterns[-1][0] * patterns[-1][1] * patterns[-1][3]
+    bias = (torch.rand(n_out) - 0.5).to(out_dt).cuda()
+    ep = _lib.KsmmEpilogue(bias.data_ptr(), _lib.ACT_GELU)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for batch in (batch1, batch2):
+        x = seeded_input(n_in, batch, bs_last, seed=82 + batch)
+        if prec == "fp8":
+            _, xq, xs = round_to(x, prec)
+            xin = xq.cuda()
+            sc = [scales[0] * xs] + scales[1:]
+        else:
+            xin = x.to(dt).cuda()
+            sc = scales
+        d = _descs(patterns, facs, sc)
+        shape = (n_out, batch) if bs_last else (batch, n_out)
+        xd, yd = dtype_code(xin.dtype), dtype_code(out_dt)
+        need = lib.ksmm_chain_workspace_layout(d, len(patterns), batch, xd, yd, int(bs_last))
+        assert 0 < need <= lib.ksmm_static_scratch_bytes(), need
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        y_ref = torch.empty(shape, dtype=out_dt, device="cuda")
+        y_sta = torch.full(shape, float("nan"), dtype=out_dt, device="cuda")
+        print("no-alloc case", patterns, prec, bs_last, batch, "workspace", need, flush=True)
+        _lib.check(lib.ksmm_chain_forward_ep(d, len(patterns), xin.data_ptr(), y_ref.data_ptr(), ws.data_ptr(), need,
+                                             batch, xd, yd, int(bs_last), fuse, ctypes.byref(ep), stream))
+        before = torch.cuda.memory_allocated()
+        _lib.check(lib.ksmm_chain_forward_static(d, len(patterns), xin.data_ptr(), y_sta.data_ptr(), batch, xd, yd,
+                                                 int(bs_last), fuse, ctypes.byref(ep), stream))
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == before
+        # same kernels on the same inputs: bit-identical
+        assert torch.equal(y_ref.view(torch.uint8), y_sta.view(torch.uint8)), (patterns, prec, batch)
+    # a chain whose intermediates exceed the fixed array is refused, not truncated
+    big = 1 << 16  # e.g. 3072 features x 65536 columns: fewer than 2^31 elements, intermediates far above 32 MiB
+    d = _descs(patterns, facs, scales)
+    rc = lib.ksmm_chain_forward_static(d, len(patterns), xin.data_ptr(), y_sta.data_ptr(), big, xd, yd, int(bs_last), fuse,
+                                       None, stream)
+    assert rc == -9
