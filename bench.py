@@ -155,6 +155,28 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
         sec = time_launches(lambda j: run_chain(j, False), n_sets, max(3, steps // 2), max(1, warmup // 2))
         result["kslinear_unfused_us"] = sec * 1e6
         final = run_chain(0)
+        # the layer as a network uses it: bias (and, for the ViT up-projection, GELU) applied by the
+        # last factor's kernel, against the same chain followed by a separate elementwise pass
+        out_size = patterns[-1][0] * patterns[-1][1] * patterns[-1][3]
+        bias = (torch.rand(out_size, generator=torch.Generator().manual_seed(SEED + 99)) - 0.5).to(out_dt).cuda()
+        act = "gelu" if name == "C4_vit_b_up" else None
+        outs_ep = [torch.empty_like(final) for _ in range(n_sets)]
+
+        def run_chain_ep(j):
+            sc = list(wscales)
+            sc[0] *= scales[j]
+            return Kernel.chain_forward(xs[j], facs, patterns, bs_last, scales=sc, fuse=True, workspace=ws_bytes,
+                                        bias=bias, act=act, out=outs_ep[j])
+
+        def run_chain_then_torch(j):
+            y = run_chain(j)
+            y = y + (bias[:, None] if bs_last else bias)
+            return torch.nn.functional.gelu(y) if act else y
+
+        sec = time_launches(run_chain_ep, n_sets, max(3, steps // 2), max(1, warmup // 2))
+        result["kslinear_bias%s_fused_us" % ("_gelu" if act else "")] = sec * 1e6
+        sec = time_launches(run_chain_then_torch, n_sets, max(3, steps // 2), max(1, warmup // 2))
+        result["kslinear_bias%s_separate_pass_us" % ("_gelu" if act else "")] = sec * 1e6
     else:
         result["kslinear_us"] = result["factors"][0]["us"]
         final = cur[0]
@@ -201,7 +223,7 @@ def copy_reference(steps, warmup):
             "bytes": nbytes, "kernel": "torch.add(x, 1, out=y) elementwise kernel"}
 
 
-def cpu_baseline(patterns, bs_last, budget_s=12.0):
+def cpu_baseline(patterns, bs_last, budget_s=12.0, min_run_time=0.25):
     """The reference's algo='bmm' CPU algorithm (restated in oracle/), fp32, on all host
     cores; protocol of the reference's ksmm_time.py: blocked_autorange(min_run_time=0.25),
     re-run with 11*max(mean, median) when fewer than 10 runs fit."""
@@ -221,7 +243,7 @@ def cpu_baseline(patterns, bs_last, budget_s=12.0):
         timer = tb.Timer(stmt="f(wb, x, patterns, bs_last)",
                          globals={"f": O.torch_bmm_chain, "wb": wb, "x": x, "patterns": patterns,
                                   "bs_last": bs_last}, num_threads=torch.get_num_threads())
-        m = timer.blocked_autorange(min_run_time=0.25)
+        m = timer.blocked_autorange(min_run_time=min_run_time)
         if m.number_per_run <= 10:
             m = timer.blocked_autorange(min_run_time=min(budget_s, 11 * max(m.mean, m.median)))
     return {"value": m.median * 1e6, "unit": "us", "cores": torch.get_num_threads(), "kind": "port",
@@ -230,15 +252,29 @@ def cpu_baseline(patterns, bs_last, budget_s=12.0):
             "mean_us": m.mean * 1e6, "iqr_us": m.iqr * 1e6, "host_cpu_count": os.cpu_count()}
 
 
-# HBM bytes per launch of the headline kernel, ks_wave_bl_f32<3,12,2,true> on (1,48,48,16) fp32 bs_last
-# at B = 25088, from two counter passes over this script
-#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 20 --warmup 5 --cpu 0 --copy-calib 10
-#   rocprofv3 --pmc WRITE_SIZE -- python3 bench.py --steps 20 --warmup 5 --cpu 0 --copy-calib 10
-# FETCH_SIZE 39453.3 KiB and WRITE_SIZE 75264.0 KiB per dispatch, each divided by what the same
-# counter reads for the torch.add calibration kernel per KiB it moves (0.5002 and 1.0000).
-# Counters cannot be collected from inside a timed run, so the figure is carried here; it
-# belongs to that kernel and workload only and is dropped if another kernel is dispatched.
-MEASURED_TRAFFIC = {"algo": 2, "variant": 0, "bytes": int((39421.5 / 0.5002 + 75264.0 / 1.0000) * 1024)}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_hbm_traffic.txt")
+
+
+def measured_traffic(name, algo, variant):
+    """HBM bytes per launch of a benchmark kernel from the tracked counter summary
+    profiles/bench_hbm_traffic.txt (counters cannot be collected from inside a timed run).  Lines:
+        CALIB fetch=<FETCH_SIZE KiB read per KiB a copy kernel of known size fetches> write=<same for WRITE_SIZE>
+        TRAFFIC <config> factor=<i> algo=<a> variant=<hex> fetch_kib=<per dispatch> write_kib=<per dispatch>
+    Returns None when there is no line for this configuration with the kernel (algo, variant) that
+    ran: a figure measured on another kernel does not carry over."""
+    try:
+        lines = open(TRAFFIC_FILE).read().splitlines()
+    except OSError:
+        return None
+    calib = None
+    for l in lines:
+        f = dict(t.split("=", 1) for t in l.split()[1:] if "=" in t)
+        if l.startswith("CALIB"):
+            calib = (float(f["fetch"]), float(f["write"]))
+        elif l.startswith("TRAFFIC") and calib and l.split()[1] == name and int(f["factor"]) == 0 \
+                and int(f["algo"]) == algo and int(f["variant"], 16) == variant:
+            return int((float(f["fetch_kib"]) / calib[0] + float(f["write_kib"]) / calib[1]) * 1024)
+    return None
 
 
 def main():
@@ -284,14 +320,20 @@ def main():
     sec = head["factors"][0]["us"] / 1e6
     roof = factor_roofline(BATCH, CONFIGS[0][1][0], torch.float32, torch.float32, torch.float32, sec)
     hf = head["factors"][0]
-    traffic = (MEASURED_TRAFFIC["bytes"]
-               if (hf["algo"], hf["variant"]) == (MEASURED_TRAFFIC["algo"], MEASURED_TRAFFIC["variant"]) else None)
+    traffic = measured_traffic(CONFIGS[0][0], hf["algo"], hf["variant"])
     others = []
     if args.all:
         for cfg in CONFIGS[1:]:
             others.append(bench_config(*cfg, steps=max(20, args.steps // 2), warmup=max(5, args.warmup // 2)))
     copy_ref = copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
+    if args.cpu:
+        # the same CPU algorithm beside every other configuration (fp32 on the host, whatever the
+        # device precision; a short sample each so that the whole run stays within minutes)
+        head["cpu_bmm_us"], head["cpu_cores"] = cpu["value"], cpu["cores"]
+        for cfg, res in zip(CONFIGS[1:], others):
+            c = cpu_baseline(cfg[1], cfg[3], budget_s=4.0, min_run_time=0.1)
+            res["cpu_bmm_us"], res["cpu_cores"], res["cpu_sample"] = c["value"], c["cores"], c["sample"]
     line = {
         "metric": "us_per_ks_factor", "value": head["factors"][0]["us"], "unit": "us",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,

@@ -139,13 +139,37 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
     const uint32_t x_lane = (uint32_t)(q * row_stride) * 4u;      // + column offset
     const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 4u;  // + column offset
-    // tiles of one wave: consecutive (rr == 0) or every n_slabs-th (rr == 1: the waves of a
-    // block then work on neighbouring tiles at any one time)
-    const int stride = rr ? n_slabs * TN : TN;                    // uniform
-    const int n_first = rr ? slab * TN : slab * iters * TN;       // uniform
-    const int n_end = rr ? batch : min(n_first + iters * TN, batch);
+    // Tiles of one wave (all uniform): `regular` tiles at n_first, n_first + stride, ... and, in
+    // the balanced mode, possibly one more at n_extra.
+    //  rr == 0: `iters` consecutive tiles;  rr == 1: every n_slabs-th tile (the waves of a block
+    //  then work on neighbouring tiles at any one time);
+    //  rr == 2 (balanced): as rr == 1 for the full rounds; the tiles of the last, partial round go
+    //  one each to wave 0 of every workgroup of the block, then to wave 1 of every workgroup, ...
+    //  so that no workgroup (CU) gets more than its share rounded up.
+    const int n_tiles_row = (batch + TN - 1) / TN;
+    int stride, n_first, regular, n_extra = -1;
+    if (rr == 2) {
+        const int wpw = (int)(blockDim.x >> 6), n_wg = n_slabs / wpw;
+        const int full = n_tiles_row / n_slabs, rest = n_tiles_row - full * n_slabs;
+        const int e = (slab % wpw) * n_wg + slab / wpw;
+        stride = n_slabs * TN;
+        n_first = slab * TN;
+        regular = full;
+        if (e < rest) n_extra = (full * n_slabs + e) * TN;
+    } else if (rr == 1) {
+        stride = n_slabs * TN;
+        n_first = slab * TN;
+        regular = n_first < batch ? (batch - n_first + stride - 1) / stride : 0;
+    } else {
+        stride = TN;
+        n_first = slab * iters * TN;
+        regular = n_first < batch ? min(iters, (batch - n_first + TN - 1) / TN) : 0;
+    }
+    const int count = regular + (n_extra >= 0 ? 1 : 0);
     const int last_vec = batch - VEC;
-    if (n_first >= n_end) return;
+    if (count <= 0) return;
+    auto tile_start = [&](int k) { return k < regular ? n_first + k * stride : n_extra; };  // k < count
+    const int n_begin = tile_start(0);
 
     // Rolling register pipeline: xc[ks] holds input rows 4*ks + q of the current tile; as soon
     // as the MFMAs of step ks are issued the same registers are refilled with the next tile's
@@ -154,7 +178,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     float4_t xc[KS];
     auto col_off = [&](int n0) { return (uint32_t)min(n0 + VEC * r, last_vec) * 4u; };
     {
-        const uint32_t off = x_lane + col_off(n_first);
+        const uint32_t off = x_lane + col_off(n_begin);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
             xc[ks] = *(const float4_t *)(xg + (size_t)(4 * ks) * row_stride * 4 + off);
@@ -171,12 +195,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     // Everything issued so far (weights, first tile) is complete before the loop, so that the
     // waits inside the loop only ever count that loop's own loads and stores.
     __builtin_amdgcn_s_waitcnt(0);
-    const int n_last = n_first + ((n_end - n_first - 1) / stride) * stride;  // first column of the last tile
-    // FULL tiles store without a predicate, which keeps the loop body free of branches; a
-    // ragged last tile (batch not a multiple of the tile) runs once more with the predicate.
-    auto do_tile = [&](int n0, auto full) {
-        // the tile after the last one is the last one again (a cache hit that is not used)
-        const uint32_t next_off = x_lane + col_off(min(n0 + stride, n_last));
+    // FULL tiles store without a predicate, which keeps the loop body free of branches; only a
+    // wave's last tile can be the ragged one (batch not a multiple of the tile): it runs with
+    // the predicate.
+    auto do_tile = [&](int n0, int n_next, auto full) {
+        // (the tile after the last one is the last one again: a cache hit that is not used)
+        const uint32_t next_off = x_lane + col_off(n_next);
         float4_t acc[MT][VEC];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -213,9 +237,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
                 }
         }
     };
-    int n0 = n_first;
-    for (; n0 + TN <= n_end; n0 += stride) do_tile(n0, std::true_type{});
-    if (n0 < n_end) do_tile(n0, std::false_type{});
+    for (int k = 0; k + 1 < count; ++k) do_tile(tile_start(k), tile_start(k + 1), std::true_type{});
+    const int n_fin = tile_start(count - 1);
+    if (n_fin + TN <= batch)
+        do_tile(n_fin, n_fin, std::true_type{});
+    else
+        do_tile(n_fin, n_fin, std::false_type{});
 }
 
 // ------------------------------------------------------------------------------------------
@@ -257,18 +284,38 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
     char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
     const uint32_t x_lane = (uint32_t)(KL * q * row_stride) * (uint32_t)sizeof(TX);
     const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 2u;
-    const int stride = rr ? n_slabs * TN : TN;
-    const int n_first = rr ? slab * TN : slab * iters * TN;
-    const int n_end = rr ? batch : min(n_first + iters * TN, batch);
+    // this wave's tiles: see the fp32 kernel
+    const int n_tiles_row = (batch + TN - 1) / TN;
+    int stride, n_first, regular, n_extra = -1;
+    if (rr == 2) {
+        const int wpw = (int)(blockDim.x >> 6), n_wg = n_slabs / wpw;
+        const int full = n_tiles_row / n_slabs, rest = n_tiles_row - full * n_slabs;
+        const int e = (slab % wpw) * n_wg + slab / wpw;
+        stride = n_slabs * TN;
+        n_first = slab * TN;
+        regular = full;
+        if (e < rest) n_extra = (full * n_slabs + e) * TN;
+    } else if (rr == 1) {
+        stride = n_slabs * TN;
+        n_first = slab * TN;
+        regular = n_first < batch ? (batch - n_first + stride - 1) / stride : 0;
+    } else {
+        stride = TN;
+        n_first = slab * iters * TN;
+        regular = n_first < batch ? min(iters, (batch - n_first + TN - 1) / TN) : 0;
+    }
+    const int count = regular + (n_extra >= 0 ? 1 : 0);
     const int last_vec = batch - VEC;
-    if (n_first >= n_end) return;
+    if (count <= 0) return;
+    auto tile_start = [&](int k) { return k < regular ? n_first + k * stride : n_extra; };
+    const int n_begin = tile_start(0);
 
     // Rolling register pipeline as in the fp32 kernel: raw[ks][jj] holds VEC packed columns of
     // input row KSTEP*ks + KL*q + jj; it is refilled for the next tile right after step ks.
     uint32_t raw[KS][KL][io::RAW];
     auto col_off = [&](int n0) { return (uint32_t)min(n0 + VEC * r, last_vec) * (uint32_t)sizeof(TX); };
     {
-        const uint32_t off = x_lane + col_off(n_first);
+        const uint32_t off = x_lane + col_off(n_begin);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -285,9 +332,8 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
                 bv[mt][i] = epi_bias<half_t>(ep, ((size_t)a_i * b + 16 * mt + 4 * q + i) * d + d_i);
     }
     __builtin_amdgcn_s_waitcnt(0);
-    const int n_last = n_first + ((n_end - n_first - 1) / stride) * stride;
-    auto do_tile = [&](int n0, auto full) {
-        const uint32_t next_off = x_lane + col_off(min(n0 + stride, n_last));
+    auto do_tile = [&](int n0, int n_next, auto full) {
+        const uint32_t next_off = x_lane + col_off(n_next);
         float4_t acc[MT][VEC];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -346,9 +392,12 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
                 }
         }
     };
-    int n0 = n_first;
-    for (; n0 + TN <= n_end; n0 += stride) do_tile(n0, std::true_type{});
-    if (n0 < n_end) do_tile(n0, std::false_type{});
+    for (int k = 0; k + 1 < count; ++k) do_tile(tile_start(k), tile_start(k + 1), std::true_type{});
+    const int n_fin = tile_start(count - 1);
+    if (n_fin + TN <= batch)
+        do_tile(n_fin, n_fin, std::true_type{});
+    else
+        do_tile(n_fin, n_fin, std::false_type{});
 }
 
 // ---- instance table ---------------------------------------------------------------------
@@ -433,11 +482,14 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const WaveInst *insts = wave_table(combo, &n_insts);
     if (!insts) return KSMM_ERR_BAD_DTYPE;
     // vector loads along the batch axis need every row start aligned to the vector
-    // variant: bits 0-7 instance index (0xff: first that fits), bits 8-15 wave iterations
-    // (0: heuristic); -1: everything automatic
+    // variant: bits 0-7 instance index (0xff: first that fits), bits 8-15 tiles per wave (0:
+    // heuristic), bits 16-17 how tiles are dealt: 0 consecutive, 1 every n_slabs-th, 2 balanced
+    // (bits 8-15 are then workgroups per block, 0: one round of workgroups over the chip);
+    // -1: everything automatic
     const int want = variant < 0 ? 0xff : (variant & 0xff);
     int iters = variant < 0 ? 0 : ((variant >> 8) & 0xff);
-    int rr = variant < 0 ? 0 : ((variant >> 16) & 1);  // tiles of a wave: 0 consecutive, 1 every n_slabs-th
+    int rr = variant < 0 ? -1 : ((variant >> 16) & 3);
+    if (rr == 3) return KSMM_ERR_BAD_ALGO;
     int pick = -1;
     for (int i = 0; i < n_insts; ++i) {
         if (insts[i].b != p.b || insts[i].c != p.c) continue;
@@ -467,18 +519,35 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     // smallest count that fits one round.
     const int64_t groups = (int64_t)p.a * p.d;
     const int wpb = 4;
-    if (iters == 0) {
-        iters = 1;
-        if (p.b * p.c > 1024)
-            while (iters < 255 && (groups * ((n_tiles + iters - 1) / iters) + wpb - 1) / wpb > 256) ++iters;
+    // (Balanced dealing, rr == 2, keeps every CU within one tile of its share: (1,48,48,16) at
+    // batch 25088 has 24.5 tiles per CU where 7 consecutive tiles per wave leave 32 CUs idle and
+    // give the others 28.  Measured, it is 1-3 % slower than the consecutive split on that shape
+    // and on (6,64,64,1): these kernels are not bound by the busiest CU.  It stays selectable.)
+    if (rr < 0) rr = 0;
+    int64_t n_slabs, blocks;
+    int iters_field = 0;  // what the variant's bits 8-15 must hold to reproduce this launch
+    if (rr == 2) {
+        int64_t wgs_pb = iters > 0 ? iters : (256 / groups > 1 ? 256 / groups : 1);
+        if (wgs_pb > 255) wgs_pb = 255;
+        if (wgs_pb > (n_tiles + wpb - 1) / wpb) wgs_pb = (n_tiles + wpb - 1) / wpb;
+        n_slabs = wpb * wgs_pb;
+        blocks = groups * wgs_pb;
+        iters_field = (int)(wgs_pb < 255 ? wgs_pb : 255);
+        iters = 2;  // (several tiles per wave: the kernel with the rolling pipeline)
+    } else {
+        if (iters == 0) {
+            iters = 1;
+            if (p.b * p.c > 1024)
+                while (iters < 255 && (groups * ((n_tiles + iters - 1) / iters) + wpb - 1) / wpb > 256) ++iters;
+        }
+        n_slabs = (n_tiles + iters - 1) / iters;
+        blocks = (groups * n_slabs + wpb - 1) / wpb;
+        iters_field = iters;
     }
-    const int64_t n_slabs = (n_tiles + iters - 1) / iters;
-    const int64_t waves = groups * n_slabs;
-    const int64_t blocks = (waves + wpb - 1) / wpb;
     if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_WAVE;
-        tile->variant = pick;
+        tile->variant = pick | (iters_field << 8) | (rr << 16);
         tile->tile_m = p.b;
         tile->tile_n = tn;
         tile->tile_k = p.c;

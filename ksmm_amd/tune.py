@@ -82,6 +82,7 @@ def candidates(bs_last=True, combo=1):
                 out.append((2, inst | (it << 8)))
             for it in (0, 2, 4):                 # the same with tiles dealt round-robin
                 out.append((2, inst | (it << 8) | (1 << 16)))
+            out.append((2, inst | (2 << 16)))    # one round of workgroups, balanced dealing
     else:
         for inst in range(_count(2, lambda i: 1000 + i, combo, False)):   # batch-size-first row kernel
             out.append((2, 1000 + inst))

@@ -162,8 +162,11 @@ def test_wave_instances_forced():
     shapes = [(2, 48, 48, 3), (2, 64, 64, 2), (3, 16, 16, 5), (2, 32, 32, 3), (1, 96, 96, 2), (2, 48, 192, 2),
               (1, 192, 48, 3)]
     cases = [(prec, True, p, 1040) for prec in ("fp32", "fp16", "hq", "fp8") for p in shapes]
-    variants = [inst | (it << 8) | (rr << 16) for inst in range(12) for it, rr in ((1, 0), (3, 0), (2, 1))]
-    _forced_sweep(cases, variants, 2, 100)
+    # tiles per wave / dealing: one tile, three consecutive, every n-th, balanced (automatic and 3
+    # workgroups per block)
+    variants = [inst | (it << 8) | (rr << 16) for inst in range(12)
+                for it, rr in ((1, 0), (3, 0), (2, 1), (0, 2), (3, 2))]
+    _forced_sweep(cases, variants, 2, 160)
 
 
 def test_row_kernel_instances_forced():

@@ -426,3 +426,38 @@ def test_unaligned_tensors_are_refused_by_forced_families(lib):
     f = lib.ksmm_factor_forward_algo
     assert f(4096 + 4, 1 << 20, 2 << 20, 64, 1, 16, 16, 1, 0, 0, 0, 1, 1.0, 2, -1, None) == -6
     assert f(4096, (1 << 20) + 8, 2 << 20, 64, 1, 16, 16, 1, 0, 0, 0, 1, 1.0, 3, -1, None) == -6
+
+
+def test_bench_csv_writes_the_reference_schema_and_replaces_rows(tmp_path, capsys):
+    """python -m ksmm_amd.bench_csv: the reference's CSV columns (ksmm_time.py:61-67), one row per
+    configuration (a second run of the same configuration replaces its row), --correctness
+    prints the relative error against the dense product, and the feed-forward granularity."""
+    import csv
+
+    from ksmm_amd import bench_csv
+
+    out = tmp_path / "res" / "t.csv"
+    base = ["--saving-csv", str(out), "--device", "cpu", "--precision", "fp32", "--batch-size", "16",
+            "--min-run-time", "0.01"]
+    bench_csv.main(base + ["--patterns", "2,3,5,4", "3,6,4,2", "--algo", "bmm", "--bs-last", "1", "--correctness"])
+    printed = capsys.readouterr().out
+    err = float(re.search(r"Relative error = ([0-9.e+-]+)", printed).group(1))
+    assert err < 1e-5
+    bench_csv.main(base + ["--patterns", "2,3,5,4", "3,6,4,2", "--algo", "bmm", "--bs-last", "1"])      # same key
+    bench_csv.main(base + ["--patterns", "2,3,5,4", "3,6,4,2", "--algo", "einsum", "--bs-last", "0"])
+    bench_csv.main(base + ["--granularity", "ffn", "--patterns_up", "2,6,4,1", "--patterns_down", "2,4,6,1",
+                           "--algo", "dense", "--correctness"])
+    assert float(re.search(r"Relative error = ([0-9.e+-]+)", capsys.readouterr().out).group(1)) < 1e-5
+    rows = list(csv.DictReader(open(out)))
+    assert list(rows[0].keys()) == ["pattern", "batch-size", "algo", "bs_position", "precision", "vsize",
+                                    "device_name", "mean", "median", "iqr", "times"]
+    assert len(rows) == 3
+    assert rows[0]["pattern"] == "[[2, 3, 5, 4], [3, 6, 4, 2]]" and rows[0]["bs_position"] == "bs_last"
+    assert rows[1]["algo"] == "einsum" and rows[1]["bs_position"] == "bs_first"
+    assert rows[2]["pattern"].startswith("ffn:") and float(rows[2]["median"]) > 0
+    # a file without the expected columns is refused, as the reference does
+    bad = tmp_path / "bad.csv"
+    bad.write_text("a,b\n1,2\n")
+    with pytest.raises(ValueError):
+        bench_csv.main(["--saving-csv", str(bad), "--device", "cpu", "--patterns", "2,3,5,4", "--algo", "bmm",
+                        "--min-run-time", "0.01"])
