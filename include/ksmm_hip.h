@@ -218,6 +218,26 @@ int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const 
                           int y_dtype, int bs_last, int fuse, const ksmm_epilogue *epilogue,
                           void *stream);
 
+/* Backward pass of one factor y = scale_fwd * K x, for F32 and F16 tensors (all three of one
+ * type).  The reference has none that works (src/ksmm_py/layer/kronecker_sparse/kernel.py:319-329
+ * names an undefined symbol, forward_bmm.py:12-15 is `pass`); these are the adjoints of its
+ * forward product (interface.py:108-113):
+ *   ksmm_factor_backward_input :  dx = scale * K^T dy, the KS factor with pattern (a, c, b, d)
+ *                                 and every b x c block transposed, on the forward kernels;
+ *   ksmm_factor_backward_weight:  dw[a_i,b_i,c_i,d_i] = scale * sum_n dy[a_i,b_i,d_i,n] x[a_i,c_i,d_i,n],
+ *                                 written in kernel format (a*d*c, b) like w.
+ * dy has y's shape and layout, dx has x's.  Both need ksmm_factor_backward_workspace() bytes of
+ * 16-byte aligned device memory (transposed blocks, an fp32 accumulator for the reduction over
+ * the batch, and the forward kernels' own workspace for the transposed factor). */
+int64_t ksmm_factor_backward_workspace(int64_t batch, int a, int b, int c, int d, int dtype,
+                                       int bs_last);
+int ksmm_factor_backward_input(const void *dy, const void *w, void *dx, int64_t batch, int a, int b,
+                               int c, int d, int dtype, int bs_last, float scale, void *workspace,
+                               int64_t workspace_bytes, void *stream);
+int ksmm_factor_backward_weight(const void *dy, const void *x, void *dw, int64_t batch, int a, int b,
+                                int c, int d, int dtype, int bs_last, float scale, void *workspace,
+                                int64_t workspace_bytes, void *stream);
+
 /* ksmm_chain_forward_ep for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): the ping-pong intermediates
  * and the transposed-route buffers live in a fixed device array inside the library,

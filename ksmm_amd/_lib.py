@@ -70,6 +70,11 @@ SIGNATURES = {
                                        c_vp]),
     "ksmm_chain_forward_ep": (c_int, [ctypes.POINTER(KsmmFactorDesc), c_int, c_vp, c_vp, c_vp, c_i64,
                                       c_i64, c_int, c_int, c_int, c_int, ctypes.POINTER(KsmmEpilogue), c_vp]),
+    "ksmm_factor_backward_workspace": (c_i64, [c_i64, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "ksmm_factor_backward_input": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                           ctypes.c_float, c_vp, c_i64, c_vp]),
+    "ksmm_factor_backward_weight": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                            ctypes.c_float, c_vp, c_i64, c_vp]),
     "ksmm_static_scratch_bytes": (c_i64, []),
     "ksmm_chain_forward_static": (c_int, [ctypes.POINTER(KsmmFactorDesc), c_int, c_vp, c_vp, c_i64, c_int,
                                           c_int, c_int, c_int, ctypes.POINTER(KsmmEpilogue), c_vp]),

@@ -280,7 +280,7 @@ int factor_forward_impl(const void *x, const void *w, void *y, int64_t batch, in
     }
     // Every kernel but the one-thread-per-output one moves 16-byte vectors: tensors that do not
     // start on a 16-byte boundary run on that kernel (a forced family refuses them).
-    if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) != 0) {
+    if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)p.bias) & 15) != 0) {
         if (algo != KSMM_ALGO_AUTO && !(algo == KSMM_ALGO_GENERIC && variant <= 0)) return KSMM_ERR_BAD_ALGO;
         return generic_run(p, 0, true, nullptr);
     }
@@ -625,6 +625,50 @@ int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const 
 {
     return chain_forward_impl(factors, n_factors, x, y, workspace, workspace_bytes, batch, x_dtype, y_dtype,
                               bs_last, fuse, epilogue, stream);
+}
+
+int64_t ksmm_factor_backward_workspace(int64_t batch, int a, int b, int c, int d, int dtype, int bs_last)
+{
+    int rc = check_shape(batch, a, b, c, d, dtype, dtype, dtype);
+    if (rc != KSMM_OK) return rc;
+    if (dtype != KSMM_F32 && dtype != KSMM_F16) return KSMM_ERR_BAD_DTYPE;
+    const int64_t nnz = (int64_t)a * b * c * d;
+    // transposed blocks (input gradient) | fp32 accumulator (weight gradient) | what the forward
+    // kernels of the transposed factor ask for
+    const int64_t fwd = ksmm_factor_workspace(batch, a, c, b, d, dtype, dtype, dtype, bs_last);
+    if (fwd < 0) return fwd;
+    return align256(nnz * (int64_t)dtype_size(dtype)) + align256(nnz * 4) + fwd;
+}
+
+int ksmm_factor_backward_input(const void *dy, const void *w, void *dx, int64_t batch, int a, int b,
+                               int c, int d, int dtype, int bs_last, float scale, void *workspace,
+                               int64_t workspace_bytes, void *stream)
+{
+    const int64_t need = ksmm_factor_backward_workspace(batch, a, b, c, d, dtype, bs_last);
+    if (need < 0) return (int)need;
+    if (!dy || !w || !dx) return KSMM_ERR_NULL_POINTER;
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
+    const int64_t nnz = (int64_t)a * b * c * d;
+    char *wt = (char *)workspace;
+    char *fwd_ws = wt + align256(nnz * (int64_t)dtype_size(dtype)) + align256(nnz * 4);
+    int rc = block_transpose_run(w, wt, a, b, c, d, dtype, (hipStream_t)stream);
+    if (rc != KSMM_OK) return rc;
+    // dX = K^T dY: the factor with pattern (a, c, b, d) and transposed blocks
+    return factor_forward_ws_impl(dy, wt, dx, batch, a, c, b, d, dtype, dtype, dtype, bs_last, scale, nullptr, fwd_ws,
+                                  workspace_bytes - (fwd_ws - wt), stream);
+}
+
+int ksmm_factor_backward_weight(const void *dy, const void *x, void *dw, int64_t batch, int a, int b,
+                                int c, int d, int dtype, int bs_last, float scale, void *workspace,
+                                int64_t workspace_bytes, void *stream)
+{
+    const int64_t need = ksmm_factor_backward_workspace(batch, a, b, c, d, dtype, bs_last);
+    if (need < 0) return (int)need;
+    if (!dy || !x || !dw) return KSMM_ERR_NULL_POINTER;
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
+    const int64_t nnz = (int64_t)a * b * c * d;
+    float *acc = (float *)((char *)workspace + align256(nnz * (int64_t)dtype_size(dtype)));
+    return wgrad_run(dy, x, dw, acc, batch, a, b, c, d, dtype, bs_last ? 1 : 0, scale, (hipStream_t)stream, nullptr);
 }
 
 int64_t ksmm_static_scratch_bytes(void) { return KSMM_STATIC_SCRATCH_BYTES; }

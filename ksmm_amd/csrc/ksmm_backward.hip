@@ -1,0 +1,310 @@
+// Backward pass of one Kronecker-sparse factor y = K x (forward: ksmm_factor_forward).
+//
+//   dX = K^T dY   is itself a KS factor: pattern (a, c, b, d) with every b x c block transposed,
+//                 so it runs on the forward kernels once the blocks are transposed (ks_block_transpose_kernel)
+//   dW[a_i, b_i, c_i, d_i] = sum_n dY[a_i, b_i, d_i, n] * X[a_i, c_i, d_i, n]
+//                 one (b x B) @ (B x c) product per (a_i, d_i) block, reduced over the batch:
+//                 MFMA kernel for batch-size-last (operand rows are batch-contiguous, so both
+//                 operands come straight from global memory in MFMA layout, no LDS), an
+//                 LDS-tiled FMA kernel for everything else; partial sums over batch splits are
+//                 accumulated with fp32 atomics in a workspace and then scaled, converted and
+//                 written in kernel format (a*d*c, b).
+//
+// The reference has no backward pass (src/ksmm_py/layer/kronecker_sparse/kernel.py:319-329 refers
+// to an undefined symbol; forward_bmm.py:12-15 is `pass`); the definition above is the adjoint of
+// its forward product (interface.py:108-113).
+#include "ksmm_common.h"
+
+namespace ksmm {
+
+namespace {
+
+// out block g (b x c, c contiguous)  <-  in block g (c x b, b contiguous); both in "kernel format"
+// of their own pattern: in = (a*d*c, b) of (a,b,c,d), out = (a*d*b, c) of (a,c,b,d)
+template <typename T>
+__global__ __launch_bounds__(256) void ks_block_transpose_kernel(const T *__restrict__ in, T *__restrict__ out,
+                                                                 int64_t total, int b, int c)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into out
+    if (i >= total) return;
+    const int64_t g = i / ((int64_t)b * c);
+    const int rem = (int)(i - g * b * c);
+    const int bi = rem / c, ci = rem - bi * c;
+    out[i] = in[(g * c + ci) * b + bi];
+}
+
+__global__ __launch_bounds__(256) void ks_fill_zero_kernel(float *__restrict__ p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void ks_wgrad_finish_kernel(const float *__restrict__ acc, T *__restrict__ dw,
+                                                              int64_t n, float scale)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dw[i] = (T)(acc[i] * scale);
+}
+
+template <typename T> struct wg_vec;
+template <> struct wg_vec<float> {
+    static constexpr int N = 4, MFMAS = 4;  // elements per 16-byte load; MFMAs fed by one load pair
+    typedef float4_t type;
+    __device__ static __forceinline__ float4_t mfma(int e, float4_t a, float4_t b, float4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], c, 0, 0, 0);
+    }
+};
+template <> struct wg_vec<half_t> {
+    static constexpr int N = 8, MFMAS = 2;
+    typedef half8_t type;
+    __device__ static __forceinline__ float4_t mfma(int e, half8_t a, half8_t b, float4_t c)
+    {
+        const half4_t ah = {a[4 * e], a[4 * e + 1], a[4 * e + 2], a[4 * e + 3]};
+        const half4_t bh = {b[4 * e], b[4 * e + 1], b[4 * e + 2], b[4 * e + 3]};
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(ah, bh, c, 0, 0, 0);
+    }
+};
+
+// Batch-size-last, batch a multiple of the 16-byte vector.  One wavefront owns a (16*MT) x (16*NT)
+// tile of one block's b x c gradient and a range of batch columns.  Lane (r = lane % 16,
+// q = lane / 16) loads N consecutive batch elements of operand row r at column n + N*q; MFMA e
+// multiplies element group e of every lane, i.e. its k-set is {n + N*q + e ...}: the same set for
+// both operands, and the order of a sum's terms is free.
+template <typename T, int MT, int NT>
+__global__ __launch_bounds__(256) void ks_wgrad_bl_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                          float *__restrict__ acc_out, int batch, int a, int b,
+                                                          int c, int d, int m_tiles, int n_tiles, int splits,
+                                                          int cols_per_split)
+{
+    typedef wg_vec<T> V;
+    constexpr int STEP = 4 * V::N;  // batch columns per step (4 lane groups)
+    const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+    int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int split = (int)(wave % splits);
+    wave /= splits;
+    const int nt = (int)(wave % n_tiles);
+    wave /= n_tiles;
+    const int mt = (int)(wave % m_tiles);
+    const int64_t g = wave / m_tiles;
+    if (g >= (int64_t)a * d) return;
+    const int a_i = (int)(g / d), d_i = (int)(g - (int64_t)a_i * d);
+    const int m0 = mt * 16 * MT, c0 = nt * 16 * NT;
+    const int n_begin = split * cols_per_split, n_end = min(batch, n_begin + cols_per_split);
+    if (n_begin >= n_end) return;
+    const size_t row_stride = (size_t)d * batch;
+    // rows behind b (or c) are clamped to the last valid one and dropped at the end
+    const T *ap[MT], *bp[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+        ap[i] = dy + ((size_t)a_i * b * d + d_i) * batch + (size_t)min(m0 + 16 * i + r, b - 1) * row_stride;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+        bp[j] = x + ((size_t)a_i * c * d + d_i) * batch + (size_t)min(c0 + 16 * j + r, c - 1) * row_stride;
+    float4_t acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    typedef typename V::type vec_t;
+    for (int n = n_begin; n < n_end; n += STEP) {
+        const int col = n + V::N * q;
+        const bool live = col < n_end;             // whole vectors: batch and the split are multiples of N
+        const int lcol = live ? col : n_begin;     // (a valid address; the value is zeroed)
+        vec_t av[MT], bv[NT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) av[i] = *(const vec_t *)(ap[i] + lcol);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) bv[j] = *(const vec_t *)(bp[j] + lcol);
+        if (!live) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) av[i][e] = 0;
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) bv[j][e] = 0;
+        }
+#pragma unroll
+        for (int e = 0; e < V::MFMAS; ++e)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[i][j] = V::mfma(e, av[i], bv[j], acc[i][j]);
+    }
+    // D: lane holds column (c index) r and rows (b index) 4*q .. 4*q + 3 of each 16 x 16 tile
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int cc = c0 + 16 * j + r;
+            if (cc >= c) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int m = m0 + 16 * i + 4 * q + e;
+                if (m < b) atomicAdd(acc_out + ((size_t)g * c + cc) * b + m, acc[i][j][e]);
+            }
+        }
+}
+
+// Any layout, any batch: 16 x 16 threads compute a 16 x 16 tile of one block's gradient over a
+// batch range, staging 16 x 16 element tiles of both operands in LDS (fp32 FMAs).
+template <typename T, bool BS_LAST>
+__global__ __launch_bounds__(256) void ks_wgrad_tiled_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                             float *__restrict__ acc_out, int64_t batch, int a,
+                                                             int b, int c, int d, int m_tiles, int n_tiles,
+                                                             int splits, int64_t cols_per_split)
+{
+    __shared__ float sa[16][17], sb[16][17];
+    int64_t t = blockIdx.x;
+    const int split = (int)(t % splits);
+    t /= splits;
+    const int nt = (int)(t % n_tiles);
+    t /= n_tiles;
+    const int mt = (int)(t % m_tiles);
+    const int64_t g = t / m_tiles;
+    const int a_i = (int)(g / d), d_i = (int)(g - (int64_t)a_i * d);
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int64_t in_size = (int64_t)a * c * d, out_size = (int64_t)a * b * d;
+    const int64_t n_begin = split * cols_per_split, n_end = min(batch, n_begin + cols_per_split);
+    // staging: thread (ty, tx) loads operand row ty, batch element n + tx (batch-size-last: tx runs
+    // along the contiguous axis) or row tx, batch element n + ty (batch-size-first: features contiguous)
+    const int lrow = BS_LAST ? ty : tx, lcol = BS_LAST ? tx : ty;
+    const int m_ld = mt * 16 + lrow, c_ld = nt * 16 + lrow;
+    const int64_t fa = ((int64_t)a_i * b + min(m_ld, b - 1)) * d + d_i;  // feature of dY
+    const int64_t fb = ((int64_t)a_i * c + min(c_ld, c - 1)) * d + d_i;  // feature of X
+    float acc = 0.f;
+    for (int64_t n = n_begin; n < n_end; n += 16) {
+        const int64_t nn = n + lcol;
+        float va = 0.f, vb = 0.f;
+        if (nn < n_end) {
+            va = elem<T>::load(BS_LAST ? dy + fa * batch + nn : dy + nn * out_size + fa);
+            vb = elem<T>::load(BS_LAST ? x + fb * batch + nn : x + nn * in_size + fb);
+        }
+        sa[lrow][lcol] = va;
+        sb[lrow][lcol] = vb;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; ++k) acc += sa[tx][k] * sb[ty][k];
+        __syncthreads();
+    }
+    const int m = mt * 16 + tx, cc = nt * 16 + ty;  // consecutive threads: consecutive b_i (contiguous in dW)
+    if (m < b && cc < c) atomicAdd(acc_out + ((size_t)g * c + cc) * b + m, acc);
+}
+
+template <typename T> int launch_block_transpose(const void *w, void *wt, int64_t total, int b, int c, hipStream_t s)
+{
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((ks_block_transpose_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)w, (T *)wt,
+                       total, b, c);
+    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+template <typename T, int MT, int NT>
+int launch_wgrad_bl(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
+                    hipStream_t s)
+{
+    const int m_tiles = (b + 16 * MT - 1) / (16 * MT), n_tiles = (c + 16 * NT - 1) / (16 * NT);
+    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
+    constexpr int STEP = 4 * wg_vec<T>::N;
+    // about 16 waves per CU; at least 8 steps per wave
+    int64_t splits = (4096 + tiles - 1) / tiles;
+    const int64_t max_splits = (batch + 8 * STEP - 1) / (8 * STEP);
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    int64_t cols = (batch + splits - 1) / splits;
+    cols = (cols + STEP - 1) / STEP * STEP;
+    splits = (batch + cols - 1) / cols;
+    const int64_t waves = tiles * splits, blocks = (waves + 3) / 4;
+    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((ks_wgrad_bl_kernel<T, MT, NT>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
+                       (const T *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols);
+    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_wgrad_tiled(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
+                       int bs_last, hipStream_t s)
+{
+    const int m_tiles = (b + 15) / 16, n_tiles = (c + 15) / 16;
+    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
+    int64_t splits = (2048 + tiles - 1) / tiles;
+    const int64_t max_splits = (batch + 255) / 256;
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    int64_t cols = (batch + splits - 1) / splits;
+    cols = (cols + 15) / 16 * 16;
+    splits = (batch + cols - 1) / cols;
+    const int64_t blocks = tiles * splits;
+    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (bs_last)
+        hipLaunchKernelGGL((ks_wgrad_tiled_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
+                           (const T *)x, acc, batch, a, b, c, d, m_tiles, n_tiles, (int)splits, cols);
+    else
+        hipLaunchKernelGGL((ks_wgrad_tiled_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
+                           (const T *)x, acc, batch, a, b, c, d, m_tiles, n_tiles, (int)splits, cols);
+    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace
+
+// wt <- the b x c blocks of w transposed: kernel format (a*d*b, c) of pattern (a, c, b, d)
+int block_transpose_run(const void *w, void *wt, int a, int b, int c, int d, int dtype, hipStream_t stream)
+{
+    const int64_t total = (int64_t)a * b * c * d;
+    switch (dtype) {
+    case KSMM_F32: return launch_block_transpose<float>(w, wt, total, b, c, stream);
+    case KSMM_F16: return launch_block_transpose<half_t>(w, wt, total, b, c, stream);
+    case KSMM_FP8_E4M3: return launch_block_transpose<uint8_t>(w, wt, total, b, c, stream);
+    default: return KSMM_ERR_BAD_DTYPE;
+    }
+}
+
+// dw (kernel format, type `dtype`) <- scale * sum over the batch of dY x X^T per block; acc is an
+// fp32 buffer of a*b*c*d elements (zeroed here).  tile_query: 1 = MFMA kernel, 0 = tiled kernel.
+int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch, int a, int b, int c, int d,
+              int dtype, int bs_last, float scale, hipStream_t stream, int *kernel_used)
+{
+    const int64_t n = (int64_t)a * b * c * d;
+    const int64_t fill_blocks = (n + 255) / 256;
+    if (fill_blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    const int vec = 16 / (int)dtype_size(dtype);
+    const bool mfma_ok = bs_last && batch % vec == 0 && ((((uintptr_t)dy | (uintptr_t)x) & 15) == 0) &&
+                         (int64_t)(b > c ? b : c) * d * batch < 0x7fffffffLL;
+    if (kernel_used) *kernel_used = mfma_ok ? 1 : 0;
+    hipLaunchKernelGGL(ks_fill_zero_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, stream, acc, n);
+    if (hipGetLastError() != hipSuccess) return KSMM_ERR_LAUNCH;
+    int rc;
+    if (dtype == KSMM_F32) {
+        if (mfma_ok)
+            rc = (b <= 16 && c <= 16) ? launch_wgrad_bl<float, 1, 1>(dy, x, acc, batch, a, b, c, d, stream)
+                 : (b <= 32 && c <= 32) ? launch_wgrad_bl<float, 2, 2>(dy, x, acc, batch, a, b, c, d, stream)
+                 : (b % 64 && c % 64 && b % 48 == 0 && c % 48 == 0) ? launch_wgrad_bl<float, 3, 3>(dy, x, acc, batch, a, b, c, d, stream)
+                                                                    : launch_wgrad_bl<float, 4, 4>(dy, x, acc, batch, a, b, c, d, stream);
+        else
+            rc = launch_wgrad_tiled<float>(dy, x, acc, batch, a, b, c, d, bs_last, stream);
+    } else if (dtype == KSMM_F16) {
+        if (mfma_ok)
+            rc = (b <= 16 && c <= 16) ? launch_wgrad_bl<half_t, 1, 1>(dy, x, acc, batch, a, b, c, d, stream)
+                 : (b <= 32 && c <= 32) ? launch_wgrad_bl<half_t, 2, 2>(dy, x, acc, batch, a, b, c, d, stream)
+                 : (b % 64 && c % 64 && b % 48 == 0 && c % 48 == 0) ? launch_wgrad_bl<half_t, 3, 3>(dy, x, acc, batch, a, b, c, d, stream)
+                                                                    : launch_wgrad_bl<half_t, 4, 4>(dy, x, acc, batch, a, b, c, d, stream);
+        else
+            rc = launch_wgrad_tiled<half_t>(dy, x, acc, batch, a, b, c, d, bs_last, stream);
+    } else {
+        return KSMM_ERR_BAD_DTYPE;
+    }
+    if (rc != KSMM_OK) return rc;
+    if (dtype == KSMM_F32)
+        hipLaunchKernelGGL((ks_wgrad_finish_kernel<float>), dim3((unsigned)fill_blocks), dim3(256), 0, stream, acc,
+                           (float *)dw, n, scale);
+    else
+        hipLaunchKernelGGL((ks_wgrad_finish_kernel<half_t>), dim3((unsigned)fill_blocks), dim3(256), 0, stream, acc,
+                           (half_t *)dw, n, scale);
+    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+}  // namespace ksmm

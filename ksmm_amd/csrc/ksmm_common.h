@@ -167,6 +167,12 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  /
 int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 
+// Backward pass pieces (ksmm_backward.hip): blockwise transpose of a kernel-format weight, and the
+// weight gradient (acc: fp32 scratch of a*b*c*d elements; kernel_used: 1 MFMA kernel, 0 tiled).
+int block_transpose_run(const void *w, void *wt, int a, int b, int c, int d, int dtype, hipStream_t stream);
+int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch, int a, int b, int c, int d,
+              int dtype, int bs_last, float scale, hipStream_t stream, int *kernel_used);
+
 // Fused radix-16 chain (intermediates in LDS); KSMM_ERR_BAD_ALGO when the chain does not qualify.
 int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream);
 int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_t batch, int x_dtype,

@@ -25,6 +25,8 @@
 // Reference counterpart: kernel_bs_{first,last}_{float,half2,half4}
 // (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-491,
 //  template_kernels_half.cuh:103-1092).
+#include <type_traits>
+
 #include "ksmm_mfma.h"
 
 
@@ -155,7 +157,7 @@ template <int COLS> struct outer_frag<float, COLS> {
     }
 };
 
-template <typename CT, typename TY, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool KT>
+template <typename CT, typename TY, bool BS_LAST, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool KT, bool EPI>
 __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__restrict__ x,
                                                               const CT *__restrict__ w,
                                                               TY *__restrict__ y, int batch, int a,
@@ -163,7 +165,9 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
                                                               int m_tiles, int n_tiles, int blocks, int pf_dist)
 {
     const float scale = ep.scale;
-    const bool has_epi = ep.bias != nullptr || ep.act != KSMM_ACT_NONE;  // uniform
+    // bias and activation live in an instantiation of their own: next to the accumulators their
+    // registers would push the plain one into scratch memory
+    constexpr bool has_epi = EPI;
     typedef GemmCfg<CT, BS_LAST, DD, TM, TN, TK, WM, WN, ST> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     // XCD-aware id: TM-tiles of one input tile get consecutive logical ids on one XCD
@@ -309,10 +313,30 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
     for (int p = 0; p < ST - 1; ++p) issue(min(p, steps - 1), p);
 
-    // MFMA operands of sub-step k0 of the slab whose operand addresses are wa[] / xa[]
+    // MFMA operands of sub-step k0 of the slab whose operand addresses are wa[] / xa[].  Reading
+    // them from LDS (read_frags) and making input operands of what was read (split_x) are separate
+    // steps: for d == 2 the latter needs the data, and placed right behind the reads it would make
+    // the wave wait out the LDS latency before it may issue the MFMAs that are already due.
     typedef typename frag<CT>::type frag_t;
-    auto load_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[DD][C::MT],
-                          frag_t(&fx)[DD][C::NT]) {
+    constexpr bool PAIRS = !BS_LAST && DD == 2;  // input rows hold (k, d_i) pairs
+    // (16 waves leave 128 registers a lane: no room to keep pairs and operands side by side)
+    constexpr bool LATE_SPLIT = PAIRS && C::THREADS <= 512;
+    struct XPairs {
+        uint4_t lo, hi;  // 16 consecutive halves = 8 (k, d_i) pairs; split early: the two operands
+    };
+    auto split_pairs = [](const uint4_t lo, const uint4_t hi, uint4_t &e, uint4_t &o) {
+        e[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100u);
+        e[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x05040100u);
+        e[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x05040100u);
+        e[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x05040100u);
+        o[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u);
+        o[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07060302u);
+        o[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07060302u);
+    };
+    typedef typename std::conditional<PAIRS, XPairs, frag_t>::type xraw_t;
+    auto read_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[DD][C::MT],
+                          xraw_t(&xr)[C::NT]) {
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
@@ -321,27 +345,35 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
         for (int j = 0; j < C::NT; ++j) {
             if constexpr (BS_LAST) {
-                fx[0][j] = outer_frag<CT, TN>::read(xa[j], k0);
+                xr[j] = outer_frag<CT, TN>::read(xa[j], k0);
             } else if constexpr (DD == 1) {
                 typedef __attribute__((address_space(3))) half8_t *lds_ptr;
-                fx[0][j] = *(lds_ptr)(lds_bytes_t)(uintptr_t)(xa[j] ^ ((k0 >> 3) << 4));
+                xr[j] = *(lds_ptr)(lds_bytes_t)(uintptr_t)(xa[j] ^ ((k0 >> 3) << 4));
             } else {
-                // 16 consecutive halves = 8 (k, d_i) pairs -> one operand per d_i
                 typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
                 const uint32_t pa = xa[j] ^ ((k0 >> 2) << 4);
                 const uint4_t lo = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa);
                 const uint4_t hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ 16);
-                uint4_t e, o;
-                e[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100u);
-                e[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x05040100u);
-                e[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x05040100u);
-                e[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x05040100u);
-                o[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u);
-                o[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u);
-                o[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07060302u);
-                o[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07060302u);
+                if constexpr (LATE_SPLIT) {
+                    xr[j].lo = lo;
+                    xr[j].hi = hi;
+                } else {
+                    split_pairs(lo, hi, xr[j].lo, xr[j].hi);
+                }
+            }
+        }
+    };
+    auto split_x = [&](const xraw_t(&xr)[C::NT], frag_t(&fx)[DD][C::NT]) {
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            if constexpr (PAIRS) {
+                // one operand per d_i
+                uint4_t e = xr[j].lo, o = xr[j].hi;
+                if constexpr (LATE_SPLIT) split_pairs(xr[j].lo, xr[j].hi, e, o);
                 fx[0][j] = __builtin_bit_cast(half8_t, e);
                 fx[DD - 1][j] = __builtin_bit_cast(half8_t, o);
+            } else {
+                fx[0][j] = xr[j];
             }
         }
     };
@@ -357,7 +389,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     // sub-step multiplies; operands of sub-step k0+1 are read while k0 multiplies.
     constexpr int SLOTS = (K0 - 1) * PER_K0;
     constexpr int STRIDE = SLOTS / C::L > 0 ? SLOTS / C::L : 1;  // MFMAs per load issued
-    frag_t fw[2][DD][C::MT], fx[2][DD][C::NT];
+    frag_t fw[2][DD][C::MT], fx[DD][C::NT];
+    xraw_t xr[2][C::NT];
     uint32_t wa[C::MT], xa[C::NT];
     auto stage_addrs = [&](int stg) {
         const uint32_t base = lds_base + stg * C::STAGE_BYTES;
@@ -378,7 +411,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     if (KT && steps == 1 && rem < TK) clear_tail(0);
     __syncthreads();  // slab 0 landed for every wave
     stage_addrs(0);
-    load_frags(wa, xa, 0, fw[0], fx[0]);
+    read_frags(wa, xa, 0, fw[0], xr[0]);
 
     for (int it = 0; it < steps; ++it) {
         const int nstep = min(it + ST - 1, steps - 1);
@@ -396,24 +429,26 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
         for (int kk = 0; kk < K0; ++kk) {
             if (kk + 1 < K0) {
-                load_frags(wa, xa, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], fx[(kk + 1) & 1]);
+                read_frags(wa, xa, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], xr[(kk + 1) & 1]);
             } else {
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(C::N_WAIT));
                 if (KT && it + 2 == steps && rem < TK) clear_tail((it + 1) % ST);
                 __syncthreads();  // slab it+1 landed for every wave, and everyone left slab it
                 if (it + 1 < steps) {
                     stage_addrs((it + 1) % ST);
-                    load_frags(wa, xa, 0, fw[0], fx[0]);
+                    read_frags(wa, xa, 0, fw[0], xr[0]);
                 }
+                __builtin_amdgcn_sched_barrier(0);  // requested before this sub-step multiplies
             }
+            split_x(xr[kk & 1], fx);
 #pragma unroll
             for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
                 for (int i = 0; i < C::MT; ++i)
 #pragma unroll
                     for (int j = 0; j < C::NT; ++j) {
-                        acc[dd][i][j] = BS_LAST ? frag<CT>::mfma(fx[kk & 1][dd][j], fw[kk & 1][dd][i], acc[dd][i][j])
-                                                : frag<CT>::mfma(fw[kk & 1][dd][i], fx[kk & 1][dd][j], acc[dd][i][j]);
+                        acc[dd][i][j] = BS_LAST ? frag<CT>::mfma(fx[dd][j], fw[kk & 1][dd][i], acc[dd][i][j])
+                                                : frag<CT>::mfma(fw[kk & 1][dd][i], fx[dd][j], acc[dd][i][j]);
                         const int m = kk * PER_K0 + (dd * C::MT + i) * C::NT + j;  // MFMA index in the slab
                         if (kk + 1 < K0 && (m + 1) % STRIDE == 0 && m / STRIDE < C::L) {
                             issue_one(m / STRIDE);
@@ -450,35 +485,42 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
         // bias and activation act on the accumulators in place, before the tile is written out;
         // the passes below then store them as they are
         float st_scale = scale;
-        if (has_epi) {
+        if constexpr (has_epi) {
+            const bool gelu = ep.act == KSMM_ACT_GELU;
 #pragma unroll
-            for (int i = 0; i < C::MT; ++i)
+            for (int i = 0; i < C::MT; ++i) {
+                const int mb = (wm * C::MT + i) * 32;
+                if constexpr (BS_LAST) {
+                    // the lane's row is one output feature
+                    const float bl = epi_bias<TY>(ep, ((size_t)a_i * b + m0 + mb + l32) * d + d_i);
 #pragma unroll
-                for (int j = 0; j < C::NT; ++j) {
-                    const int mb = (wm * C::MT + i) * 32, nb = (wn * C::NT + j) * 32;
-                    // bs_last: the lane's row is one output feature; bs_first: element u of group eg
-                    // is output m0 + mb + 4*lq + 8*eg + u (x DD interleaved d_i)
-                    const size_t f0 = BS_LAST ? ((size_t)a_i * b + m0 + mb + l32) * d + d_i
-                                              : ((size_t)a_i * b + m0 + mb + 4 * lq) * DD;
-                    const float bl = BS_LAST ? epi_bias<TY>(ep, f0) : 0.f;
-                    (void)nb;
-#pragma unroll
-                    for (int dd = 0; dd < DD; ++dd)
+                    for (int j = 0; j < C::NT; ++j)
 #pragma unroll
                         for (int e = 0; e < 16; ++e) {
-                            const float bv = BS_LAST ? bl : epi_bias<TY>(ep, f0 + (size_t)(8 * (e >> 2) + (e & 3)) * DD + dd);
-                            acc[dd][i][j][e] = fmaf(acc[dd][i][j][e], scale, bv);
+                            const float v = fmaf(acc[0][i][j][e], scale, bl);
+                            acc[0][i][j][e] = gelu ? gelu_erf(v) : v;
                         }
-                }
-            if (ep.act == KSMM_ACT_GELU) {
+                } else {
+                    // element u of group eg is output m0 + mb + 4*lq + 8*eg + u (x DD interleaved
+                    // d_i): the lane's 4 * DD bias values of a group are consecutive, one vector load
+                    static_assert(BS_LAST || sizeof(TY) == 2, "batch-size-first tiles write fp16");
+                    typedef TY bias_v __attribute__((ext_vector_type(4 * DD)));
+                    const size_t f0 = ((size_t)a_i * b + m0 + mb + 4 * lq) * DD;
 #pragma unroll
-                for (int dd = 0; dd < DD; ++dd)
-#pragma unroll
-                    for (int i = 0; i < C::MT; ++i)
+                    for (int eg = 0; eg < 4; ++eg) {
+                        bias_v bb = {};
+                        if (ep.bias) bb = *(const bias_v *)((const TY *)ep.bias + f0 + 8 * eg * DD);
 #pragma unroll
                         for (int j = 0; j < C::NT; ++j)
 #pragma unroll
-                            for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = gelu_erf(acc[dd][i][j][e]);
+                            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                                for (int dd = 0; dd < DD; ++dd) {
+                                    const float v = fmaf(acc[dd][i][j][4 * eg + u], scale, (float)bb[u * DD + dd]);
+                                    acc[dd][i][j][4 * eg + u] = gelu ? gelu_erf(v) : v;
+                                }
+                    }
+                }
             }
             st_scale = 1.f;
         }
@@ -536,11 +578,362 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
     }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Persistent form for fp16 batch-size-first blocks with d == 2: the same tile, ring and MFMA
+// schedule as ks_gemm_kernel, with three differences that take the per-tile overheads out:
+//  * a workgroup stays on its CU and walks through its tiles; the slab stream of the ring runs
+//    on across tile boundaries, so the next tile's first slabs arrive while the current tile is
+//    finished (no launch gap, no exposed first-slab latency);
+//  * the lower half of the waves issues every direct-to-LDS load, so the other half never waits
+//    on the vector-memory counter.  Operations of one wave complete in the order they were
+//    issued: after a tile's output stores a loader's first wait also covers those stores, which
+//    have had a slab's time to complete by then;
+//  * the output tile leaves through the ring stage that has just been consumed (the other
+//    stages already hold the next tile's slabs): every wave turns its 32x32 blocks around in a
+//    private piece of it and stores whole 128-byte lines, without a workgroup barrier.
+// All waves multiply and store their own part of the output.
+template <typename CT, typename TY, int DD, int TM, int TN, int TK, int WM, int WN, int ST, bool EPI>
+__global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbf_kernel(const CT *__restrict__ x,
+                                                                const CT *__restrict__ w,
+                                                                TY *__restrict__ y, int batch, int a,
+                                                                int b, int c, int d, Epi ep,
+                                                                int m_tiles, int n_tiles, int blocks)
+{
+    typedef GemmCfg<CT, false, DD, TM, TN, TK, WM, WN, ST> C;
+    constexpr int NWAVES = WM * WN, LOADERS = 64 * (NWAVES / 2);      // loader threads (lower half)
+    constexpr int LW = C::W_CHUNKS / LOADERS, LX = C::X_CHUNKS / LOADERS, L = LW + LX;
+    constexpr int N_WAIT = (ST - 2) * L;
+    static_assert(NWAVES % 2 == 0 && C::W_CHUNKS % LOADERS == 0 && C::X_CHUNKS % LOADERS == 0, "loader split");
+    static_assert(ST >= 3 && N_WAIT <= 63, "ring");
+    static_assert(sizeof(CT) == 2 && sizeof(TY) == 2, "fp16 only");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const float scale = ep.scale;
+    // bias and activation live in an instantiation of their own: next to the accumulators their
+    // registers would push the plain one into scratch memory
+    constexpr bool has_epi = EPI;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const bool loader = wave < NWAVES / 2;  // uniform per wave
+    const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
+
+    // ---- the tiles of this workgroup: XCD blockIdx % 8 owns a contiguous eighth of the logical
+    // tile ids (TM-tile fastest, then batch tile, then a_i), its workgroup blockIdx / 8 takes
+    // every slots-th one: the workgroups of an XCD work on neighbouring ids at any one time, so
+    // the TM-tiles of one input tile share it through that XCD's L2
+    const int per_xcd = (blocks + 7) / 8;
+    const int slots = (int)gridDim.x / 8;  // the grid is a multiple of 8
+    const int xcd_first = ((int)blockIdx.x % 8) * per_xcd;
+    const int xcd_end = min(xcd_first + per_xcd, blocks);
+    const int first = xcd_first + (int)blockIdx.x / 8;
+    if (first >= xcd_end) return;
+    const int my_tiles = (xcd_end - first + slots - 1) / slots;
+    struct Tile {
+        int m0, n0, a_i;
+    };
+    auto decode = [&](int t) {
+        const int lid = first + t * slots;
+        const int mt_id = lid % m_tiles, rest = lid / m_tiles;
+        return Tile{mt_id * TM, (rest % n_tiles) * TN, rest / n_tiles};
+    };
+
+    // ---- load side (loader waves): a stream of slabs that runs ST-1 slabs ahead of the
+    // multiplication, across tile boundaries.  uniform base + 32-bit per-lane offset
+    const int steps = c / TK;
+    const size_t w_step = (size_t)TK * b * C::ES, x_step = (size_t)TK * DD * C::ES;  // bytes per slab
+    // Weight chunk i of a lane is LOADERS chunks = W_ROWS_PER rows further down than chunk i - 1,
+    // in the same column and with the same swizzle (a multiple of 4 rows), and after LW_PER_DD
+    // chunks it moves on to the next d_i: one per-lane offset, the rest are uniform additions.
+    constexpr int W_ROWS_PER = LOADERS / C::W_CPR, LW_PER_DD = LW / DD;
+    static_assert(LOADERS % C::W_CPR == 0 && W_ROWS_PER % 4 == 0 && LW % DD == 0 && W_ROWS_PER * LW_PER_DD == TK,
+                  "uniform weight chunk strides");
+    uint32_t wvoff0, xvoff[LX];
+    {
+        const int q = tid & (LOADERS - 1);
+        const int row = q / C::W_CPR, pc = q % C::W_CPR;
+        const int col = (pc ^ swz_outer<CT, C::W_CPR>(row)) * C::EPC;
+        wvoff0 = (uint32_t)(((size_t)row * b + col) * C::ES);
+    }
+    const size_t w_chunk_step = (size_t)W_ROWS_PER * b * C::ES, w_dd_step = (size_t)c * b * C::ES;
+    const char *i_w = nullptr, *i_x = nullptr;  // slab the load side is at
+    int i_t = 0, i_k = 0;
+    auto i_open = [&](int t) {
+        const Tile q = decode(t);
+        i_w = (const char *)(w + ((size_t)(q.a_i * DD) * c) * b + q.m0);
+        i_x = (const char *)(x + (size_t)q.n0 * in_size + (size_t)q.a_i * c * DD);
+        // the last batch tile repeats its last row instead of reading past the end
+        int tid_ = tid & (LOADERS - 1);
+        asm volatile("" : "+v"(tid_));
+#pragma unroll
+        for (int i = 0; i < LX; ++i) {
+            const int qq = tid_ + i * LOADERS;
+            const int row = qq / C::X_CPR, pc = qq % C::X_CPR;
+            const int col = (pc ^ swz_inner<C::X_CPR>(row)) * C::EPC;
+            xvoff[i] = (uint32_t)(((size_t)min(row, batch - 1 - q.n0) * in_size + col) * C::ES);
+        }
+    };
+    // next slab of the stream; after the last one the load side stays there (the ring then
+    // receives repeats of it, which keeps the number of loads per slab constant)
+    auto i_advance = [&]() {
+        if (i_k + 1 < steps) {
+            ++i_k;
+            i_w += w_step;
+            i_x += x_step;
+        } else if (i_t + 1 < my_tiles) {
+            ++i_t;
+            i_k = 0;
+            i_open(i_t);
+        }
+    };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    auto issue_one = [&](const char *wsrc, const char *xsrc, uint32_t dst, int q) {
+        // dst: stage base + this wave's kilobyte; chunk q of the lane
+        if (q < LW)
+            dma16s(wsrc + (q / LW_PER_DD) * w_dd_step + (q % LW_PER_DD) * w_chunk_step, wvoff0, dst + q * (LOADERS * 16));
+        else
+            dma16s(xsrc, xvoff[q >= LW ? q - LW : 0], dst + C::W_BYTES + (q - LW) * (LOADERS * 16));
+    };
+
+    // ---- per-lane byte offsets of the MFMA operands inside a stage (sub-step 0) --------------
+    uint32_t woff[C::MT], xoff[C::NT];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i) woff[i] = outer_frag<CT, TM>::off((wm * C::MT + i) * 32, lane);
+#pragma unroll
+    for (int j = 0; j < C::NT; ++j) {
+        const int row = (wn * C::NT + j) * 32 + (lane & 31), lq = lane >> 5;
+        xoff[j] = C::W_BYTES + row * (TK * DD * 2) + (((DD == 2 ? 2 * lq : lq) ^ swz_inner<C::X_CPR>(row)) << 4);
+    }
+    float16_t acc[DD][C::MT][C::NT];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = 0.f;
+    };
+    clear_acc();
+
+    i_open(0);
+#pragma unroll
+    for (int p = 0; p < ST - 1; ++p) {
+        if (loader) {
+            const uint32_t dst = lds_base + p * C::STAGE_BYTES + wave * 1024;
+#pragma unroll
+            for (int q = 0; q < L; ++q) issue_one(i_w, i_x, dst, q);
+        }
+        i_advance();
+    }
+
+    // reading operands from LDS and splitting the (k, d_i) pairs of the input rows into one
+    // operand per d_i are separate steps, as in ks_gemm_kernel
+    typedef typename frag<CT>::type frag_t;
+    struct XPairs {
+        uint4_t lo, hi;
+    };
+    auto read_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[DD][C::MT],
+                          XPairs(&xr)[C::NT]) {
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+                fw[dd][i] = outer_frag<CT, TM>::read(wa[i] + dd * (TK * TM * C::ES), k0);
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
+            const uint32_t pa = xa[j] ^ ((k0 >> 2) << 4);
+            xr[j].lo = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa);
+            xr[j].hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ 16);
+        }
+    };
+    auto split_x = [&](const XPairs(&xr)[C::NT], frag_t(&fx)[DD][C::NT]) {
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            const uint4_t lo = xr[j].lo, hi = xr[j].hi;
+            uint4_t e, o;
+            e[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100u);
+            e[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x05040100u);
+            e[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x05040100u);
+            e[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x05040100u);
+            o[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u);
+            o[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u);
+            o[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07060302u);
+            o[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07060302u);
+            fx[0][j] = __builtin_bit_cast(half8_t, e);
+            fx[1][j] = __builtin_bit_cast(half8_t, o);
+        }
+    };
+    constexpr int K0 = TK / C::KSTEP;           // MFMA sub-steps per slab
+    constexpr int PER_K0 = DD * C::MT * C::NT;  // MFMAs per sub-step
+    static_assert(K0 >= 2 && K0 % 2 == 0, "operand double buffer alternates inside a slab");
+    constexpr int SLOTS = (K0 - 1) * PER_K0;
+    constexpr int STRIDE = SLOTS / L > 0 ? SLOTS / L : 1;  // MFMAs per load issued (loader waves)
+    frag_t fw[2][DD][C::MT], fx[DD][C::NT];
+    XPairs xr[2][C::NT];
+    uint32_t wa[C::MT], xa[C::NT];
+    auto stage_addrs = [&](int stg) {
+        const uint32_t base = lds_base + stg * C::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i) {
+            wa[i] = woff[i] + base;
+            asm volatile("" : "+v"(wa[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            xa[j] = xoff[j] + base;
+            asm volatile("" : "+v"(xa[j]));
+        }
+    };
+    if (loader) __builtin_amdgcn_s_waitcnt(vmcnt_imm(N_WAIT));
+    __syncthreads();  // slab 0 landed
+    stage_addrs(0);
+    read_frags(wa, xa, 0, fw[0], xr[0]);
+
+    const int l32 = lane & 31, lq = lane >> 5;
+    constexpr int OP = 128 + 16;  // bytes per row of a wave's output piece
+    static_assert(DD == 2 && NWAVES * 32 * OP <= C::STAGE_BYTES, "output pieces fit the consumed stage");
+
+    constexpr int TILE_STORES = C::MT * C::NT * 4;  // stores of a wave per full tile
+    static_assert(N_WAIT + TILE_STORES <= 63, "counter range");
+    bool stores_behind = false;  // the previous tile issued exactly TILE_STORES stores (uniform)
+    Tile cur = decode(0);
+    int stg = 0;  // ring stage of the slab being multiplied
+    for (int c_t = 0; c_t < my_tiles; ++c_t) {
+        for (int c_k = 0; c_k < steps; ++c_k) {
+            const char *const wsrc = i_w;
+            const char *const xsrc = i_x;
+            const int stg_fill = stg == 0 ? ST - 1 : stg - 1;  // stage of the slab ST-1 ahead
+            const int stg_next = stg + 1 == ST ? 0 : stg + 1;
+            const uint32_t dst = lds_base + stg_fill * C::STAGE_BYTES + wave * 1024;
+#pragma unroll
+            for (int kk = 0; kk < K0; ++kk) {
+                if (kk + 1 < K0) {
+                    read_frags(wa, xa, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], xr[(kk + 1) & 1]);
+                } else {
+                    if (loader) {
+                        // behind the next slab's loads the counter holds the loads of the slab after
+                        // it and, on the first slab of a tile, the previous tile's output stores
+                        if (c_k == 0 && stores_behind)
+                            __builtin_amdgcn_s_waitcnt(vmcnt_imm(N_WAIT + TILE_STORES));
+                        else
+                            __builtin_amdgcn_s_waitcnt(vmcnt_imm(N_WAIT));
+                    }
+                    __syncthreads();  // the next slab has landed, and everyone has left this one
+                    // (at the end of a tile the next tile's first operands are read after its output
+                    // has left: their registers are needed for that)
+                    if (c_k + 1 < steps) {
+                        stage_addrs(stg_next);
+                        read_frags(wa, xa, 0, fw[0], xr[0]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);  // requested before this sub-step multiplies
+                }
+                split_x(xr[kk & 1], fx);
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+                    for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                        for (int j = 0; j < C::NT; ++j) {
+                            acc[dd][i][j] = frag<CT>::mfma(fw[kk & 1][dd][i], fx[dd][j], acc[dd][i][j]);
+                            const int m = kk * PER_K0 + (dd * C::MT + i) * C::NT + j;  // MFMA index in the slab
+                            if (kk + 1 < K0 && (m + 1) % STRIDE == 0 && m / STRIDE < L) {
+                                if (loader) issue_one(wsrc, xsrc, dst, m / STRIDE);
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+                        }
+                if (kk == K0 - 2) {
+                    // loads that did not get a slot above (fewer MFMAs than loads)
+                    if (loader) {
+#pragma unroll
+                        for (int q = SLOTS / STRIDE; q < L; ++q) issue_one(wsrc, xsrc, dst, q);
+                    }
+                }
+            }
+            i_advance();
+            if (c_k + 1 < steps) stg = stg_next;
+        }
+        // ---- the tile is complete.  Stage `stg` is consumed (every wave passed the barrier of its
+        // last sub-step, so nobody reads it any more) and the other stages already hold slabs of
+        // the next tile: each wave takes a private piece of it to turn its 32x32 blocks around.
+        // In the accumulators a lane holds, per group eg, 4 outputs x 2 d_i of one batch row =
+        // 16 of the row's 128 bytes; written like that a store touches 32 lines.  Through the
+        // private piece (OP bytes per row: 16 lanes of a vector access fall on distinct banks)
+        // eight neighbouring lanes get the eight pieces of a row: whole lines, 8 per store.
+        // LDS accesses of one wave execute in order, so the piece needs no barrier.
+        if constexpr (has_epi) {
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i) {
+                const size_t f0 = ((size_t)cur.a_i * b + cur.m0 + (wm * C::MT + i) * 32 + 4 * lq) * DD;
+#pragma unroll
+                for (int eg = 0; eg < 4; ++eg) {
+                    // the lane's 8 bias values of this group: (4 outputs) x (2 d_i), one 16-byte load
+                    half8_t bb = {0, 0, 0, 0, 0, 0, 0, 0};
+                    if (ep.bias) bb = *(const half8_t *)((const TY *)ep.bias + f0 + 16 * eg);
+#pragma unroll
+                    for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int dd = 0; dd < DD; ++dd) {
+                                const float v = fmaf(acc[dd][i][j][4 * eg + u], scale, (float)bb[2 * u + dd]);
+                                acc[dd][i][j][4 * eg + u] = ep.act == KSMM_ACT_GELU ? gelu_erf(v) : v;
+                            }
+                }
+            }
+        }
+        const float st_scale = has_epi ? 1.f : scale;
+        {
+            unsigned char *const piece = smem + stg * C::STAGE_BYTES + wave * (32 * OP);
+            unsigned char *const wr = piece + l32 * OP + 16 * lq;           // + 32 * eg
+            const unsigned char *const rd = piece + (lane >> 3) * OP + 16 * (lane & 7);  // + 8 * t rows
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j) {
+                    const int mb = (wm * C::MT + i) * 32, nb = (wn * C::NT + j) * 32;
+#pragma unroll
+                    for (int eg = 0; eg < 4; ++eg) {
+                        half8_t v;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            v[2 * u] = (half_t)(acc[0][i][j][4 * eg + u] * st_scale);
+                            v[2 * u + 1] = (half_t)(acc[1][i][j][4 * eg + u] * st_scale);
+                        }
+                        *(half8_t *)(wr + 32 * eg) = v;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                    const int n = cur.n0 + nb + (lane >> 3);  // + 8 * t
+                    TY *const dstp = y + (size_t)n * out_size + ((size_t)cur.a_i * b + cur.m0 + mb) * DD + 8 * (lane & 7);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const uint4_t v = *(const uint4_t *)(rd + 8 * t * OP);
+                        if (n + 8 * t < batch) __builtin_nontemporal_store(v, (uint4_t *)(dstp + (size_t)8 * t * out_size));
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+        }
+        stores_behind = cur.n0 + TN <= batch;  // a ragged tile skips stores: then wait the safe way
+        if (c_t + 1 < my_tiles) {
+            __syncthreads();  // every private piece is read: the stage may receive slabs again
+            clear_acc();
+            cur = decode(c_t + 1);
+            stg = stg + 1 == ST ? 0 : stg + 1;
+            stage_addrs(stg);
+            read_frags(wa, xa, 0, fw[0], xr[0]);
+        }
+    }
+    if (loader) __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // repeats of the last slab must land before LDS is released
+}
+
 struct GemmInst {
     int combo, bs_last, dd, tm, tn, tk, threads, lds, epc;
     int ktail;  // takes c that is not a multiple of tk
     int wm;     // waves along the TM side
-    const void *fn;
+    int pers;   // persistent workgroups with split memory roles (ks_gemm_pbf_kernel)
+    const void *fn[2];  // plain, with bias/activation
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
 // so that one multiplies while the other stores its output tile)
@@ -548,7 +941,12 @@ struct GemmInst {
     {COMBO_, BL_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_,                                                \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES,                                 \
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::EPC,                                       \
-     KT_, WM_, (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_>}
+     KT_, WM_, 0, {(const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_, false>, \
+                   (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_, true>}}
+#define GEMM_INST_P(DD_, TM_, TN_, TK_, WM_, WN_, ST_)                                                \
+    {1, false, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
+     8, 0, WM_, 1, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, false>, \
+                    (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
 #define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
     GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
@@ -603,6 +1001,9 @@ const GemmInst gemm_insts[] = {
     // fp16, bs_first, d == 2: 16 waves on the 256 x 128 tile (4 per SIMD: more to issue from while
     // others wait at the slab barrier)
     GEMM_INST(1, half_t, false, 2, 256, 128, 32, 4, 4, 3),
+    // fp16, bs_first: persistent workgroups, loads and stores issued by different waves
+    GEMM_INST_P(2, 256, 128, 32, 4, 2, 3),
+    GEMM_INST_P(2, 128, 256, 32, 2, 4, 3),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
@@ -637,8 +1038,8 @@ uint32_t gemm_inst_id(int i)
     if (i < 0 || i >= N_GEMM_INSTS) return 0;
     const GemmInst &t = gemm_insts[i];
     // threads and the LDS footprint stand for the wave grid and the ring depth
-    const int v[10] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm};
-    return inst_hash('G', v, 10);
+    const int v[11] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm, t.pers};
+    return inst_hash('G', v, 11);
 }
 
 // variant: index into the instance table; -1: first that fits with enough workgroups to fill
@@ -655,6 +1056,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         // kernels) and partial K slabs; otherwise the stream and weight-stationary tiles come
         // first, then these (variant -4: 15-25 % faster than the k-loop tiles on 180 patterns
         // of the reference's list), then the k-loop tiles
+        if (variant < 0 && t.pers) continue;  // measured choices only (the table names them)
         if (variant == -1 && t.tm < 128 && t.combo != 2 && !(t.ktail && p.c % t.tk)) continue;
         if (variant == -4 && t.tm >= 128) continue;  // -4: the TM = 64 tiles, after stream / weight-stationary
         // few K slabs: the 8-wave 256 x 256 tiles spend their time in prologue and epilogue; two
@@ -671,12 +1073,28 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         break;
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
+    if (variant < 0 && !gemm_insts[pick].pers) {
+        // three or more tiles per CU: the persistent form of the same tile saves the per-tile
+        // prologue and keeps the load stream running (8 % on (1,1536,384,2) at batch 25088)
+        const GemmInst &o = gemm_insts[pick];
+        const int64_t groups = o.dd == 1 ? (int64_t)p.a * p.d : p.a;
+        const int64_t wgs = groups * (p.b / o.tm) * ((p.batch + o.tn - 1) / o.tn);
+        for (int i = 0; i < N_GEMM_INSTS && wgs >= 3 * 256; ++i) {
+            const GemmInst &q = gemm_insts[i];
+            if (q.pers && q.combo == o.combo && q.bs_last == o.bs_last && q.dd == o.dd && q.tm == o.tm && q.tn == o.tn &&
+                q.tk == o.tk && gemm_fits(q, p, combo)) {
+                pick = i;
+                break;
+            }
+        }
+    }
     const GemmInst &t = gemm_insts[pick];
     const int m_tiles = p.b / t.tm;
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
     const int64_t groups = t.dd == 1 ? (int64_t)p.a * p.d : p.a;
     const int64_t blocks = groups * m_tiles * n_tiles;
-    const int64_t grid = (blocks + 7) / 8 * 8;
+    int64_t grid = (blocks + 7) / 8 * 8;
+    if (t.pers && grid > 256) grid = 256;  // one persistent workgroup per CU
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_TILE;
@@ -690,7 +1108,9 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->grid = grid;
     }
     if (!launch) return KSMM_OK;
-    if (ensure_dynamic_lds(t.fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
+    Epi ep = epi_of(p);
+    const void *fn = t.fn[ep.bias != nullptr || ep.act != KSMM_ACT_NONE];
+    if (ensure_dynamic_lds(fn, t.lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
     // L2 prefetch for the successor workgroup (bs_last): when the TM-tiles of an input tile can
     // cover it with PF lines per thread; distance = workgroups resident on an XCD (32 CUs)
@@ -702,10 +1122,15 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         const int64_t in_l2 = 2 * (int64_t)p.c * t.tn * es * ((resident + m_tiles - 1) / m_tiles);
         if (lines <= (int64_t)GEMM_PF * t.threads && in_l2 <= (5 << 19)) pf_dist = resident;
     }
-    Epi ep = epi_of(p);
+    if (t.pers) {
+        void *pargs[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
+                         (void *)&p.c, (void *)&p.d, &ep, &m_tiles_i, &n_tiles_i, &blocks_i};
+        hipError_t pe = hipLaunchKernel(fn, dim3((unsigned)grid), dim3(t.threads), pargs, t.lds, p.stream);
+        return pe == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+    }
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
                     (void *)&p.c, (void *)&p.d, &ep, &m_tiles_i, &n_tiles_i, &blocks_i, &pf_dist};
-    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
+    hipError_t e = hipLaunchKernel(fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 

@@ -123,6 +123,43 @@ class Kernel:
         return out
 
     @staticmethod
+    def backward(grad_output, input, factor, bs_last, a, b, c, d, scale=1.0, need_input=True, need_weight=True,
+                 workspace=None):
+        """(grad_input, grad_factor) of ``forward(input, factor, bs_last, a, b, c, d, scale=scale)``
+        for fp32 / fp16 tensors: grad_input = scale * K^T grad_output on the forward kernels (the
+        factor with pattern (a, c, b, d) and transposed blocks), grad_factor in kernel format
+        (a*d*c, b) from a reduction over the batch.  The reference's ``Kernel.backward``
+        (kernel.py:319-329) refers to an undefined symbol; this is the adjoint of its forward."""
+        lib = _lib.load()
+        for t, name in ((grad_output, "grad_output"), (input, "input"), (factor, "factor")):
+            _check_input(t, name)
+        bs_last = bool(bs_last)
+        assert input.dtype == factor.dtype == grad_output.dtype and input.dtype in (torch.float32, torch.float16)
+        batch = input.size(1 if bs_last else 0)
+        assert input.size(0 if bs_last else 1) == a * c * d and grad_output.size(0 if bs_last else 1) == a * b * d
+        assert grad_output.size(1 if bs_last else 0) == batch and tuple(factor.shape) == (a * c * d, b)
+        dt = dtype_code(input.dtype)
+        need = lib.ksmm_factor_backward_workspace(batch, a, b, c, d, dt, int(bs_last))
+        if need < 0:
+            _lib.check(int(need))
+        if workspace is None or workspace.numel() * workspace.element_size() < need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=input.device)
+        ws_bytes = workspace.numel() * workspace.element_size()
+        grad_input = grad_factor = None
+        with torch.cuda.device(input.device):
+            if need_input:
+                grad_input = torch.empty_like(input)
+                _lib.check(lib.ksmm_factor_backward_input(
+                    grad_output.data_ptr(), factor.data_ptr(), grad_input.data_ptr(), batch, a, b, c, d, dt,
+                    int(bs_last), float(scale), workspace.data_ptr(), ws_bytes, _stream_ptr(input)))
+            if need_weight:
+                grad_factor = torch.empty_like(factor)
+                _lib.check(lib.ksmm_factor_backward_weight(
+                    grad_output.data_ptr(), input.data_ptr(), grad_factor.data_ptr(), batch, a, b, c, d, dt,
+                    int(bs_last), float(scale), workspace.data_ptr(), ws_bytes, _stream_ptr(input)))
+        return grad_input, grad_factor
+
+    @staticmethod
     def chain_forward(input, factors, patterns, bs_last, scales=None, fuse=True, workspace=None,
                       bias=None, act=None, static_scratch=False, out=None):
         """All factors of a KSLinear in one call (factor-chain launcher).  ``bias``/``act`` are
@@ -179,6 +216,23 @@ class Kernel:
                                            int(bs_last), int(bool(fuse)), ep_ref, _stream_ptr(input))
         _lib.check(rc)
         return out
+
+
+class KSFactorFunction(torch.autograd.Function):
+    """One factor with a backward pass, for training through ``KSLinear(algo='kernel')``."""
+
+    @staticmethod
+    def forward(ctx, input, factor, bs_last, pattern):
+        ctx.save_for_backward(input, factor)
+        ctx.bs_last, ctx.pattern = bs_last, pattern
+        return Kernel.forward(input, factor, bs_last, *pattern)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, factor = ctx.saved_tensors
+        gi, gf = Kernel.backward(grad_output.contiguous(), input, factor, ctx.bs_last, *ctx.pattern,
+                                 need_input=ctx.needs_input_grad[0], need_weight=ctx.needs_input_grad[1])
+        return gi, gf, None, None
 
 
 def query_tile(batch, pattern, x_dtype, w_dtype=None, bs_last=True, algo=_lib.ALGO_AUTO, variant=-1):

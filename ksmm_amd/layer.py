@@ -175,6 +175,18 @@ class KSLinear(nn.Module):
     def _kernel_chain(self, x, x_scale):
         from .kernel import Kernel
 
+        if torch.is_grad_enabled() and self.dtype != FP8 and (
+                x.requires_grad or any(f.requires_grad for f in self.factors)):
+            # training: factor by factor through the autograd function (intermediates are kept for
+            # the weight gradients); bias and activation stay PyTorch ops so that autograd sees them
+            from .kernel import KSFactorFunction
+
+            out = x
+            for f, p in zip(self.factors, self.patterns):
+                out = KSFactorFunction.apply(out, f, self.bs_last, p)
+            if self.bias is not None:
+                out = out + self.bias
+            return F.gelu(out) if self.act == "gelu" else out
         scales = list(self.w_scales)
         if self.dtype == FP8:
             if x.dtype != FP8:

@@ -203,10 +203,10 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
 
 def _entry_id(e):
     """(instance id, parameter) of an entry; entries of older runs carry only the variant."""
-    if "id" in e:
-        return e["id"], e["param"]
     from .kernel import variant_id
 
+    # always from (family, variant) with the library at hand: the id recorded at measuring time
+    # belongs to the build that measured
     return variant_id(e["algo"], e["variant"], COMBO[e["prec"]], e["bs_last"])
 
 
@@ -261,9 +261,10 @@ def emit_best(entries, directory):
                 for e in sel:
                     a, b, c, d = e["pattern"]
                     use_best = e.get("best_us") is not None and e["algo"] != 0 and e["best_us"] <= e["auto_us"]
-                    if use_best and "id" in e:
+                    if use_best:
                         t = e.get("tile", {})
-                        fam, iid, par = FAMILY[e["algo"]], e["id"], e["param"]
+                        fam = FAMILY[e["algo"]]
+                        iid, par = _entry_id(e)
                         ms, std, mse = e.get("best_mean_us", e["best_us"]) / 1e3, e.get("best_std_us", 0.0) / 1e3, e.get("mse", float("nan"))
                     else:
                         t = e.get("auto_tile", {})

@@ -183,6 +183,24 @@ def chain_dense(w4_list):
     return dense
 
 
+def ks_backward(w4, x, dy, bs_last):
+    """Adjoints of y = K x for one factor, float64: (dX, dW4) with
+    dX[a,c,d,n] = sum_b W[a,b,c,d] dY[a,b,d,n]  (= K^T dY, the dense form of interface.py:108-113
+    transposed) and dW[a,b,c,d] = sum_n dY[a,b,d,n] X[a,c,d,n].  The reference has no backward
+    pass of its own (kernel.py:319-329, forward_bmm.py:12-15)."""
+    w4 = np.asarray(w4, dtype=np.float64)
+    x = np.asarray(x, dtype=np.float64)
+    dy = np.asarray(dy, dtype=np.float64)
+    a, b, c, d = w4.shape
+    if not bs_last:
+        x, dy = x.T, dy.T
+    n = x.shape[1]
+    x4, dy4 = x.reshape(a, c, d, n), dy.reshape(a, b, d, n)
+    dx = np.einsum("abdn,abcd->acdn", dy4, w4).reshape(a * c * d, n)
+    dw = np.einsum("abdn,acdn->abcd", dy4, x4)
+    return (dx if bs_last else dx.T), dw
+
+
 def rel_fro_error(y, z):
     """||y - z||_F / ||z||_F with z the oracle (scripts/example.py:22-23)."""
     y = np.asarray(y, dtype=np.float64)

@@ -314,7 +314,10 @@ def test_tuner_best_files_have_the_reference_columns(tmp_path):
     lines = (tmp_path / "kernel_bs_last_float.best").read_text().splitlines()
     assert lines[0].startswith("# batch a b c d family instance_id parameter")
     f = lines[1].split()
-    assert f[:8] == ["25088", "1", "48", "48", "16", "wave", "12345", "7"]
+    from ksmm_amd.kernel import variant_id
+
+    iid, par = variant_id(2, 0x700, 0, True)   # ids come from (family, variant) with the library at hand
+    assert f[:8] == ["25088", "1", "48", "48", "16", "wave", str(iid), str(par)] and par == 7
     assert float(f[13]) == pytest.approx(0.0342) and float(f[14]) == pytest.approx(0.0001) and float(f[15]) == 2e-14
     g = lines[2].split()
     assert g[:8] == ["25088", "2", "64", "64", "1", "wave", "0", "0"] and float(g[13]) == pytest.approx(0.0355)

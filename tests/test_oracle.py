@@ -249,3 +249,46 @@ def test_checker_fails_on_plausible_mistakes(tol_name):
     rng = np.random.default_rng(0)
     y = z * (1 + noise * rng.uniform(-1, 1, z.shape))
     assert O.rel_fro_error(y, z) <= tol
+
+
+@pytest.mark.parametrize("bs_last", [True, False])
+@pytest.mark.parametrize("pattern", [(2, 3, 5, 4), (1, 4, 3, 2), (3, 2, 2, 1)])
+def test_backward_matches_autograd_on_the_dense_form(pattern, bs_last):
+    """ks_backward against torch autograd through the explicit dense matrix (float64): dX is
+    K^T dY, dW is the gradient of the dense matrix read back on the factor's support; and a
+    central finite difference of one weight and one input entry."""
+    import torch
+
+    a, b, c, d = pattern
+    w4, x = _rand(pattern, 7, seed=3)
+    if not bs_last:
+        x = x.T.copy()
+    rng = np.random.default_rng(4)
+    dy = rng.standard_normal((a * b * d, 7)) if bs_last else rng.standard_normal((7, a * b * d))
+    dx, dw = O.ks_backward(w4, x, dy, bs_last)
+    with torch.enable_grad():
+        K = torch.tensor(O.ks_dense(w4), requires_grad=True)
+        xt = torch.tensor(x, requires_grad=True)
+        y = K @ xt if bs_last else xt @ K.T
+        (y * torch.tensor(dy)).sum().backward()
+    assert np.allclose(dx, xt.grad.numpy(), rtol=1e-12, atol=1e-12)
+    # dense gradient -> (a,b,c,d): entry ((i*b+j)*d+l, (i*c+k)*d+l)
+    gK = K.grad.numpy()
+    want = np.zeros_like(w4)
+    for i in range(a):
+        for j in range(b):
+            for k in range(c):
+                for l in range(d):
+                    want[i, j, k, l] = gK[(i * b + j) * d + l, (i * c + k) * d + l]
+    assert np.allclose(dw, want, rtol=1e-12, atol=1e-12)
+    f = lambda w, xx: float((O.ks_apply_einsum(w, xx, bs_last) * dy).sum())
+    eps = 1e-6
+    wp, wm = w4.copy(), w4.copy()
+    wp[a - 1, b - 1, 0, d - 1] += eps
+    wm[a - 1, b - 1, 0, d - 1] -= eps
+    assert (f(wp, x) - f(wm, x)) / (2 * eps) == pytest.approx(dw[a - 1, b - 1, 0, d - 1], rel=1e-6)
+    xp, xm = x.copy(), x.copy()
+    idx = (1, 2) if bs_last else (2, 1)
+    xp[idx] += eps
+    xm[idx] -= eps
+    assert (f(w4, xp) - f(w4, xm)) / (2 * eps) == pytest.approx(dx[idx], rel=1e-6)
