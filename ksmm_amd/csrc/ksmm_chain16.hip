@@ -72,26 +72,22 @@ __device__ __forceinline__ half4_t fp8x4_to_half4(uint32_t v)
 // FULL: 1024 features (every wave has MAXB blocks per factor) and a batch that is a multiple of
 // the chunk: no tile is ragged, so the chunk loop has no branches and the compiler's memory
 // counters stay exact (a chunk's stores drain while the next chunk is staged and multiplied).
-// `unit` > 0 (with FULL == false): instead of whole chunks dealt round-robin, the batch is cut
-// into gridDim.x contiguous ranges of `unit`-column pieces, as even as the piece count allows
-// (25088 columns over 256 workgroups: 96 or 112 columns each, one full chunk and a partial one,
-// where round-robin chunks give 136 workgroups 128 columns and 120 workgroups 64).
 template <typename TX, typename TW, int NF, bool FULL>
 __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__restrict__ x, half_t *__restrict__ y,
-                                                         Chain16Args args, int batch, int n_feat, int unit)
+                                                         Chain16Args args, int batch, int n_feat)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // chunk c = columns 64c .. 64c+63 (64- and 128-byte aligned row pieces in HBM); this
-    // workgroup takes chunks blockIdx.x, blockIdx.x + gridDim.x, ...
-    int c_begin = blockIdx.x * CH_TN, c_step = gridDim.x * CH_TN, c_end = batch;
-    if (!FULL && unit > 0) {
-        const int64_t units = batch / unit;  // (the host makes batch a multiple of unit)
-        c_begin = (int)(units * blockIdx.x / gridDim.x) * unit;
-        c_end = (int)(units * (blockIdx.x + 1) / gridDim.x) * unit;
-        c_step = CH_TN;
-    }
+    // chunk c = columns 64c .. 64c+63; this workgroup takes chunks c0, c0 + gridDim.x, ...
+    // An e4m3fn row piece of a chunk is 64 bytes, half a 128-byte line whose other half belongs
+    // to the neighbouring chunk.  On a full grid (a multiple of 16 workgroups) the two chunks of a
+    // line go to workgroups blockIdx.x and blockIdx.x + 8: same XCD (blockIdx.x % 8), same round,
+    // same row order, so the second request meets the first in that XCD's L2 and the line comes
+    // from HBM once.  Dealt to unrelated workgroups every line was fetched twice.
+    int c0 = blockIdx.x;
+    if (gridDim.x % 16 == 0) c0 = 2 * (8 * (c0 / 16) + c0 % 8) + (c0 / 8) % 2;
+    const int c_begin = c0 * CH_TN, c_step = gridDim.x * CH_TN, c_end = batch;
     if (c_begin >= c_end) return;
     const int c_last = c_begin + ((c_end - 1 - c_begin) / c_step) * c_step;  // this workgroup's last chunk
     const int n_blocks = n_feat / 16;  // blocks per factor
@@ -308,12 +304,7 @@ int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_
     // one persistent workgroup per CU
     const int64_t n_chunks = (batch + CH_TN - 1) / CH_TN;
     int64_t wgs = n_chunks < 256 ? n_chunks : 256;
-    // Whole chunks dealt round-robin leave the chip unevenly loaded when their number is not close
-    // to a multiple of the workgroups (392 chunks: 136 workgroups get two, 120 get one); then the
-    // batch is cut into even contiguous ranges instead, the last chunk of a range being partial.
-    int unit = 0;
-    if (n_chunks > 256 && n_chunks % 256 != 0 && n_chunks < 8 * 256 && batch % vec == 0) unit = vec;
-    const bool full = n_feat == 1024 && batch % CH_TN == 0 && unit == 0;
+    const bool full = n_feat == 1024 && batch % CH_TN == 0;
     const void *fn;
     if (x_dtype == KSMM_FP8_E4M3)
         fn = chain16_fn<fp8_t, fp8_t>(n, full);
@@ -333,7 +324,7 @@ int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_
     const int lds = (int)n_feat * CH_ROW;
     if (ensure_dynamic_lds(fn, lds) != KSMM_OK) return KSMM_ERR_LAUNCH;
     int batch_i = (int)batch, n_feat_i = (int)n_feat;
-    void *kargs[] = {(void *)&x, (void *)&y, (void *)&args, &batch_i, &n_feat_i, &unit};
+    void *kargs[] = {(void *)&x, (void *)&y, (void *)&args, &batch_i, &n_feat_i};
     hipError_t e = hipLaunchKernel(fn, dim3((unsigned)wgs), dim3(CH_THREADS), kargs, lds, stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
