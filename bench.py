@@ -223,6 +223,32 @@ def copy_reference(steps, warmup):
             "bytes": nbytes, "kernel": "torch.add(x, 1, out=y) elementwise kernel"}
 
 
+def mfma_reference():
+    """Rate at which the matrix cores multiply operands held in registers (no memory traffic at
+    all), with all-ones and with random operands: what this GPU sustains next to the datasheet
+    peaks the MFMA-bound rooflines are priced against (fp16 2516.6, fp32 157.3 TFLOP/s)."""
+    import ctypes
+
+    from ksmm_amd import _lib
+    from ksmm_amd.kernel import dtype_code
+
+    lib = _lib.load()
+    out = torch.empty(lib.ksmm_mfma_probe_bytes(), dtype=torch.uint8, device="cuda")
+    res = {}
+    for name, dt, iters in (("f16_32x32x16", dtype_code(torch.float16), 20000),
+                            ("f32_16x16x4", dtype_code(torch.float32), 20000)):
+        for random in (0, 1):
+            flops = ctypes.c_double(0.0)
+
+            def run(_):
+                stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                _lib.check(lib.ksmm_mfma_probe(dt, iters, random, out.data_ptr(), out.numel(), ctypes.byref(flops), stream))
+
+            sec = time_launches(run, 1, 3, 1)
+            res["%s_%s_tflops" % (name, "random" if random else "ones")] = flops.value / sec / 1e12
+    return res
+
+
 def cpu_baseline(patterns, bs_last, budget_s=12.0, min_run_time=0.25):
     """The reference's algo='bmm' CPU algorithm (restated in oracle/), fp32, on all host
     cores; protocol of the reference's ksmm_time.py: blocked_autorange(min_run_time=0.25),
@@ -326,6 +352,7 @@ def main():
         for cfg in CONFIGS[1:]:
             others.append(bench_config(*cfg, steps=max(20, args.steps // 2), warmup=max(5, args.warmup // 2)))
     copy_ref = copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
+    mfma_ref = mfma_reference()
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
     if args.cpu:
         # the same CPU algorithm beside every other configuration (fp32 on the host, whatever the
@@ -345,6 +372,7 @@ def main():
                      "unit": roof["unit"], "frac": roof["frac"], "traffic": traffic},
         "cpu_baseline": cpu,
         "copy_reference": copy_ref,
+        "mfma_reference": mfma_ref,
         "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),
                    "ok": head.get("parity_ok")},
         "configs": [head] + others,

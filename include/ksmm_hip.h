@@ -252,6 +252,15 @@ int ksmm_chain_forward_static(const ksmm_factor_desc *factors, int n_factors, co
                               int64_t batch, int x_dtype, int y_dtype, int bs_last, int fuse,
                               const ksmm_epilogue *epilogue, void *stream);
 
+/* Measurement aid, no counterpart in the reference: launches a kernel of 256 workgroups x 8 waves
+ * that only issues matrix-core instructions on register operands (KSMM_F16: 32x32x16 fp16,
+ * KSMM_F32: 16x16x4 fp32; `random` != 0: operands uniform in [-1, 1], else all ones) and
+ * returns the flops it performs in *flops; timed by the caller, it gives the rate the matrix
+ * cores sustain, which a benchmark prints beside the published peak.  `out` receives
+ * ksmm_mfma_probe_bytes() bytes of checksums (so that the work cannot be optimised away). */
+int64_t ksmm_mfma_probe_bytes(void);
+int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_bytes, double *flops, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

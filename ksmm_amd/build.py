@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libksmm_hip.so")
-SOURCES = ["ksmm_api.hip", "ksmm_generic.hip", "ksmm_wave.hip", "ksmm_tile.hip", "ksmm_stream.hip", "ksmm_tile_bf.hip", "ksmm_rows_bf.hip", "ksmm_gemm.hip", "ksmm_chain16.hip", "ksmm_transpose.hip", "ksmm_backward.hip"]
+SOURCES = ["ksmm_api.hip", "ksmm_generic.hip", "ksmm_wave.hip", "ksmm_tile.hip", "ksmm_stream.hip", "ksmm_tile_bf.hip", "ksmm_rows_bf.hip", "ksmm_gemm.hip", "ksmm_chain16.hip", "ksmm_transpose.hip", "ksmm_backward.hip", "ksmm_probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 VALU ops are switched off on purpose for this hardware pool
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
