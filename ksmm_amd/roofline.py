@@ -19,10 +19,12 @@ def factor_work(batch, pattern, x_dtype, w_dtype, y_dtype):
 def factor_roofline(batch, pattern, x_dtype, w_dtype, y_dtype, seconds):
     """Which roof bounds the factor and what fraction of it ``seconds`` per launch reaches.
 
-    The matrix peak used is the one of the type the kernel multiplies in: fp32 for fp32,
-    fp16 otherwise (e4m3fn operands are decoded to fp16 before the MFMA, exactly)."""
+    The matrix peak used is the one of the operand types: fp32 for fp32, fp8 when input and
+    weights are both e4m3fn (the GEMM tiles feed the bytes to the fp8 MFMA; the small-block
+    kernels decode to fp16 first, for which this peak is the stricter price), fp16 otherwise."""
     nbytes, flops = factor_work(batch, pattern, x_dtype, w_dtype, y_dtype)
-    prec = "fp32" if x_dtype == torch.float32 else "fp16"
+    fp8 = torch.float8_e4m3fn
+    prec = "fp32" if x_dtype == torch.float32 else "fp8" if (x_dtype == fp8 and w_dtype == fp8) else "fp16"
     t_hbm = nbytes / (HBM_PEAK_GBS * 1e9)
     t_mfma = flops / (MFMA_PEAK_TFLOPS[prec] * 1e12)
     gbs = nbytes / seconds / 1e9
