@@ -8,7 +8,7 @@
 // applied in place: wave w owns blocks w, w+8, ... of every factor, reads the 16 input rows of
 // a block for all columns of the chunk, multiplies with v_mfma_f32_16x16x16_f16 (the 16x16
 // weight block is stationary in registers for the life of the wave), and writes the 16 output
-// rows back; the last factor stores to global memory straight from the accumulators.  Only the
+// rows back; after the last factor the rows go to global memory as whole 128-byte lines.  Only the
 // chain input (e4m3fn or fp16) and the final fp16 output touch HBM: 77 MB instead of 283 MB for
 // the 3-factor 1024-feature chain at batch 25088.
 //
@@ -17,8 +17,7 @@
 // 16-lane group) and the accumulator stores (16 rows per 16-lane group) of a block with any
 // power-of-two stride d are free of bank conflicts.  Piece p of slot s holds the 4 columns
 // 32*(s/2) + 8*p + 4*(s%2) .. +3 of the chunk: sub-tile s of the MFMA then takes columns that
-// leave every lane with 8 consecutive columns over sub-tiles (2t, 2t+1), i.e. 16-byte global
-// stores.  e4m3fn input is expanded to fp16 while it is staged.  The weights pass through the
+// make 8 consecutive columns (16 bytes of a global row) two pieces 32 bytes apart.  e4m3fn input is expanded to fp16 while it is staged.  The weights pass through the
 // same LDS once, at the start, to be picked up in MFMA operand order by transpose loads.
 //
 // MFMA roles: A = X^T (rows = batch columns, k from ds_read_b64_tr_b16), B = W^T (lanes =
@@ -202,7 +201,8 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         else if (n0 + c_step < c_end)
             gload(n0 + c_step, true);
         // an opaque zero: keeps the compiler from hoisting the per-block address arithmetic of
-        // all NF x 8 blocks out of this loop (it would spill them)
+        // all NF x 8 blocks, and the addresses of the output pieces, out of this loop (it would
+        // spill them)
         int opaque = 0;
         asm volatile("" : "+s"(opaque));
 #pragma unroll
@@ -248,23 +248,40 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
                         o[s] = half4_t{(half_t)(acc[s][0] * scale), (half_t)(acc[s][1] * scale),
                                        (half_t)(acc[s][2] * scale), (half_t)(acc[s][3] * scale)};
                 }
-                if (f + 1 < NF) {
-                    // all inputs of the block are in registers: write its 16 output rows in place
-                    const int obase = lds_piece(row0, 0, 0) ^ v_out[f];
+                // all inputs of the block are in registers: write its 16 output rows in place (the
+                // last factor too: its rows leave for global memory from LDS, see below)
+                const int obase = lds_piece(row0, 0, 0) ^ v_out[f];
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) *(half4_t *)(smem + (obase ^ (s << 5))) = o[s];
-                } else {
-                    // last factor: slots 2t, 2t+1 of piece q are columns 32t + 8q .. +7
-                    half_t *yrow = y + (size_t)(row0 | (r << ld)) * batch + n0 + 8 * q;
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-                        if (FULL || n0 + 32 * t + 8 * q < c_end)
-                            *(half8_t *)(yrow + 32 * t) = half8_t{o[2 * t][0], o[2 * t][1], o[2 * t][2], o[2 * t][3],
-                                                                  o[2 * t + 1][0], o[2 * t + 1][1], o[2 * t + 1][2], o[2 * t + 1][3]};
-                }
+                for (int s = 0; s < 4; ++s) *(half4_t *)(smem + (obase ^ (s << 5))) = o[s];
             }
             __syncthreads();
         }
+        // ---- the chunk's result: N rows x 128 bytes, eight neighbouring lanes per row, so every
+        // store instruction writes whole lines (straight from the accumulators a lane holds
+        // 16 bytes of 16 different rows per 16-lane group: 64 separate pieces per instruction,
+        // which took 2.5x the time of this round trip through LDS).  In parts of OB pieces, to stay
+        // within the registers the input prefetch leaves (a spilled prefetch would be reloaded
+        // behind these stores and wait for them).
+        constexpr int O_PER_T = 1024 * 8 / CH_THREADS;  // 16-byte pieces per thread for 1024 rows
+        constexpr int OB = 2;
+#pragma unroll
+        for (int h = 0; h < O_PER_T / OB; ++h) {
+            uint4_t v[OB];
+#pragma unroll
+            for (int i = 0; i < OB; ++i) {
+                const int pp = tid + opaque + (h * OB + i) * CH_THREADS, row = pp >> 3, pc = pp & 7;
+                const int off = lds_piece(FULL ? row : min(row, n_feat - 1), 2 * (pc >> 2), pc & 3);
+                const uint2_t lo = *(const uint2_t *)(smem + off), hi = *(const uint2_t *)(smem + (off ^ 32));
+                v[i] = uint4_t{lo[0], lo[1], hi[0], hi[1]};
+            }
+#pragma unroll
+            for (int i = 0; i < OB; ++i) {
+                const int pp = tid + opaque + (h * OB + i) * CH_THREADS, row = pp >> 3, pc = pp & 7;
+                if (FULL || (row < n_feat && n0 + 8 * pc < c_end))
+                    *(uint4_t *)(y + (size_t)row * batch + n0 + 8 * pc) = v[i];
+            }
+        }
+        __syncthreads();  // the rows are read: the next chunk may be staged over them
     }
 }
 
