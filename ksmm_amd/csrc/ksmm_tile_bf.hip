@@ -1,12 +1,15 @@
-// Tile kernel for the batch-size-first layout with a small d > 1.
+// Tile kernel for the batch-size-first layout with d > 1.
 //
 // Batch-size-first rows hold the features as (a_i, c_i, d_i) with d_i fastest, so for d > 1
-// the c inputs of one (a_i, d_i) block are strided by d.  A workgroup therefore takes all d
-// blocks of one a_i at once: it reads the contiguous run x[n][(a_i*c + k0)*d .. (a_i*c + k0 +
-// TK)*d) with 16-byte loads, splits it by d_i while writing it to LDS (one k-contiguous plane
-// per d_i), runs d independent TM x TN x TK MFMA products against the d weight blocks, and
-// interleaves the d results again in registers, so that a lane stores d consecutive output
-// features and a tile row is one contiguous run of y.
+// the c inputs of one (a_i, d_i) block are strided by d.  A workgroup therefore takes DD
+// neighbouring blocks d_i = dg*DD .. dg*DD + DD-1 of one a_i at once (all of them when d = DD):
+// it reads x[n][(a_i*c + k)*d + dg*DD ..] with 16-byte loads (one contiguous run per row when
+// d = DD; one vector of DD elements per (row, k) when d > DD, which needs DD elements to fill
+// the vector), splits the vectors by d_i while writing them to LDS (one k-contiguous plane
+// per d_i), runs DD independent TM x TN x TK MFMA products against the DD weight blocks, and
+// interleaves the DD results again in registers, so that a lane stores DD consecutive output
+// features (16 bytes when d > DD).  Workgroups that read the same rows (the TM-tiles and the
+// d-groups of one batch tile) get neighbouring ids on one XCD and share them through its L2.
 //
 // MFMA roles as in the batch-size-first case of the plain tile kernel: A = X (rows = batch),
 // B = W (lanes = outputs), fp32 accumulation, 32x32 tiles.
@@ -47,7 +50,7 @@ template <typename CT, typename TW, typename TY, int DD, int TM, int TN, int TK,
 __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__restrict__ x,
                                                                  const TW *__restrict__ w,
                                                                  TY *__restrict__ y, int batch, int a,
-                                                                 int b, int c, Epi ep,
+                                                                 int b, int c, int d, Epi ep,
                                                                  int m_tiles, int n_tiles, int blocks)
 {
     typedef BfCfg<CT, TW, DD, TM, TN, TK, WM, WN> C;
@@ -61,15 +64,18 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
     const int per_xcd = (blocks + 7) / 8;
     const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (lid >= blocks) return;
+    const int n_dg = d / DD;  // groups of DD blocks
     const int mt_id = lid % m_tiles;
-    const int rest = lid / m_tiles;
+    int rest = lid / m_tiles;
+    const int dg = rest % n_dg;
+    rest /= n_dg;
     const int nt_id = rest % n_tiles;
     const int a_i = rest / n_tiles;
     const int m0 = mt_id * TM, n0 = nt_id * TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
-    const size_t in_size = (size_t)a * c * DD, out_size = (size_t)a * b * DD;
-    const CT *xg = x + (size_t)a_i * c * DD;  // + n * in_size + k * DD + dd
+    const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
+    const CT *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
 
     stage<TW, CT> wreg[C::W_PER_T];
     uint4_t xreg[C::X_PER_T];
@@ -81,7 +87,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
                 const int per_dd = TK * TM / C::W_EPV;
                 const int dd = v / per_dd, r = v % per_dd;
                 const int kk = r / (TM / C::W_EPV), mm = (r % (TM / C::W_EPV)) * C::W_EPV;
-                wreg[i].load(w + ((size_t)(a_i * DD + dd) * c + k0 + kk) * b + m0 + mm);
+                wreg[i].load(w + ((size_t)(a_i * d + dg * DD + dd) * c + k0 + kk) * b + m0 + mm);
             }
         }
 #pragma unroll
@@ -89,9 +95,10 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
             const int v = tid + i * C::THREADS;
             if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
                 const int vpr = TK * DD / C::EPV;  // vectors per row
-                const int nn = v / vpr, e0 = (v % vpr) * C::EPV;
+                const int nn = v / vpr, kk = (v % vpr) * C::KPV;
                 const int row = min(n0 + nn, batch - 1);
-                xreg[i] = *(const uint4_t *)(xg + (size_t)row * in_size + (size_t)k0 * DD + e0);
+                // KPV consecutive k share a vector only when d == DD (the host checks)
+                xreg[i] = *(const uint4_t *)(xg + (size_t)row * in_size + (size_t)(k0 + kk) * d);
             }
         }
     };
@@ -176,7 +183,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
             const int nb = n0 + (wn * C::NT + j) * 32;
             float bv[DD];  // bias of the lane's DD adjacent outputs
 #pragma unroll
-            for (int dd = 0; dd < DD; ++dd) bv[dd] = epi_bias<TY>(ep, ((size_t)a_i * b + m) * DD + dd);
+            for (int dd = 0; dd < DD; ++dd) bv[dd] = epi_bias<TY>(ep, ((size_t)a_i * b + m) * d + dg * DD + dd);
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int n = nb + 8 * (e >> 2) + 4 * lq + (e & 3);
@@ -184,7 +191,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
 #pragma unroll
                 for (int dd = 0; dd < DD; ++dd) o.e[dd] = (TY)epi_finish(ep, acc[dd][i][j][e], bv[dd]);
                 if (n < batch)
-                    *(pack_t<TY, DD> *)(y + (size_t)n * out_size + ((size_t)a_i * b + m) * DD) = o;
+                    *(pack_t<TY, DD> *)(y + (size_t)n * out_size + ((size_t)a_i * b + m) * d + dg * DD) = o;
             }
         }
 }
@@ -201,6 +208,10 @@ struct BfInst {
         BF_INST(COMBO_, half_t, TW_, 2, 128, 256, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 2, 64, 128, 32, 1, 4), \
         BF_INST(COMBO_, half_t, TW_, 2, 32, 128, 32, 1, 4), BF_INST(COMBO_, half_t, TW_, 4, 64, 128, 32, 1, 4), \
         BF_INST(COMBO_, half_t, TW_, 4, 32, 128, 32, 1, 4)
+// groups of 8 blocks out of any d that is a multiple of 8 (a 16-byte vector per row and k)
+#define BF_SET_H8(COMBO_, TW_)                                                                   \
+    BF_INST(COMBO_, half_t, TW_, 8, 64, 64, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 8, 64, 64, 16, 2, 2), \
+        BF_INST(COMBO_, half_t, TW_, 8, 32, 128, 16, 1, 4), BF_INST(COMBO_, half_t, TW_, 8, 128, 64, 16, 4, 2)
 const BfInst bf_insts[] = {
     BF_SET_H(1, half_t),
     BF_SET_H(3, fp8_t),
@@ -209,14 +220,19 @@ const BfInst bf_insts[] = {
     BF_INST(0, float, float, 2, 32, 128, 16, 1, 4),
     BF_INST(0, float, float, 4, 64, 128, 16, 1, 4),
     BF_INST(0, float, float, 4, 32, 128, 16, 1, 4),
+    // appended (ids of the rows above stay): 16-bit groups of 8 blocks
+    BF_SET_H8(1, half_t),
+    BF_SET_H8(3, fp8_t),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
 bool bf_fits(const BfInst &t, const Problem &p, int combo)
 {
-    if (t.combo != combo || p.bs_last || p.d != t.dd) return false;
+    if (t.combo != combo || p.bs_last || p.d % t.dd) return false;
     if (p.b % t.tm || p.c % t.tk) return false;
     const int x_epv = 16 / (int)dtype_size(p.x_dtype), w_epv = 16 / (int)dtype_size(p.w_dtype);
+    // d > DD: the DD elements of one (row, k) must fill the 16-byte vector
+    if (p.d != t.dd && t.dd != x_epv) return false;
     if (p.b % w_epv) return false;
     // rows of x start at multiples of in_size, slabs at multiples of TK * d: keep 16-byte alignment
     if (((int64_t)p.a * p.c * p.d) % x_epv || ((int64_t)p.c * p.d) % x_epv) return false;
@@ -248,7 +264,16 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         for (int i = 0; i < N_BF_INSTS; ++i) {
             const BfInst &t = bf_insts[i];
             if (!bf_fits(t, p, combo)) continue;
-            const int64_t wgs = (int64_t)p.a * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
+            // Groups out of a larger d: every line of x is shared by d/DD groups x b/TM tiles, and
+            // the loads are 16-byte pieces d elements apart.  Against the transposed route (two
+            // extra passes, but the fastest kernels in between) this wins for moderate d and b:
+            // measured over 178 patterns at batch 25088, mean time ratio 0.6-0.9 inside these
+            // bounds and 1.1-1.4 outside (large b re-reads x too often, large d scatters it).
+            if (p.d != t.dd) {
+                const bool pays = combo == 0 ? (p.d <= 16 && p.b <= 192) : (p.d <= 32 && p.b <= 384 && t.tm >= 64);
+                if (!pays) continue;
+            }
+            const int64_t wgs = (int64_t)p.a * (p.d / t.dd) * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
             int64_t score = (int64_t)t.tm * 1000 + t.tn;
             if (wgs < 512) score -= 100000;
             if (score > best) {
@@ -261,7 +286,7 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const BfInst &t = bf_insts[pick];
     const int m_tiles = p.b / t.tm;
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
-    const int64_t blocks = (int64_t)p.a * m_tiles * n_tiles;
+    const int64_t blocks = (int64_t)p.a * (p.d / t.dd) * m_tiles * n_tiles;
     const int64_t grid = (blocks + 7) / 8 * 8;
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
@@ -280,7 +305,7 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int batch_i = (int)p.batch, n_tiles_i = (int)n_tiles, blocks_i = (int)blocks, m_tiles_i = m_tiles;
     Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
-                    (void *)&p.c, &ep, &m_tiles_i, &n_tiles_i, &blocks_i};
+                    (void *)&p.c, (void *)&p.d, &ep, &m_tiles_i, &n_tiles_i, &blocks_i};
     hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(t.threads), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

@@ -77,6 +77,50 @@ def test_factor_small(prec, bs_last, algo):
     assert ran >= floor, (prec, bs_last, algo, ran, floor)
 
 
+def test_tile_bf_groups_of_blocks_forced():
+    """Batch-size-first tile kernel on groups of DD neighbouring d_i out of a larger d (tile
+    variant 3<<24 | i): every instance on shapes with d = DD, d a multiple of DD, several a_i,
+    ragged batches, and the automatic choice with a bias, against the oracle."""
+    from ksmm_amd import Kernel, generate_factor, _lib
+
+    cases = [("fp16", (1, 128, 64, 16)), ("fp16", (2, 64, 32, 8)), ("fp16", (1, 64, 64, 24)), ("fp16", (1, 128, 32, 2)),
+             ("fp16", (2, 64, 32, 4)), ("fp32", (1, 128, 32, 8)), ("fp32", (2, 64, 16, 12)), ("fp32", (1, 64, 32, 4)),
+             ("fp32", (1, 128, 32, 2)), ("fp8", (1, 128, 64, 16))]
+    ran, strided = 0, 0
+    for prec, pattern in cases:
+        a, b, c, d = pattern
+        dt = TORCH_DTYPE[prec]
+        (w4,) = seeded_weights([pattern], seed=31)
+        if prec == "fp8":  # e4m3 weights, fp16 input
+            wr, wq, ws = round_to(w4, "fp8")
+            fac, scale, x_dt, xprec = generate_factor(a, b, c, d, "kernel", wq.to(torch.float32), dt, "cuda"), ws, torch.float16, "fp16"
+        else:
+            wr = round_to(w4, prec)[0]
+            fac, scale, x_dt, xprec = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda"), 1.0, dt, prec
+        bias = (torch.rand(a * b * d, generator=torch.Generator().manual_seed(5)) - 0.5).to(x_dt)
+        for batch in (520, 77):
+            x = seeded_input(a * c * d, batch, False, seed=32)
+            z = O.ks_apply_einsum(wr, round_to(x, xprec)[0], False)
+            zb = z + bias.double().numpy()[None, :]
+            for inst in range(40):
+                try:
+                    y = Kernel.forward(x.to(x_dt).cuda(), fac, False, a, b, c, d, scale=scale, algo=3,
+                                       variant=(3 << 24) | inst)
+                except _lib.KsmmError as e:
+                    assert e.status == -6
+                    continue
+                ran += 1
+                strided += d > 4 or (prec == "fp32" and d > 2 and d != 4)
+                err = O.rel_fro_error(y.float().cpu().numpy(), z)
+                assert err <= TOL[prec], (prec, pattern, batch, inst, err)
+            # the automatic choice with the bias applied in the kernel
+            y = Kernel.forward(x.to(x_dt).cuda(), fac, False, a, b, c, d, scale=scale, bias=bias.cuda())
+            err = O.rel_fro_error(y.float().cpu().numpy(), zb)
+            assert err <= TOL[prec], (prec, pattern, batch, "bias", err)
+    print("tile_bf forced: ran", ran, "of which d > DD", strided, flush=True)
+    assert ran >= 30 and strided >= 12, (ran, strided)
+
+
 def test_gemm_kernels_forced():
     """Every instance of the direct-to-LDS GEMM sub-family (tile variant 4<<24 | i), forced on
     shapes with batch tails, several blocks per factor and d > 1."""

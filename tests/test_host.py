@@ -254,8 +254,10 @@ def test_every_pattern_shape_class_has_a_kernel_family():
     """Host-only view of the dispatch for the shape classes of the reference's pattern list that
     used to end on the one-thread-per-output kernel: b not a multiple of 16, c not a multiple of the
     K tile, blocks of a few elements, batch-size-first blocks with d > 1."""
-    from ksmm_amd.kernel import query_tile
+    from ksmm_amd import _lib
+    from ksmm_amd.kernel import dtype_code, query_tile
 
+    lib = _lib.load()
     f16, f32, f8 = torch.float16, torch.float32, torch.float8_e4m3fn
     B = 25088
     for dt in (f32, f16, f8):
@@ -271,7 +273,16 @@ def test_every_pattern_shape_class_has_a_kernel_family():
         assert t["algo"] == 2 and t["variant"] >= 1000 and t["tile_d"] == 16, (dt, t)
     t = query_tile(B, (1, 768, 192, 16), f8, None, True, variant=-3)           # e4m3 GEMM tiles
     assert t["algo"] == 3 and (t["variant"] >> 24) == 4
-    assert query_tile(B, (1, 192, 192, 16), f16, None, False, variant=-3)["algo"] == 1  # transposed route
+    # batch-size-first, big blocks, d a multiple of the 16-byte vector: groups of d_i on the tile_bf kernel
+    t = query_tile(B, (1, 192, 192, 16), f16, None, False, variant=-3)
+    assert t["algo"] == 3 and (t["variant"] >> 24) == 3 and t["tile_d"] == 8, t
+    assert lib.ksmm_factor_workspace(B, 1, 192, 192, 16, dtype_code(f16), dtype_code(f16), dtype_code(f16), 0) == 0
+    t = query_tile(B, (1, 128, 128, 8), f32, None, False, variant=-3)
+    assert t["algo"] == 3 and (t["variant"] >> 24) == 3 and t["tile_d"] == 4, t
+    # fp32 groups out of a large d, and d that is not a multiple of the vector: transposed route
+    assert query_tile(B, (1, 256, 256, 32), f32, None, False, variant=-3)["algo"] == 1
+    assert query_tile(B, (1, 192, 192, 12), f16, None, False, variant=-3)["algo"] == 1
+    assert lib.ksmm_factor_workspace(B, 1, 192, 192, 12, dtype_code(f16), dtype_code(f16), dtype_code(f16), 0) > 0
 
 
 def test_tuner_emit_keeps_one_sorted_row_per_key_above_the_threshold(tmp_path):
