@@ -117,9 +117,14 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     const int lane = threadIdx.x & 63;
     const int q = lane >> 4, r = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
-    const int g = wave / n_slabs;  // block index a_i * d + d_i
+    // A wave multiplies 16*MT output rows of a block: the whole block, or (b a multiple of that)
+    // row group h of it, the groups of a block then reading the same input rows.
+    const int m_split = b / (16 * MT);
+    const int gh = wave / n_slabs;
+    const int g = gh / m_split;  // block index a_i * d + d_i
     if (g >= a * d) return;
-    const int slab = wave - g * n_slabs;
+    const int m_off = (gh - g * m_split) * (16 * MT);
+    const int slab = wave - gh * n_slabs;
     const int a_i = g / d, d_i = g - a_i * d;
 
     // weights -> A operands, once per wave
@@ -129,14 +134,14 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = wg[(4 * ks + q) * b + 16 * mt + r];
+            for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = wg[(4 * ks + q) * b + m_off + 16 * mt + r];
     }
     // Addressing: uniform (scalar) row base + one 32-bit per-lane byte offset, so that the
     // loads and stores need no per-row vector address registers.  The host checks that the
     // offsets fit in 32 bits.
     const size_t row_stride = (size_t)d * batch;  // elements between consecutive c_i (or b_i)
     const char *xg = (const char *)(x + ((size_t)a_i * c * d + d_i) * batch);
-    char *yg = (char *)(y + ((size_t)a_i * b * d + d_i) * batch);
+    char *yg = (char *)(y + (((size_t)a_i * b + m_off) * d + d_i) * batch);
     const uint32_t x_lane = (uint32_t)(q * row_stride) * 4u;      // + column offset
     const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 4u;  // + column offset
     // Tiles of one wave (all uniform): `regular` tiles at n_first, n_first + stride, ... and, in
@@ -190,7 +195,7 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * b + 16 * mt + 4 * q + i) * d + d_i);
+                bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * b + m_off + 16 * mt + 4 * q + i) * d + d_i);
     }
     // Everything issued so far (weights, first tile) is complete before the loop, so that the
     // waits inside the loop only ever count that loop's own loads and stores.
@@ -420,6 +425,10 @@ using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int,
 const WaveInst f32_insts[] = {
     F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
     F32_INST(16, 16, 4), F32_INST(32, 32, 3), F32_INST(48, 192, 1),
+    // also takes the two row groups of a 64 x 64 block (forced or from the table): half the
+    // weight registers, three waves per SIMD; 6 % faster than the whole block per wave on
+    // (6,64,64,1) at batch 25088 (groups of 16 rows were 15-40 % slower there and on 48 x 48)
+    F32_INST(32, 64, 3),
 };
 
 #define H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, ROLL_, EPI_) \
@@ -492,7 +501,9 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if (rr == 3) return KSMM_ERR_BAD_ALGO;
     int pick = -1;
     for (int i = 0; i < n_insts; ++i) {
-        if (insts[i].b != p.b || insts[i].c != p.c) continue;
+        // fp32: a forced instance also takes blocks whose b is a multiple of its rows (row groups)
+        const bool rows_ok = insts[i].b == p.b || (combo == 0 && want == i && p.b % insts[i].b == 0);
+        if (!rows_ok || insts[i].c != p.c) continue;
         if (p.batch % insts[i].vec) continue;
         if (want != 0xff && want != i) continue;
         pick = i;
@@ -517,7 +528,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     // 4 waves each) with the rolling pipeline over several tiles is best, and a few workgroups
     // beyond 256 double the run time (two share a CU while the others have finished): take the
     // smallest count that fits one round.
-    const int64_t groups = (int64_t)p.a * p.d;
+    const int64_t groups = (int64_t)p.a * p.d * (p.b / in.b);  // blocks x row groups
     const int wpb = 4;
     // (Balanced dealing, rr == 2, keeps every CU within one tile of its share: (1,48,48,16) at
     // batch 25088 has 24.5 tiles per CU where 7 consecutive tiles per wave leave 32 CUs idle and
@@ -537,7 +548,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     } else {
         if (iters == 0) {
             iters = 1;
-            if (p.b * p.c > 1024)
+            if (in.b * p.c > 1024)
                 while (iters < 255 && (groups * ((n_tiles + iters - 1) / iters) + wpb - 1) / wpb > 256) ++iters;
         }
         n_slabs = (n_tiles + iters - 1) / iters;
@@ -548,7 +559,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if (tile) {
         tile->algo = KSMM_ALGO_WAVE;
         tile->variant = pick | (iters_field << 8) | (rr << 16);
-        tile->tile_m = p.b;
+        tile->tile_m = in.b;
         tile->tile_n = tn;
         tile->tile_k = p.c;
         tile->tile_d = 1;

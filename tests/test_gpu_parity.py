@@ -121,6 +121,29 @@ def test_tile_bf_groups_of_blocks_forced():
     assert ran >= 30 and strided >= 12, (ran, strided)
 
 
+def test_wave_row_groups_forced():
+    """fp32 wave instance for 32-row blocks forced on 64-row blocks (two row groups per block,
+    variant 7 | tiles-per-wave << 8 | dealing << 16), with a_i, d_i > 1, ragged batches and a bias."""
+    from ksmm_amd import Kernel, generate_factor, _lib
+    from ksmm_amd.kernel import query_tile
+
+    ran = 0
+    for pattern in [(6, 64, 64, 1), (2, 64, 64, 3), (1, 32, 64, 2), (1, 96, 64, 2)]:
+        a, b, c, d = pattern
+        (w4,) = seeded_weights([pattern], seed=41)
+        fac = generate_factor(a, b, c, d, "kernel", w4, torch.float32, "cuda")
+        for batch in (1024, 200):
+            x = seeded_input(a * c * d, batch, True, seed=42)
+            z = O.ks_apply_einsum(w4.double().numpy(), x.double().numpy(), True)
+            for variant in (7, 7 | (3 << 8), 7 | (2 << 8) | (1 << 16), 7 | (1 << 16 + 1)):
+                t = query_tile(batch, pattern, torch.float32, None, True, algo=2, variant=variant)
+                assert t["tile_m"] == 32, t
+                y = Kernel.forward(x.cuda(), fac, True, a, b, c, d, algo=2, variant=variant)
+                ran += 1
+                assert O.rel_fro_error(y.cpu().numpy(), z) <= TOL["fp32"], (pattern, batch, variant)
+    assert ran == 32
+
+
 def test_gemm_kernels_forced():
     """Every instance of the direct-to-LDS GEMM sub-family (tile variant 4<<24 | i), forced on
     shapes with batch tails, several blocks per factor and d > 1."""
