@@ -259,7 +259,7 @@ __global__ __launch_bounds__(CH_THREADS) void ks_chain16_kernel(const TX *__rest
         // ---- the chunk's result: N rows x 128 bytes, eight neighbouring lanes per row, so every
         // store instruction writes whole lines (straight from the accumulators a lane holds
         // 16 bytes of 16 different rows per 16-lane group: 64 separate pieces per instruction,
-        // which took 2.5x the time of this round trip through LDS).  In parts of OB pieces, to stay
+        // which took 2.5x the time of this detour through LDS).  In parts of OB pieces, to stay
         // within the registers the input prefetch leaves (a spilled prefetch would be reloaded
         // behind these stores and wait for them).
         constexpr int O_PER_T = 1024 * 8 / CH_THREADS;  // 16-byte pieces per thread for 1024 rows
