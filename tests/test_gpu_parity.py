@@ -269,7 +269,7 @@ def test_tile_subfamilies_forced():
             for p in [(2, 64, 64, 1), (3, 128, 128, 1), (2, 192, 192, 1)]:
                 cases.append((prec, bs_last, p, 1000))
     cases += [("fp32", True, (2, 64, 64, 1), 1000), ("fp32", True, (1, 128, 128, 1), 1000)]
-    _forced_sweep(cases, [(2 << 24) | i for i in range(28)], 3, 24)                      # stream
+    _forced_sweep(cases, [(2 << 24) | i for i in range(32)], 3, 24)                      # stream
     kcases = [("fp16", True, (2, 128, 64, 2), 520), ("fp16", False, (2, 128, 64, 1), 520),
               ("fp32", True, (1, 128, 64, 3), 520), ("fp32", False, (2, 64, 32, 1), 520),
               ("fp8", True, (2, 128, 64, 2), 528), ("hq", False, (1, 256, 128, 1), 520),
