@@ -364,6 +364,13 @@ const StreamInst stream_insts[] = {
     STREAM_INST(0, float, float, true, 64, 64, 64, 1, 2, 4, 0),
     STREAM_INST(0, float, float, true, 64, 64, 128, 1, 4, 3, 0),
     STREAM_INST(0, float, float, true, 128, 128, 64, 2, 2, 2, 0),
+    // more waves per block (forced or from the table)
+    STREAM_INST(1, half_t, half_t, false, 128, 128, 64, 4, 2, 4, 0),
+    STREAM_INST(1, half_t, half_t, true, 128, 128, 64, 4, 2, 4, 0),
+    STREAM_INST(1, half_t, half_t, false, 64, 64, 64, 2, 2, 3, 0),
+    STREAM_INST(1, half_t, half_t, true, 64, 64, 64, 2, 2, 3, 0),
+    STREAM_INST(1, half_t, half_t, false, 64, 64, 128, 2, 4, 3, 0),
+    STREAM_INST(1, half_t, half_t, true, 64, 64, 128, 2, 4, 3, 0),
 };
 constexpr int N_STREAM_INSTS = sizeof(stream_insts) / sizeof(StreamInst);
 
