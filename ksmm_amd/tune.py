@@ -202,12 +202,35 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
 
 
 def _entry_id(e):
-    """(instance id, parameter) of an entry; entries of older runs carry only the variant."""
-    from .kernel import variant_id
+    """(instance id, parameter) of an entry for the library at hand, or None when the kernel it
+    measured cannot be named any more.  The id recorded at measuring time is used when it still
+    resolves to a kernel with the recorded tile; otherwise (an older run, or a build whose ids
+    were formed differently) the recorded variant is tried, under the same check: a variant is a
+    position in an instance table and only means the same kernel while that table is unchanged."""
+    from . import _lib
+    from .kernel import query_tile, variant_from_id, variant_id
 
-    # always from (family, variant) with the library at hand: the id recorded at measuring time
-    # belongs to the build that measured
-    return variant_id(e["algo"], e["variant"], COMBO[e["prec"]], e["bs_last"])
+    a, b, c, d = e["pattern"]
+    dt = DT[e["prec"]]
+    want = e.get("tile") or {}
+
+    def same_kernel(variant):
+        try:
+            t = query_tile(e.get("batch", 25088), (a, b, c, d), dt, None, e["bs_last"], e["algo"], variant)
+        except _lib.KsmmError:
+            return False
+        return all(t[k] == want[k] for k in ("tile_m", "tile_n", "tile_k", "tile_d", "threads") if k in want)
+
+    if "id" in e and e["id"]:
+        try:
+            v = variant_from_id(e["algo"], e["id"], e.get("param", 0), COMBO[e["prec"]], e["bs_last"])
+            if same_kernel(v):
+                return e["id"], e.get("param", 0)
+        except _lib.KsmmError:
+            pass
+    if same_kernel(e["variant"]):
+        return variant_id(e["algo"], e["variant"], COMBO[e["prec"]], e["bs_last"])
+    return None
 
 
 def emit(entries, path, batch):
@@ -219,7 +242,12 @@ def emit(entries, path, batch):
         if not e["best_us"] < 0.97 * e["auto_us"]:
             continue
         a, b, c, d = e["pattern"]
-        iid, par = _entry_id(e)
+        named = _entry_id(e)
+        if named is None:
+            print("dropped (kernel not in this library): %s %s bs_last=%s variant %s" % (
+                e["pattern"], e["prec"], e["bs_last"], hex(e["variant"])), file=sys.stderr)
+            continue
+        iid, par = named
         rows.append((a, b, c, d, COMBO[e["prec"]], 1 if e["bs_last"] else 0, e["algo"], iid, par,
                      e["best_us"], e["auto_us"]))
     rows.sort(key=lambda r: (r[:6], r[9]))  # by key, fastest first
@@ -264,7 +292,7 @@ def emit_best(entries, directory):
                     if use_best:
                         t = e.get("tile", {})
                         fam = FAMILY[e["algo"]]
-                        iid, par = _entry_id(e)
+                        iid, par = _entry_id(e) or (0, 0)
                         ms, std, mse = e.get("best_mean_us", e["best_us"]) / 1e3, e.get("best_std_us", 0.0) / 1e3, e.get("mse", float("nan"))
                     else:
                         t = e.get("auto_tile", {})
@@ -295,6 +323,10 @@ def main():
     entries = []
     for p in args.merge:
         entries += json.load(open(p))
+    # the same (pattern, type, layout) measured twice: the file named first wins
+    seen = set()
+    entries = [e for e in entries
+               if (k := (tuple(e["pattern"]), e["prec"], bool(e["bs_last"]))) not in seen and not seen.add(k)]
     if args.patterns:
         from . import _lib
 

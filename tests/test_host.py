@@ -294,19 +294,29 @@ def test_tuner_emit_keeps_one_sorted_row_per_key_above_the_threshold(tmp_path):
         return {"pattern": list(p), "prec": prec, "bs_last": bs_last, "auto_us": auto, "best_us": best,
                 "algo": algo, "variant": variant}
 
-    entries = [entry((2, 64, 64, 1), "fp16", True, 10.0, 9.0),
+    entries = [entry((2, 64, 64, 1), "fp16", True, 10.0, 9.0, 2, 0),
                entry((1, 48, 48, 16), "fp32", True, 10.0, 9.9),            # within 3 %: dropped
                entry((1, 48, 48, 16), "fp32", False, 10.0, 8.0, 2, 1000),
-               entry((2, 64, 64, 1), "fp16", True, 10.0, 8.5, 3, 7),        # duplicate key: the faster one
+               entry((2, 64, 64, 1), "fp16", True, 10.0, 8.5, 2, 1),        # duplicate key: the faster one
+               entry((4, 64, 64, 1), "fp16", True, 10.0, 5.0, 3, 5),        # a kernel that does not take it: dropped
                entry((1, 16, 16, 4), "fp8", True, None, None, 0, -1)]       # nothing measured
     path = tmp_path / "t.inc"
     assert emit(entries, str(path), 25088) == 2
     rows = [l for l in path.read_text().splitlines() if l.startswith("{")]
     # rows name the kernel by stable instance id and parameter, not by table position
-    from ksmm_amd.kernel import variant_id
+    from ksmm_amd.kernel import variant_from_id, variant_id
 
     assert rows[0].startswith("{1, 48, 48, 16, 0, 0, 2, %du, %d}" % variant_id(2, 1000, 0, False))
-    assert rows[1].startswith("{2, 64, 64, 1, 1, 1, 3, %du, %d}" % variant_id(3, 7, 1, True))
+    assert rows[1].startswith("{2, 64, 64, 1, 1, 1, 2, %du, %d}" % variant_id(2, 1, 1, True))
+    # an id recorded at measuring time wins over the (positional) variant when it still names a
+    # kernel with the recorded tile; a stale variant alone must not be trusted
+    iid, par = variant_id(2, 1, 1, True)
+    moved = dict(entry((2, 64, 64, 1), "fp16", True, 10.0, 8.0, 2, 0), id=iid, param=par,
+                 tile={"tile_m": 64, "tile_n": 128, "tile_k": 64, "tile_d": 1, "threads": 256})
+    assert emit([moved], str(path), 25088) == 1
+    row = [l for l in path.read_text().splitlines() if l.startswith("{")][0]
+    assert row.startswith("{2, 64, 64, 1, 1, 1, 2, %du, %d}" % (iid, par))
+    assert variant_from_id(2, iid, par, 1, True) == 1
 
 
 def test_tuner_best_files_have_the_reference_columns(tmp_path):
