@@ -757,5 +757,25 @@ def test_persistent_gemm_walks_several_tiles_per_workgroup():
             err = ((y.float() - ref.float()).norm() / ref.float().norm()).item()
             assert err <= 1e-6, (pattern, inst, err)
     assert ran >= 5, ran
-    # epilogue through the automatic choice is covered elsewhere; here: the persistent instances
-    # reached through the measured table keep bias and GELU (forced instances take no epilogue)
+    # bias + GELU on the persistent kernel (its epilogue is an instantiation of its own): forced
+    # instances take no epilogue, so a problem with three tiles per CU, where the heuristic picks
+    # the persistent form by itself
+    from ksmm_amd.kernel import query_tile
+
+    pattern, batch = (1, 512, 96, 2), 49152
+    a, b, c, d = pattern
+    t = query_tile(batch, pattern, torch.float16, None, False)
+    assert t["algo"] == 3 and (t["variant"] >> 24) == 4 and t["grid"] == 256, t
+    (w4,) = seeded_weights([pattern], seed=103)
+    x = seeded_input(a * c * d, batch, False, seed=104)
+    fac = generate_factor(a, b, c, d, "kernel", w4, torch.float16, "cuda")
+    bias = (torch.rand(a * b * d, generator=torch.Generator().manual_seed(7)) - 0.5).half()
+    rows = sample_columns(batch, step=911)
+    z = O.ks_apply_einsum(round_to(w4, "fp16")[0], round_to(x, "fp16")[0][rows], False)
+    zb = z + bias.double().numpy()[None, :]
+    import scipy.special
+
+    zg = 0.5 * zb * (1.0 + scipy.special.erf(zb / np.sqrt(2.0)))
+    for act, want in ((None, zb), ("gelu", zg)):
+        y = Kernel.forward(x.half().cuda(), fac, False, a, b, c, d, bias=bias.cuda(), act=act)
+        assert O.rel_fro_error(y.float().cpu().numpy()[rows], want) <= TOL["fp16"], act
