@@ -583,6 +583,8 @@ EPILOGUE_CASES = [
     ((1, 48, 48, 16), 1040), ((6, 64, 64, 1), 520), ((2, 192, 192, 1), 520), ((1, 256, 64, 2), 520),
     ((2, 3, 5, 4), 203), ((1, 96, 48, 2), 520), ((3, 16, 16, 4), 528), ((1, 192, 192, 16), 264),
     ((2, 128, 70, 1), 520), ((1, 2, 4, 112), 64), ((2, 77, 64, 1), 520), ((1, 128, 128, 1), 1024),
+    # enough batch tiles for the direct-to-LDS GEMM tiles (d = 2 and d = 1 epilogues differ)
+    ((2, 256, 64, 2), 8192), ((2, 256, 64, 1), 8192),
 ]
 
 
@@ -626,6 +628,8 @@ def test_bias_and_gelu_in_the_kernel_epilogue(prec, bs_last):
         assert O.rel_fro_error(y.float().cpu().numpy(), _gelu64(z)) <= TOL[prec], (pattern, prec, bs_last)
     print("families seen", prec, bs_last, sorted(seen), flush=True)
     assert len(seen) >= (4 if bs_last else 3), seen
+    if bs_last or prec == "fp16":
+        assert (3, 4) in seen, seen  # the GEMM tiles' bias/activation instantiation ran
 
 
 @pytest.mark.parametrize("prec", ["fp16", "fp8"])
