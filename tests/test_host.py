@@ -250,6 +250,25 @@ def test_tuned_table_is_sorted_and_every_row_names_a_kernel_that_fits():
         assert small == heur
 
 
+def test_wave_row_group_instance_only_when_named():
+    """The fp32 wave instance for 32-row blocks takes row groups of a 64- or 96-row block when it
+    is forced (or named by a table row); the heuristics keep whole blocks per wave."""
+    from ksmm_amd import _lib
+    from ksmm_amd.kernel import query_tile
+
+    f32 = torch.float32
+    forced = query_tile(25088, (6, 64, 64, 1), f32, None, True, algo=2, variant=7)
+    assert forced["tile_m"] == 32 and forced["tile_k"] == 64
+    whole = query_tile(25088, (6, 64, 64, 1), f32, None, True, algo=2, variant=-1)
+    assert whole["tile_m"] == 64 and (whole["variant"] & 0xff) != 7
+    assert forced["grid"] >= whole["grid"]  # twice the waves for the same tiles per wave or fewer
+    assert query_tile(25088, (2, 96, 64, 3), f32, None, True, algo=2, variant=7)["tile_m"] == 32
+    with pytest.raises(_lib.KsmmError):   # 48 rows are not a multiple of 32
+        query_tile(25088, (1, 48, 64, 2), f32, None, True, algo=2, variant=7)
+    with pytest.raises(_lib.KsmmError):   # other c
+        query_tile(25088, (1, 64, 32, 2), f32, None, True, algo=2, variant=7)
+
+
 def test_every_pattern_shape_class_has_a_kernel_family():
     """Host-only view of the dispatch for the shape classes of the reference's pattern list that
     used to end on the one-thread-per-output kernel: b not a multiple of 16, c not a multiple of the
