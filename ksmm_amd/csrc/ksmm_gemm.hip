@@ -928,11 +928,310 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbf_kernel(const CT *
     if (loader) __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // repeats of the last slab must land before LDS is released
 }
 
+// ------------------------------------------------------------------------------------------
+// Persistent form for batch-size-last blocks (fp32, fp16 and e4m3, any d): the scheme of
+// ks_gemm_pbf_kernel with the operand roles of the batch-size-last tiles.  Both operands are
+// k-outer, so every chunk of a loader lane is a whole number of rows further down than the one
+// before it, with the same column and swizzle: one per-lane offset each for weights and input,
+// the rest are uniform additions.  The accumulator rows run along the batch axis; a wave turns
+// its blocks around in a piece of LDS of its own behind the ring (32 output rows x 128 bytes:
+// two neighbouring 32-column blocks for fp16, one for fp32) and stores whole lines.  The pieces
+// are private, so a tile switch needs no workgroup barrier: waves that finish their part of
+// the tile early start on the next tile's first slab while the others still store.
+template <typename CT, typename TY, int TM, int TN, int TK, int WM, int WN, int ST, bool EPI>
+__global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbl_kernel(const CT *__restrict__ x,
+                                                                const CT *__restrict__ w,
+                                                                TY *__restrict__ y, int batch, int a,
+                                                                int b, int c, int d, Epi ep,
+                                                                int m_tiles, int n_tiles, int blocks)
+{
+    typedef GemmCfg<CT, true, 1, TM, TN, TK, WM, WN, ST> C;
+    constexpr int NWAVES = WM * WN, LOADERS = 64 * (NWAVES / 2);      // loader threads (lower half)
+    constexpr int LW = C::W_CHUNKS / LOADERS, LX = C::X_CHUNKS / LOADERS, L = LW + LX;
+    constexpr int N_WAIT = (ST - 2) * L;
+    static_assert(NWAVES % 2 == 0 && C::W_CHUNKS % LOADERS == 0 && C::X_CHUNKS % LOADERS == 0, "loader split");
+    static_assert(ST >= 3 && N_WAIT <= 63, "ring");
+    static_assert(sizeof(CT) == sizeof(TY) || (sizeof(CT) == 1 && sizeof(TY) == 2), "fp32, fp16, e4m3 -> fp16");
+    constexpr int OES = (int)sizeof(TY);
+    constexpr int JP = OES == 2 ? 2 : 1;  // 32-column blocks per 128 bytes of an output row
+    static_assert(C::NT % JP == 0, "blocks pair up into whole lines");
+    constexpr int OP = 128 + 16;          // bytes per row of a wave's output piece
+    constexpr int OUT_BASE = C::LDS_BYTES;  // the pieces follow the ring
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const float scale = ep.scale;
+    // bias and activation live in an instantiation of their own: next to the accumulators their
+    // registers would push the plain one into scratch memory
+    constexpr bool has_epi = EPI;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const bool loader = wave < NWAVES / 2;  // uniform per wave
+
+    // ---- the tiles of this workgroup: XCD blockIdx % 8 owns a contiguous eighth of the logical
+    // tile ids (TM-tile fastest, then batch tile, then the block a_i * d + d_i), its workgroup
+    // blockIdx / 8 takes every slots-th one
+    const int per_xcd = (blocks + 7) / 8;
+    const int slots = (int)gridDim.x / 8;  // the grid is a multiple of 8
+    const int xcd_first = ((int)blockIdx.x % 8) * per_xcd;
+    const int xcd_end = min(xcd_first + per_xcd, blocks);
+    const int first = xcd_first + (int)blockIdx.x / 8;
+    if (first >= xcd_end) return;
+    const int my_tiles = (xcd_end - first + slots - 1) / slots;
+    struct Tile {
+        int m0, n0, a_i, d_i;
+    };
+    auto decode = [&](int t) {
+        const int lid = first + t * slots;
+        const int mt_id = lid % m_tiles, rest = lid / m_tiles;
+        const int g = rest / n_tiles, a_i = g / d;
+        return Tile{mt_id * TM, (rest % n_tiles) * TN, a_i, g - a_i * d};
+    };
+
+    // ---- load side (loader waves): a stream of slabs that runs ST-1 slabs ahead of the
+    // multiplication, across tile boundaries.  uniform base + 32-bit per-lane offset
+    const int steps = c / TK;
+    const size_t w_step = (size_t)TK * b * C::ES, x_step = (size_t)TK * d * batch * C::ES;  // bytes per slab
+    constexpr int W_ROWS_PER = LOADERS / C::W_CPR, X_ROWS_PER = LOADERS / C::X_CPR;
+    constexpr int SWZ_ROWS = C::ES == 1 ? 8 : C::ES == 2 ? 4 : 2;  // rows after which the chunk swizzle repeats
+    static_assert(LOADERS % C::W_CPR == 0 && W_ROWS_PER % SWZ_ROWS == 0 && W_ROWS_PER * LW == TK, "uniform weight chunk strides");
+    static_assert(LOADERS % C::X_CPR == 0 && X_ROWS_PER % SWZ_ROWS == 0 && X_ROWS_PER * LX == TK, "uniform input chunk strides");
+    uint32_t wvoff0, xvoff0, xrow_off;
+    int xcol;
+    {
+        const int q = tid & (LOADERS - 1);
+        const int row = q / C::W_CPR, pc = q % C::W_CPR;
+        const int col = (pc ^ swz_outer<CT, C::W_CPR>(row)) * C::EPC;
+        wvoff0 = (uint32_t)(((size_t)row * b + col) * C::ES);
+        const int xrow = q / C::X_CPR, xpc = q % C::X_CPR;
+        xcol = (xpc ^ swz_outer<CT, C::X_CPR>(xrow)) * C::EPC;
+        xrow_off = (uint32_t)((size_t)xrow * d * batch * C::ES);
+    }
+    const size_t w_chunk_step = (size_t)W_ROWS_PER * b * C::ES, x_chunk_step = (size_t)X_ROWS_PER * d * batch * C::ES;
+    const char *i_w = nullptr, *i_x = nullptr;  // slab the load side is at
+    int i_t = 0, i_k = 0;
+    auto i_open = [&](int t) {
+        const Tile q = decode(t);
+        i_w = (const char *)(w + ((size_t)(q.a_i * d + q.d_i) * c) * b + q.m0);
+        i_x = (const char *)(x + ((size_t)q.a_i * c * d + q.d_i) * batch + q.n0);
+        // the last batch tile repeats its last 16 bytes instead of reading past the end of a row
+        xvoff0 = xrow_off + (uint32_t)(min(xcol, batch - C::EPC - q.n0) * C::ES);
+    };
+    // next slab of the stream; after the last one the load side stays there (the ring then
+    // receives repeats of it, which keeps the number of loads per slab constant)
+    auto i_advance = [&]() {
+        if (i_k + 1 < steps) {
+            ++i_k;
+            i_w += w_step;
+            i_x += x_step;
+        } else if (i_t + 1 < my_tiles) {
+            ++i_t;
+            i_k = 0;
+            i_open(i_t);
+        }
+    };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    auto issue_one = [&](const char *wsrc, const char *xsrc, uint32_t dst, int q) {
+        // dst: stage base + this wave's kilobyte; chunk q of the lane
+        if (q < LW)
+            dma16s(wsrc + q * w_chunk_step, wvoff0, dst + q * (LOADERS * 16));
+        else
+            dma16s(xsrc + (q - LW) * x_chunk_step, xvoff0, dst + C::W_BYTES + (q - LW) * (LOADERS * 16));
+    };
+
+    // ---- per-lane byte offsets of the MFMA operands inside a stage (sub-step 0) --------------
+    uint32_t woff[C::MT], xoff[C::NT];
+#pragma unroll
+    for (int i = 0; i < C::MT; ++i) woff[i] = outer_frag<CT, TM>::off((wm * C::MT + i) * 32, lane);
+#pragma unroll
+    for (int j = 0; j < C::NT; ++j) xoff[j] = C::W_BYTES + outer_frag<CT, TN>::off((wn * C::NT + j) * 32, lane);
+    float16_t acc[C::MT][C::NT];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+            for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    };
+    clear_acc();
+
+    i_open(0);
+#pragma unroll
+    for (int p = 0; p < ST - 1; ++p) {
+        if (loader) {
+            const uint32_t dst = lds_base + p * C::STAGE_BYTES + wave * 1024;
+#pragma unroll
+            for (int q = 0; q < L; ++q) issue_one(i_w, i_x, dst, q);
+        }
+        i_advance();
+    }
+
+    typedef typename frag<CT>::type frag_t;
+    auto read_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[C::MT],
+                          frag_t(&fx)[C::NT]) {
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i) fw[i] = outer_frag<CT, TM>::read(wa[i], k0);
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) fx[j] = outer_frag<CT, TN>::read(xa[j], k0);
+    };
+    constexpr int K0 = TK / C::KSTEP;      // MFMA sub-steps per slab
+    constexpr int PER_K0 = C::MT * C::NT;  // MFMAs per sub-step
+    static_assert(K0 >= 2 && K0 % 2 == 0, "operand double buffer alternates inside a slab");
+    constexpr int SLOTS = (K0 - 1) * PER_K0;
+    constexpr int STRIDE = SLOTS / L > 0 ? SLOTS / L : 1;  // MFMAs per load issued (loader waves)
+    frag_t fw[2][C::MT], fx[2][C::NT];
+    uint32_t wa[C::MT], xa[C::NT];
+    auto stage_addrs = [&](int stg) {
+        const uint32_t base = lds_base + stg * C::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < C::MT; ++i) {
+            wa[i] = woff[i] + base;
+            asm volatile("" : "+v"(wa[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < C::NT; ++j) {
+            xa[j] = xoff[j] + base;
+            asm volatile("" : "+v"(xa[j]));
+        }
+    };
+    if (loader) __builtin_amdgcn_s_waitcnt(vmcnt_imm(N_WAIT));
+    __syncthreads();  // slab 0 landed
+    stage_addrs(0);
+    read_frags(wa, xa, 0, fw[0], fx[0]);
+
+    const int l32 = lane & 31, lq = lane >> 5;
+    constexpr int TILE_STORES = C::MT * (C::NT / JP) * 4;  // stores of a wave per full tile
+    static_assert(N_WAIT + TILE_STORES <= 63, "counter range");
+    static_assert(OUT_BASE + NWAVES * 32 * OP <= 160 * 1024, "ring and output pieces fit");
+    unsigned char *const piece = smem + OUT_BASE + wave * (32 * OP);
+    bool stores_behind = false;  // the previous tile issued exactly TILE_STORES stores (uniform)
+    Tile cur = decode(0);
+    int stg = 0;  // ring stage of the slab being multiplied
+    for (int c_t = 0; c_t < my_tiles; ++c_t) {
+        for (int c_k = 0; c_k < steps; ++c_k) {
+            const char *const wsrc = i_w;
+            const char *const xsrc = i_x;
+            const int stg_fill = stg == 0 ? ST - 1 : stg - 1;  // stage of the slab ST-1 ahead
+            const int stg_next = stg + 1 == ST ? 0 : stg + 1;
+            const uint32_t dst = lds_base + stg_fill * C::STAGE_BYTES + wave * 1024;
+#pragma unroll
+            for (int kk = 0; kk < K0; ++kk) {
+                if (kk + 1 < K0) {
+                    read_frags(wa, xa, (kk + 1) * C::KSTEP, fw[(kk + 1) & 1], fx[(kk + 1) & 1]);
+                } else {
+                    if (loader) {
+                        // behind the next slab's loads the counter holds the loads of the ST-2 slabs
+                        // after it and, while the load of the next slab is older than the previous
+                        // tile's output stores, those stores
+                        if (c_k < ST - 2 && stores_behind)
+                            __builtin_amdgcn_s_waitcnt(vmcnt_imm(N_WAIT + TILE_STORES));
+                        else
+                            __builtin_amdgcn_s_waitcnt(vmcnt_imm(N_WAIT));
+                    }
+                    __syncthreads();  // the next slab has landed, and everyone has left this one
+                    // (at the end of a tile the next tile's first operands are read after its output
+                    // has left: their registers are needed for that)
+                    if (c_k + 1 < steps) {
+                        stage_addrs(stg_next);
+                        read_frags(wa, xa, 0, fw[0], fx[0]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);  // requested before this sub-step multiplies
+                }
+#pragma unroll
+                for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::NT; ++j) {
+                        acc[i][j] = frag<CT>::mfma(fx[kk & 1][j], fw[kk & 1][i], acc[i][j]);
+                        const int m = kk * PER_K0 + i * C::NT + j;  // MFMA index in the slab
+                        if (kk + 1 < K0 && (m + 1) % STRIDE == 0 && m / STRIDE < L) {
+                            if (loader) issue_one(wsrc, xsrc, dst, m / STRIDE);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                if (kk == K0 - 2) {
+                    // loads that did not get a slot above (fewer MFMAs than loads)
+                    if (loader) {
+#pragma unroll
+                        for (int q = SLOTS / STRIDE; q < L; ++q) issue_one(wsrc, xsrc, dst, q);
+                    }
+                }
+            }
+            i_advance();
+            if (c_k + 1 < steps) stg = stg_next;
+        }
+        // ---- the tile is complete.  In the accumulators a lane holds one output feature (row
+        // l32 of the block) and, per group eg, 4 consecutive batch columns: written like that a
+        // store touches 32 rows.  Through the wave's piece (OP bytes per row) eight neighbouring
+        // lanes get the eight 16-byte parts of a row: whole lines, 8 rows per store.  LDS
+        // accesses of one wave execute in order, so the piece needs no barrier.
+        if constexpr (has_epi) {
+            const bool gelu = ep.act == KSMM_ACT_GELU;
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i) {
+                const int mb = (wm * C::MT + i) * 32;
+                const float bl = epi_bias<TY>(ep, ((size_t)cur.a_i * b + cur.m0 + mb + l32) * d + cur.d_i);
+#pragma unroll
+                for (int j = 0; j < C::NT; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const float v = fmaf(acc[i][j][e], scale, bl);
+                        acc[i][j][e] = gelu ? gelu_erf(v) : v;
+                    }
+            }
+        }
+        const float st_scale = has_epi ? 1.f : scale;
+        {
+            unsigned char *const wr = piece + l32 * OP + (4 * OES) * lq;                  // + block, + 8 * OES * eg
+            const unsigned char *const rd = piece + (lane >> 3) * OP + 16 * (lane & 7);  // + 8 * t rows
+#pragma unroll
+            for (int i = 0; i < C::MT; ++i)
+#pragma unroll
+                for (int jp = 0; jp < C::NT / JP; ++jp) {
+                    const int mb = (wm * C::MT + i) * 32, nb = (wn * C::NT + jp * JP) * 32;
+#pragma unroll
+                    for (int jj = 0; jj < JP; ++jj)
+#pragma unroll
+                        for (int eg = 0; eg < 4; ++eg) {
+                            const float16_t &ac = acc[i][jp * JP + jj];
+                            if constexpr (OES == 4) {
+                                const float4_t v = {ac[4 * eg] * st_scale, ac[4 * eg + 1] * st_scale,
+                                                    ac[4 * eg + 2] * st_scale, ac[4 * eg + 3] * st_scale};
+                                *(float4_t *)(wr + 32 * eg) = v;
+                            } else {
+                                const half4_t v = {(half_t)(ac[4 * eg] * st_scale), (half_t)(ac[4 * eg + 1] * st_scale),
+                                                   (half_t)(ac[4 * eg + 2] * st_scale), (half_t)(ac[4 * eg + 3] * st_scale)};
+                                *(half4_t *)(wr + 64 * jj + 16 * eg) = v;
+                            }
+                        }
+                    __builtin_amdgcn_wave_barrier();
+                    const int n = cur.n0 + nb + (16 / OES) * (lane & 7);
+                    const int row = cur.m0 + mb + (lane >> 3);  // + 8 * t
+                    TY *const dstp = y + (((size_t)cur.a_i * b + row) * d + cur.d_i) * batch + n;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const uint4_t v = *(const uint4_t *)(rd + 8 * t * OP);
+                        if (n < batch) __builtin_nontemporal_store(v, (uint4_t *)(dstp + (size_t)8 * t * d * batch));
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+        }
+        stores_behind = cur.n0 + TN <= batch;  // a ragged tile skips stores: then wait the safe way
+        if (c_t + 1 < my_tiles) {
+            clear_acc();
+            cur = decode(c_t + 1);
+            stg = stg + 1 == ST ? 0 : stg + 1;
+            stage_addrs(stg);
+            read_frags(wa, xa, 0, fw[0], fx[0]);
+        }
+    }
+    if (loader) __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // repeats of the last slab must land before LDS is released
+}
+
 struct GemmInst {
     int combo, bs_last, dd, tm, tn, tk, threads, lds, epc;
     int ktail;  // takes c that is not a multiple of tk
     int wm;     // waves along the TM side
-    int pers;   // persistent workgroups with split memory roles (ks_gemm_pbf_kernel)
+    int pers;   // persistent workgroups with split memory roles (ks_gemm_pbf_kernel, ks_gemm_pbl_kernel)
     const void *fn[2];  // plain, with bias/activation
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
@@ -947,6 +1246,12 @@ struct GemmInst {
     {1, false, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
      8, 0, WM_, 1, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, false>, \
                     (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
+#define GEMM_INST_PL(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_)                                  \
+    {COMBO_, true, 1, TM_, TN_, TK_, 64 * WM_ * WN_,                                                  \
+     GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES + WM_ * WN_ * 32 * 144,           \
+     GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::EPC, 0, WM_, 1,                             \
+     {(const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, false>,               \
+      (const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
 #define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
     GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
@@ -1004,6 +1309,13 @@ const GemmInst gemm_insts[] = {
     // fp16, bs_first: persistent workgroups, loads and stores issued by different waves
     GEMM_INST_P(2, 256, 128, 32, 4, 2, 3),
     GEMM_INST_P(2, 128, 256, 32, 2, 4, 3),
+    // persistent, bs_last
+    GEMM_INST_PL(1, half_t, half_t, 256, 256, 32, 2, 4, 3),
+    GEMM_INST_PL(1, half_t, half_t, 128, 256, 32, 2, 4, 4),
+    GEMM_INST_PL(0, float, float, 128, 256, 16, 2, 4, 4),
+    GEMM_INST_PL(0, float, float, 256, 256, 16, 2, 4, 3),
+    GEMM_INST_PL(2, fp8_t, half_t, 256, 256, 64, 2, 4, 3),
+    GEMM_INST_PL(2, fp8_t, half_t, 128, 256, 64, 2, 4, 4),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
@@ -1074,18 +1386,20 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
     if (variant < 0 && !gemm_insts[pick].pers) {
-        // three or more tiles per CU: the persistent form of the same tile saves the per-tile
-        // prologue and keeps the load stream running (8 % on (1,1536,384,2) at batch 25088)
+        // three or more tiles per CU: the persistent forms save the per-tile prologue and keep the
+        // load stream running (8 % on (1,1536,384,2) fp16 batch-size-first at batch 25088 with the
+        // tile of the pick; batch-size-last: 12 % with the first persistent tile that still
+        // gives three tiles per CU, 5 % on fp32 (1,768,192,16))
         const GemmInst &o = gemm_insts[pick];
-        const int64_t groups = o.dd == 1 ? (int64_t)p.a * p.d : p.a;
-        const int64_t wgs = groups * (p.b / o.tm) * ((p.batch + o.tn - 1) / o.tn);
-        for (int i = 0; i < N_GEMM_INSTS && wgs >= 3 * 256; ++i) {
+        for (int i = 0; i < N_GEMM_INSTS; ++i) {
             const GemmInst &q = gemm_insts[i];
-            if (q.pers && q.combo == o.combo && q.bs_last == o.bs_last && q.dd == o.dd && q.tm == o.tm && q.tn == o.tn &&
-                q.tk == o.tk && gemm_fits(q, p, combo)) {
-                pick = i;
-                break;
-            }
+            if (!q.pers || q.combo != o.combo || q.bs_last != o.bs_last || q.dd != o.dd) continue;
+            if (!q.bs_last && (q.tm != o.tm || q.tn != o.tn || q.tk != o.tk)) continue;
+            if (!gemm_fits(q, p, combo)) continue;
+            const int64_t groups = q.dd == 1 ? (int64_t)p.a * p.d : p.a;
+            if (groups * (p.b / q.tm) * ((p.batch + q.tn - 1) / q.tn) < 3 * 256) continue;
+            pick = i;
+            break;
         }
     }
     const GemmInst &t = gemm_insts[pick];

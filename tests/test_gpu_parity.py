@@ -182,7 +182,7 @@ def test_gemm_kernels_forced_e4m3():
              ("fp8", True, (2, 256, 192, 1), 528), ("fp8", True, (1, 256, 96, 2), 1024),
              ("fp8", True, (1, 128, 70, 2), 1008), ("fp8", True, (2, 256, 40, 1), 272), ("fp8", True, (1, 128, 9, 1), 64),
              ("fp8", True, (1, 192, 128, 2), 528), ("fp8", True, (2, 64, 72, 1), 1008)]
-    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 36)], 3, 18)
+    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 48)], 3, 18)
 
 
 def _forced_sweep(cases, variants, algo, min_ran):
@@ -783,3 +783,63 @@ def test_persistent_gemm_walks_several_tiles_per_workgroup():
     for act, want in ((None, zb), ("gelu", zg)):
         y = Kernel.forward(x.half().cuda(), fac, False, a, b, c, d, bias=bias.cuda(), act=act)
         assert O.rel_fro_error(y.float().cpu().numpy()[rows], want) <= TOL["fp16"], act
+
+
+def test_persistent_gemm_batch_size_last():
+    """The persistent batch-size-last GEMM instances (fp16 and fp32) on problems with two to five
+    tiles per workgroup, d > 1, several a_i, a ragged last batch tile and 2-4 K slabs: the whole
+    output against the automatic choice, sampled columns against the oracle."""
+    from ksmm_amd import Kernel, generate_factor, _lib
+    from ksmm_amd.kernel import query_tile
+
+    batch = 20008
+    ran = 0
+    for prec, pattern in [("fp16", (1, 512, 96, 2)), ("fp16", (2, 256, 64, 3)), ("fp32", (2, 512, 64, 2)),
+                          ("fp32", (1, 768, 48, 3))]:
+        a, b, c, d = pattern
+        dt = TORCH_DTYPE[prec]
+        (w4,) = seeded_weights([pattern], seed=111)
+        x = seeded_input(a * c * d, batch, True, seed=112)
+        fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+        xin = x.to(dt).cuda()
+        ref = Kernel.forward(xin, fac, True, a, b, c, d)
+        cols = sample_columns(batch, step=389)
+        z = O.ks_apply_einsum(round_to(w4, prec)[0], round_to(x, prec)[0][:, cols], True)
+        assert O.rel_fro_error(ref.float().cpu().numpy()[:, cols], z) <= TOL[prec]
+        for inst in range(32, 64):
+            try:
+                t = query_tile(batch, pattern, dt, None, True, algo=3, variant=(4 << 24) | inst)
+            except _lib.KsmmError:
+                continue  # no such instance, or one that does not fit
+            if t["grid"] != 256:
+                continue  # one workgroup per tile: not a persistent instance
+            y = Kernel.forward(xin, fac, True, a, b, c, d, algo=3, variant=(4 << 24) | inst)
+            torch.cuda.synchronize()
+            ran += 1
+            assert torch.isfinite(y).all(), (prec, pattern, inst)
+            err = ((y.float() - ref.float()).norm() / ref.float().norm()).item()
+            assert err <= (1e-3 if prec == "fp16" else 2e-6), (prec, pattern, inst, err)
+            assert O.rel_fro_error(y.float().cpu().numpy()[:, cols], z) <= TOL[prec], (prec, pattern, inst)
+    assert ran >= 6, ran
+    # the e4m3 instances (the persistent ones are the last of the table), whole output against the oracle
+    _forced_sweep([("fp8", True, (1, 512, 128, 2), 20016)], [(4 << 24) | i for i in range(39, 48)], 3, 2)
+    # bias + GELU (an instantiation of its own), reached through the automatic choice: three
+    # tiles per CU make the heuristic take the persistent form
+    import scipy.special
+
+    for prec, pattern, batch in [("fp16", (1, 512, 96, 2), 49152), ("fp32", (2, 256, 64, 3), 32772)]:
+        a, b, c, d = pattern
+        dt = TORCH_DTYPE[prec]
+        t = query_tile(batch, pattern, dt, None, True)
+        assert t["algo"] == 3 and (t["variant"] >> 24) == 4 and t["grid"] == 256, t
+        (w4,) = seeded_weights([pattern], seed=113)
+        x = seeded_input(a * c * d, batch, True, seed=114)
+        fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+        bias = torch.from_numpy(np.random.default_rng(115).standard_normal(a * b * d).astype(np.float32)).to(dt)
+        cols = sample_columns(batch, step=997)
+        z = O.ks_apply_einsum(round_to(w4, prec)[0], round_to(x, prec)[0][:, cols], True)
+        zb = z + bias.double().numpy()[:, None]
+        zg = 0.5 * zb * (1.0 + scipy.special.erf(zb / np.sqrt(2.0)))
+        for act, want in ((None, zb), ("gelu", zg)):
+            y = Kernel.forward(x.to(dt).cuda(), fac, True, a, b, c, d, bias=bias.cuda(), act=act)
+            assert O.rel_fro_error(y.float().cpu().numpy()[:, cols], want) <= TOL[prec], (prec, act)
