@@ -938,8 +938,8 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbf_kernel(const CT *
 // two neighbouring 32-column blocks for fp16, one for fp32) and stores whole lines.  The pieces
 // are private, so a tile switch needs no workgroup barrier: waves that finish their part of
 // the tile early start on the next tile's first slab while the others still store.
-template <typename CT, typename TY, int TM, int TN, int TK, int WM, int WN, int ST, bool EPI>
-__global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbl_kernel(const CT *__restrict__ x,
+template <typename CT, typename TY, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool EPI>
+__global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT *__restrict__ x,
                                                                 const CT *__restrict__ w,
                                                                 TY *__restrict__ y, int batch, int a,
                                                                 int b, int c, int d, Epi ep,
@@ -1102,7 +1102,7 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbl_kernel(const CT *
     const int l32 = lane & 31, lq = lane >> 5;
     constexpr int TILE_STORES = C::MT * (C::NT / JP) * 4;  // stores of a wave per full tile
     static_assert(N_WAIT + TILE_STORES <= 63, "counter range");
-    static_assert(OUT_BASE + NWAVES * 32 * OP <= 160 * 1024, "ring and output pieces fit");
+    static_assert(OUT_BASE + NWAVES * 32 * OP <= 160 * 1024 / OCC, "ring and output pieces fit");
     unsigned char *const piece = smem + OUT_BASE + wave * (32 * OP);
     bool stores_behind = false;  // the previous tile issued exactly TILE_STORES stores (uniform)
     Tile cur = decode(0);
@@ -1231,7 +1231,7 @@ struct GemmInst {
     int combo, bs_last, dd, tm, tn, tk, threads, lds, epc;
     int ktail;  // takes c that is not a multiple of tk
     int wm;     // waves along the TM side
-    int pers;   // persistent workgroups with split memory roles (ks_gemm_pbf_kernel, ks_gemm_pbl_kernel)
+    int pers;   // persistent workgroups (per CU) with split memory roles (ks_gemm_pbf_kernel, ks_gemm_pbl_kernel)
     const void *fn[2];  // plain, with bias/activation
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
@@ -1246,12 +1246,13 @@ struct GemmInst {
     {1, false, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
      8, 0, WM_, 1, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, false>, \
                     (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
-#define GEMM_INST_PL(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_)                                  \
+// OCC_: persistent workgroups per CU (4-wave tiles: two)
+#define GEMM_INST_PL(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                            \
     {COMBO_, true, 1, TM_, TN_, TK_, 64 * WM_ * WN_,                                                  \
      GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES + WM_ * WN_ * 32 * 144,           \
-     GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::EPC, 0, WM_, 1,                             \
-     {(const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, false>,               \
-      (const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
+     GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::EPC, 0, WM_, OCC_,                          \
+     {(const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false>,         \
+      (const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, true>}}
 #define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
     GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
@@ -1310,12 +1311,17 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_P(2, 256, 128, 32, 4, 2, 3),
     GEMM_INST_P(2, 128, 256, 32, 2, 4, 3),
     // persistent, bs_last
-    GEMM_INST_PL(1, half_t, half_t, 256, 256, 32, 2, 4, 3),
-    GEMM_INST_PL(1, half_t, half_t, 128, 256, 32, 2, 4, 4),
-    GEMM_INST_PL(0, float, float, 128, 256, 16, 2, 4, 4),
-    GEMM_INST_PL(0, float, float, 256, 256, 16, 2, 4, 3),
-    GEMM_INST_PL(2, fp8_t, half_t, 256, 256, 64, 2, 4, 3),
-    GEMM_INST_PL(2, fp8_t, half_t, 128, 256, 64, 2, 4, 4),
+    GEMM_INST_PL(1, half_t, half_t, 256, 256, 32, 2, 4, 3, 1),
+    GEMM_INST_PL(1, half_t, half_t, 128, 256, 32, 2, 4, 4, 1),
+    GEMM_INST_PL(0, float, float, 128, 256, 16, 2, 4, 4, 1),
+    GEMM_INST_PL(0, float, float, 256, 256, 16, 2, 4, 3, 1),
+    GEMM_INST_PL(2, fp8_t, half_t, 256, 256, 64, 2, 4, 3, 1),
+    GEMM_INST_PL(2, fp8_t, half_t, 128, 256, 64, 2, 4, 4, 1),
+    // 4-wave tiles for b = 64, 192, ...: two persistent workgroups per CU
+    GEMM_INST_PL(1, half_t, half_t, 64, 256, 32, 1, 4, 3, 2),
+    GEMM_INST_PL(1, half_t, half_t, 64, 128, 32, 2, 2, 5, 2),
+    GEMM_INST_PL(0, float, float, 64, 256, 16, 1, 4, 3, 2),
+    GEMM_INST_PL(0, float, float, 64, 128, 16, 2, 2, 5, 2),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
@@ -1397,7 +1403,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             if (!q.bs_last && (q.tm != o.tm || q.tn != o.tn || q.tk != o.tk)) continue;
             if (!gemm_fits(q, p, combo)) continue;
             const int64_t groups = q.dd == 1 ? (int64_t)p.a * p.d : p.a;
-            if (groups * (p.b / q.tm) * ((p.batch + q.tn - 1) / q.tn) < 3 * 256) continue;
+            if (groups * (p.b / q.tm) * ((p.batch + q.tn - 1) / q.tn) < 3 * 256 * q.pers) continue;
             pick = i;
             break;
         }
@@ -1408,7 +1414,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int64_t groups = t.dd == 1 ? (int64_t)p.a * p.d : p.a;
     const int64_t blocks = groups * m_tiles * n_tiles;
     int64_t grid = (blocks + 7) / 8 * 8;
-    if (t.pers && grid > 256) grid = 256;  // one persistent workgroup per CU
+    if (t.pers && grid > 256 * t.pers) grid = 256 * t.pers;  // persistent workgroups: pers per CU
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_TILE;

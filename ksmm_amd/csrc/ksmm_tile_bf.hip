@@ -196,9 +196,445 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
         }
 }
 
+// ------------------------------------------------------------------------------------------
+// Groups of 8 fp16 blocks with a register pipeline several slabs deep (TK = 16, one MFMA step
+// per slab and block).  The plain kernel above keeps one slab in flight while it multiplies the
+// previous one, and its padded planes leave room for one workgroup per CU: with 8 blocks per
+// group a slab is 32 KB (half of it weights, which every batch tile reads again through L2),
+// so it waits out a memory latency per slab.  Here
+//  * a thread's loads of input slab s + PDX and weight slab s + PDW are issued before slab s is
+//    multiplied (16 registers per slab and operand);
+//  * eight neighbouring lanes read the 128 bytes (8 k x 8 d_i) a row holds per line, so a load
+//    instruction touches 8 whole lines when d = 8; a thread gets k and k + 8 of its row, turns
+//    the two vectors into 8 x (2 k of one d_i) with 8 byte permutes and writes them with
+//    4-byte LDS stores.  Inside a slab k therefore sits at position 2 * (k % 8) + k / 8, in the
+//    planes and in the weight rows alike (the order of a sum does not matter to the product);
+//  * the planes are unpadded rows of 16 k, their two 16-byte halves swapped for rows 8..15 of
+//    every 16 (the 16 rows a 16-byte operand read covers then fall on distinct banks);
+// which brings LDS to 72 KB: two workgroups per CU, four slabs of 32 KB in flight.
+template <typename TW, int TM, int TN, int WM, int WN, int PDX, int PDW>
+__global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_bf8_kernel(const half_t *__restrict__ x,
+                                                                const TW *__restrict__ w,
+                                                                half_t *__restrict__ y, int batch, int a,
+                                                                int b, int c, int d, Epi ep,
+                                                                int m_tiles, int n_tiles, int blocks)
+{
+    constexpr int DD = 8, TK = 16, THREADS = 64 * WM * WN;
+    constexpr int MT = TM / WM / 32, NT = TN / WN / 32;
+    constexpr int LDW = pads<half_t>::outer(TM);
+    constexpr int W_ELEMS = DD * TK * LDW, X_ELEMS = DD * TN * TK;
+    constexpr int W_EPV = stage<TW, half_t>::EPV;
+    constexpr int W_VECS = DD * TK * TM / W_EPV, W_PER_T = W_VECS / THREADS;
+    constexpr int X_QUADS = TN * TK / 2, XQ_PER_T = X_QUADS / THREADS;  // pairs (k, k + 8) of a row
+    static_assert(W_VECS % THREADS == 0 && X_QUADS % THREADS == 0, "whole loads per thread");
+    static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0, "wave tiling");
+    static_assert(2 * (W_ELEMS + X_ELEMS) * 2 <= (WM * WN >= 8 ? 160 : 80) * 1024, "8 waves per CU");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    half_t *const lds = (half_t *)smem;
+    auto ws = [&](int buf, int dd) { return lds + buf * W_ELEMS + dd * TK * LDW; };
+    auto xs = [&](int buf, int dd) { return lds + 2 * W_ELEMS + buf * X_ELEMS + dd * TN * TK; };
+
+    const int per_xcd = (blocks + 7) / 8;
+    const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lid >= blocks) return;
+    const int n_dg = d / DD;  // groups of DD blocks
+    const int mt_id = lid % m_tiles;
+    int rest = lid / m_tiles;
+    const int dg = rest % n_dg;
+    rest /= n_dg;
+    const int nt_id = rest % n_tiles;
+    const int a_i = rest / n_tiles;
+    const int m0 = mt_id * TM, n0 = nt_id * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
+    const half_t *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
+
+    stage<TW, half_t> wreg[PDW][W_PER_T];
+    uint4_t xreg[PDX][XQ_PER_T][2];
+    // The loads of a slab are issued unconditionally: a branch around them would leave the
+    // compiler two histories of the load counter to merge, and it would then wait for every
+    // load in flight before it touches a register of the pipeline.  Behind the last slab
+    // (live == false) every lane reads the first 16 bytes of the tile instead (one line): the
+    // offsets are masked, not selected, so that no branch comes back.  Addresses are a uniform
+    // base per tile plus a 32-bit offset per lane (the host checks that they fit).
+    const TW *const wt = w + ((size_t)(a_i * d + dg * DD) * c) * b + m0;
+    const half_t *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DD;
+    uint32_t woff[W_PER_T], xoff[XQ_PER_T];
+#pragma unroll
+    for (int i = 0; i < W_PER_T; ++i) {
+        const int v = tid + i * THREADS;
+        constexpr int per_dd = TK * TM / W_EPV;
+        const int dd = v / per_dd, r = v % per_dd;
+        const int kk = r / (TM / W_EPV), mm = (r % (TM / W_EPV)) * W_EPV;
+        woff[i] = (uint32_t)((dd * c + kk) * b + mm);
+    }
+#pragma unroll
+    for (int i = 0; i < XQ_PER_T; ++i) {
+        const int v = tid + i * THREADS;
+        const int nn = v >> 3, k8 = v & 7;
+        xoff[i] = (uint32_t)(min(nn, batch - 1 - n0) * (uint32_t)in_size + k8 * d);
+    }
+    auto live_mask = [](bool live) {
+        int lv = live;
+        asm volatile("" : "+v"(lv));  // opaque: stays a mask
+        return 0u - (uint32_t)lv;
+    };
+    auto gload_w = [&](int slot, int k0, bool live) {
+        const uint32_t mk = live_mask(live);
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) wreg[slot][i].load(wt + ((woff[i] + (uint32_t)(k0 * b)) & mk));
+    };
+    auto gload_x = [&](int slot, int k0, bool live) {
+        const uint32_t mk = live_mask(live);
+#pragma unroll
+        for (int i = 0; i < XQ_PER_T; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                xreg[slot][i][j] = *(const uint4_t *)(xt + ((xoff[i] + (uint32_t)((k0 + 8 * j) * d)) & mk));
+    };
+    auto lstore = [&](int wslot, int slot, int buf) {
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) {
+            const int v = tid + i * THREADS;
+            constexpr int per_dd = TK * TM / W_EPV;
+            const int dd = v / per_dd, r = v % per_dd;
+            const int kk = r / (TM / W_EPV), mm = (r % (TM / W_EPV)) * W_EPV;
+            wreg[wslot][i].store(ws(buf, dd) + (2 * (kk & 7) + (kk >> 3)) * LDW + mm);
+        }
+#pragma unroll
+        for (int i = 0; i < XQ_PER_T; ++i) {
+            const int v = tid + i * THREADS;
+            const int nn = v >> 3, k8 = v & 7;
+            // k = k8 and k8 + 8 of row nn: positions 2 * k8 and 2 * k8 + 1, i.e. 4-byte piece k8 & 3
+            // of the 16-byte half k8 >> 2 (swapped for rows 8..15 of every 16)
+            half_t *const dst = xs(buf, 0) + nn * TK + ((((k8 >> 2) ^ ((nn >> 3) & 1)) << 3) | ((k8 & 3) << 1));
+            const uint4_t c0 = xreg[slot][i][0], c1 = xreg[slot][i][1];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                // register p of a vector holds d_i = 2p (low half) and 2p + 1 (high half)
+                *(uint32_t *)(dst + (2 * p) * TN * TK) = __builtin_amdgcn_perm(c1[p], c0[p], 0x05040100u);
+                *(uint32_t *)(dst + (2 * p + 1) * TN * TK) = __builtin_amdgcn_perm(c1[p], c0[p], 0x07060302u);
+            }
+        }
+    };
+
+    float16_t acc[DD][MT][NT];
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = 0.f;
+
+    const int l32 = lane & 31, lq = lane >> 5;
+    int xrow[NT];  // the lane's operand inside a plane, in elements
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int n = (wn * NT + j) * 32 + l32;
+        xrow[j] = n * TK + ((lq ^ ((n >> 3) & 1)) << 3);
+    }
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) {
+            const half_t *wb = ws(buf, dd), *xb = xs(buf, dd);
+            half8_t fw[MT], fx[NT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i) fw[i] = frag<half_t>::k_outer(wb, LDW, (wm * MT + i) * 32, 0, lane);
+#pragma unroll
+            for (int j = 0; j < NT; ++j) fx[j] = *(const half8_t *)(xb + xrow[j]);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[dd][i][j] = frag<half_t>::mfma(fx[j], fw[i], acc[dd][i][j]);
+        }
+    };
+
+    const int steps = c / TK;
+    // slab s: request weights PDW and input PDX slabs ahead into the slots slab s came from (it
+    // went to LDS an iteration ago), multiply slab s, move slab s + 1 from its registers to
+    // the other LDS buffer.  The weights come from L2 and get the shorter lead; they are
+    // requested first, so that waiting for them leaves the younger input loads in flight.
+    constexpr int PERIOD = PDX * PDW / (PDX % PDW == 0 ? PDW : PDW % PDX == 0 ? PDX : 1);
+    static_assert(PERIOD % PDX == 0 && PERIOD % PDW == 0, "slots repeat after PERIOD slabs");
+    auto slab = [&](int u, int s) {
+        gload_w(u % PDW, (s + PDW) * TK, s + PDW < steps);
+        gload_x(u % PDX, (s + PDX) * TK, s + PDX < steps);
+        // (the permutes of the next slab's vectors must not move up here: they would wait for
+        // that slab before this one is multiplied)
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(s & 1);
+        __builtin_amdgcn_sched_barrier(0);
+        lstore((u + 1) % PDW, (u + 1) % PDX, (s & 1) ^ 1);  // behind the last slab: whatever the idle loads brought
+        __syncthreads();
+    };
+#pragma unroll
+    for (int u = 0; u < (PDX > PDW ? PDX : PDW); ++u) {
+        if (u < PDW) gload_w(u, u * TK, u < steps);
+        if (u < PDX) gload_x(u, u * TK, u < steps);
+    }
+    lstore(0, 0, 0);
+    __syncthreads();
+    int s = 0;
+    for (; s + PERIOD <= steps; s += PERIOD) {
+#pragma unroll
+        for (int u = 0; u < PERIOD; ++u) slab(u, s + u);
+    }
+#pragma unroll
+    for (int u = 0; u < PERIOD - 1; ++u)
+        if (s + u < steps) slab(u, s + u);
+
+    // D tile: lane holds output column m = lane % 32, batch rows 8*(e/4) + 4*(lane/32) + e%4;
+    // the 8 results of one (n, m) are adjacent in y: one 16-byte store
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int m = m0 + (wm * MT + i) * 32 + l32;
+            const int nb = n0 + (wn * NT + j) * 32;
+            float bv[DD];
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) bv[dd] = epi_bias<half_t>(ep, ((size_t)a_i * b + m) * d + dg * DD + dd);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int n = nb + 8 * (e >> 2) + 4 * lq + (e & 3);
+                pack_t<half_t, DD> o;
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd) o.e[dd] = (half_t)epi_finish(ep, acc[dd][i][j][e], bv[dd]);
+                if (n < batch)
+                    *(pack_t<half_t, DD> *)(y + (size_t)n * out_size + ((size_t)a_i * b + m) * d + dg * DD) = o;
+            }
+        }
+}
+
+// The same pipeline for groups of 4 fp32 blocks (a 16-byte vector is one k of 4 d_i, so the
+// vectors are split by plain 4-byte LDS stores and k keeps its place).  One MFMA step is 2 k:
+// 32 steps per slab and wave, so this form is matrix-core-bound where the fp16 one waits for
+// memory; what it buys over the plain kernel is a second wave per SIMD (64 KB of LDS, 64
+// accumulator registers), which hides the LDS latency in front of every MFMA.  Plane rows are
+// 16 floats, element k of row n at k ^ 2 * ((n / 4) % 8): the 32 rows an operand read covers
+// fall on distinct banks.  Weight rows are unpadded too: the columns of odd k are XORed with 32,
+// so the two rows an operand read covers use different bank halves.
+template <int TM, int TN, int WM, int WN, int PDX, int PDW>
+__global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_bf4_kernel(const float *__restrict__ x,
+                                                                const float *__restrict__ w,
+                                                                float *__restrict__ y, int batch, int a,
+                                                                int b, int c, int d, Epi ep,
+                                                                int m_tiles, int n_tiles, int blocks)
+{
+    typedef float TW;
+    constexpr int DD = 4, TK = 16, THREADS = 64 * WM * WN;
+    constexpr int MT = TM / WM / 32, NT = TN / WN / 32;
+    constexpr int LDW = TM;  // unpadded: columns of odd rows are XORed with 32 instead
+    constexpr int W_ELEMS = DD * TK * LDW, X_ELEMS = DD * TN * TK;
+    constexpr int W_EPV = stage<float, float>::EPV;
+    constexpr int W_VECS = DD * TK * TM / W_EPV, W_PER_T = W_VECS / THREADS;
+    constexpr int X_QUADS = TN * TK / 2, XQ_PER_T = X_QUADS / THREADS;  // pairs (k, k + 8) of a row
+    static_assert(W_VECS % THREADS == 0 && X_QUADS % THREADS == 0, "whole loads per thread");
+    static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0, "wave tiling");
+    static_assert(2 * (W_ELEMS + X_ELEMS) * 4 <= (WM * WN >= 8 ? 160 : 80) * 1024, "8 waves per CU");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float *const lds = (float *)smem;
+    auto ws = [&](int buf, int dd) { return lds + buf * W_ELEMS + dd * TK * LDW; };
+    auto xs = [&](int buf, int dd) { return lds + 2 * W_ELEMS + buf * X_ELEMS + dd * TN * TK; };
+
+    const int per_xcd = (blocks + 7) / 8;
+    const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lid >= blocks) return;
+    const int n_dg = d / DD;  // groups of DD blocks
+    const int mt_id = lid % m_tiles;
+    int rest = lid / m_tiles;
+    const int dg = rest % n_dg;
+    rest /= n_dg;
+    const int nt_id = rest % n_tiles;
+    const int a_i = rest / n_tiles;
+    const int m0 = mt_id * TM, n0 = nt_id * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
+    const float *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
+
+    stage<float, float> wreg[PDW][W_PER_T];
+    uint4_t xreg[PDX][XQ_PER_T][2];
+    // The loads of a slab are issued unconditionally: a branch around them would leave the
+    // compiler two histories of the load counter to merge, and it would then wait for every
+    // load in flight before it touches a register of the pipeline.  Behind the last slab
+    // (live == false) every lane reads the first 16 bytes of the tile instead (one line): the
+    // offsets are masked, not selected, so that no branch comes back.  Addresses are a uniform
+    // base per tile plus a 32-bit offset per lane (the host checks that they fit).
+    const TW *const wt = w + ((size_t)(a_i * d + dg * DD) * c) * b + m0;
+    const float *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DD;
+    uint32_t woff[W_PER_T], xoff[XQ_PER_T];
+#pragma unroll
+    for (int i = 0; i < W_PER_T; ++i) {
+        const int v = tid + i * THREADS;
+        constexpr int per_dd = TK * TM / W_EPV;
+        const int dd = v / per_dd, r = v % per_dd;
+        const int kk = r / (TM / W_EPV), mm = (r % (TM / W_EPV)) * W_EPV;
+        woff[i] = (uint32_t)((dd * c + kk) * b + mm);
+    }
+#pragma unroll
+    for (int i = 0; i < XQ_PER_T; ++i) {
+        const int v = tid + i * THREADS;
+        const int nn = v >> 3, k8 = v & 7;
+        xoff[i] = (uint32_t)(min(nn, batch - 1 - n0) * (uint32_t)in_size + k8 * d);
+    }
+    auto live_mask = [](bool live) {
+        int lv = live;
+        asm volatile("" : "+v"(lv));  // opaque: stays a mask
+        return 0u - (uint32_t)lv;
+    };
+    auto gload_w = [&](int slot, int k0, bool live) {
+        const uint32_t mk = live_mask(live);
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) wreg[slot][i].load(wt + ((woff[i] + (uint32_t)(k0 * b)) & mk));
+    };
+    auto gload_x = [&](int slot, int k0, bool live) {
+        const uint32_t mk = live_mask(live);
+#pragma unroll
+        for (int i = 0; i < XQ_PER_T; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                xreg[slot][i][j] = *(const uint4_t *)(xt + ((xoff[i] + (uint32_t)((k0 + 8 * j) * d)) & mk));
+    };
+    auto lstore = [&](int wslot, int slot, int buf) {
+#pragma unroll
+        for (int i = 0; i < W_PER_T; ++i) {
+            const int v = tid + i * THREADS;
+            constexpr int per_dd = TK * TM / W_EPV;
+            const int dd = v / per_dd, r = v % per_dd;
+            const int kk = r / (TM / W_EPV), mm = (r % (TM / W_EPV)) * W_EPV;
+            wreg[wslot][i].store(ws(buf, dd) + kk * LDW + (mm ^ (32 * (kk & 1))));
+        }
+#pragma unroll
+        for (int i = 0; i < XQ_PER_T; ++i) {
+            const int v = tid + i * THREADS;
+            const int nn = v >> 3, k8 = v & 7;
+            // k = k8 and k8 + 8 of row nn, element k at k ^ 2 * ((nn / 4) % 8)
+            float *const dst = xs(buf, 0) + nn * TK;
+            const int fn = 2 * ((nn >> 2) & 7);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint4_t cj = xreg[slot][i][j];
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd) *(uint32_t *)(dst + dd * TN * TK + ((k8 + 8 * j) ^ fn)) = cj[dd];
+            }
+        }
+    };
+
+    float16_t acc[DD][MT][NT];
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[dd][i][j][e] = 0.f;
+
+    const int l32 = lane & 31, lq = lane >> 5;
+    int xrow[NT], xfn[NT];  // the lane's row inside a plane (elements) and its column swizzle
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int n = (wn * NT + j) * 32 + l32;
+        xrow[j] = n * TK;
+        xfn[j] = 2 * ((n >> 2) & 7);
+    }
+    // operands of MFMA step k0 + 2 are requested before the MFMAs of step k0 are issued
+    auto multiply = [&](int buf) {
+        float fw[2][DD][MT], fx[2][DD][NT];
+        auto read = [&](int k0, float(&rw)[DD][MT], float(&rx)[DD][NT]) {
+            int xcol[NT];
+#pragma unroll
+            for (int j = 0; j < NT; ++j) xcol[j] = xrow[j] + ((k0 + lq) ^ xfn[j]);
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) {
+                const float *wb = ws(buf, dd), *xb = xs(buf, dd);
+#pragma unroll
+                for (int i = 0; i < MT; ++i) rw[dd][i] = wb[(k0 + lq) * LDW + (((wm * MT + i) * 32 + l32) ^ (32 * lq))];
+#pragma unroll
+                for (int j = 0; j < NT; ++j) rx[dd][j] = xb[xcol[j]];
+            }
+        };
+        read(0, fw[0], fx[0]);
+#pragma unroll
+        for (int ks = 0; ks < TK / 2; ++ks) {
+            if (ks + 1 < TK / 2) read(2 * ks + 2, fw[(ks + 1) & 1], fx[(ks + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);  // (the scheduler would sink the reads to their uses)
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        acc[dd][i][j] = frag<float>::mfma(fx[ks & 1][dd][j], fw[ks & 1][dd][i], acc[dd][i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const int steps = c / TK;
+    // slab s: request weights PDW and input PDX slabs ahead into the slots slab s came from (it
+    // went to LDS an iteration ago), multiply slab s, move slab s + 1 from its registers to
+    // the other LDS buffer.  The weights come from L2 and get the shorter lead; they are
+    // requested first, so that waiting for them leaves the younger input loads in flight.
+    constexpr int PERIOD = PDX * PDW / (PDX % PDW == 0 ? PDW : PDW % PDX == 0 ? PDX : 1);
+    static_assert(PERIOD % PDX == 0 && PERIOD % PDW == 0, "slots repeat after PERIOD slabs");
+    auto slab = [&](int u, int s) {
+        gload_w(u % PDW, (s + PDW) * TK, s + PDW < steps);
+        gload_x(u % PDX, (s + PDX) * TK, s + PDX < steps);
+        // (the LDS stores of the next slab must not move up here: they would wait for that slab
+        // before this one is multiplied)
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(s & 1);
+        __builtin_amdgcn_sched_barrier(0);
+        lstore((u + 1) % PDW, (u + 1) % PDX, (s & 1) ^ 1);  // behind the last slab: whatever the idle loads brought
+        __syncthreads();
+    };
+#pragma unroll
+    for (int u = 0; u < (PDX > PDW ? PDX : PDW); ++u) {
+        if (u < PDW) gload_w(u, u * TK, u < steps);
+        if (u < PDX) gload_x(u, u * TK, u < steps);
+    }
+    lstore(0, 0, 0);
+    __syncthreads();
+    int s = 0;
+    for (; s + PERIOD <= steps; s += PERIOD) {
+#pragma unroll
+        for (int u = 0; u < PERIOD; ++u) slab(u, s + u);
+    }
+#pragma unroll
+    for (int u = 0; u < PERIOD - 1; ++u)
+        if (s + u < steps) slab(u, s + u);
+
+    // D tile: lane holds output column m = lane % 32, batch rows 8*(e/4) + 4*(lane/32) + e%4;
+    // the 4 results of one (n, m) are adjacent in y: one 16-byte store
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int m = m0 + (wm * MT + i) * 32 + l32;
+            const int nb = n0 + (wn * NT + j) * 32;
+            float bv[DD];
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) bv[dd] = epi_bias<float>(ep, ((size_t)a_i * b + m) * d + dg * DD + dd);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int n = nb + 8 * (e >> 2) + 4 * lq + (e & 3);
+                pack_t<float, DD> o;
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd) o.e[dd] = epi_finish(ep, acc[dd][i][j][e], bv[dd]);
+                if (n < batch)
+                    *(pack_t<float, DD> *)(y + (size_t)n * out_size + ((size_t)a_i * b + m) * d + dg * DD) = o;
+            }
+        }
+}
+
 struct BfInst {
     int combo, dd, tm, tn, tk, threads, lds, wm;
     const void *fn;
+    int pd;  // slabs in flight in registers, input * 16 + weights (ks_tile_bf8_kernel); 0: the plain kernel
 };
 #define BF_INST(COMBO_, CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_)                                  \
     {COMBO_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, BfCfg<CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, WM_, \
@@ -212,6 +648,15 @@ struct BfInst {
 #define BF_SET_H8(COMBO_, TW_)                                                                   \
     BF_INST(COMBO_, half_t, TW_, 8, 64, 64, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 8, 64, 64, 16, 2, 2), \
         BF_INST(COMBO_, half_t, TW_, 8, 32, 128, 16, 1, 4), BF_INST(COMBO_, half_t, TW_, 8, 128, 64, 16, 4, 2)
+#define BF8_INST(COMBO_, TW_, TM_, TN_, WM_, WN_, PDX_, PDW_)                                    \
+    {COMBO_, 8, TM_, TN_, 16, 64 * WM_ * WN_,                                                    \
+     2 * 2 * (8 * 16 * pads<half_t>::outer(TM_) + 8 * TN_ * 16), WM_,                            \
+     (const void *)ks_tile_bf8_kernel<TW_, TM_, TN_, WM_, WN_, PDX_, PDW_>, PDX_ * 16 + PDW_}
+#define BF4_INST(TM_, TN_, WM_, WN_, PDX_, PDW_)                                                 \
+    {0, 4, TM_, TN_, 16, 64 * WM_ * WN_, 2 * 4 * (4 * 16 * TM_ + 4 * TN_ * 16), WM_,                 \
+     (const void *)ks_tile_bf4_kernel<TM_, TN_, WM_, WN_, PDX_, PDW_>, PDX_ * 16 + PDW_}
+#define BF8_SET(COMBO_, TW_)                                                                     \
+    BF8_INST(COMBO_, TW_, 64, 64, 2, 2, 2, 2), BF8_INST(COMBO_, TW_, 64, 128, 2, 4, 2, 2)
 const BfInst bf_insts[] = {
     BF_SET_H(1, half_t),
     BF_SET_H(3, fp8_t),
@@ -223,6 +668,12 @@ const BfInst bf_insts[] = {
     // appended (ids of the rows above stay): 16-bit groups of 8 blocks
     BF_SET_H8(1, half_t),
     BF_SET_H8(3, fp8_t),
+    // the same groups with a register pipeline (ks_tile_bf8_kernel)
+    BF8_SET(1, half_t),
+    BF8_SET(3, fp8_t),
+    // fp32 groups of 4 (ks_tile_bf4_kernel)
+    BF4_INST(64, 64, 2, 2, 2, 2),
+    BF4_INST(64, 128, 2, 4, 2, 2),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
@@ -236,6 +687,11 @@ bool bf_fits(const BfInst &t, const Problem &p, int combo)
     if (p.b % w_epv) return false;
     // rows of x start at multiples of in_size, slabs at multiples of TK * d: keep 16-byte alignment
     if (((int64_t)p.a * p.c * p.d) % x_epv || ((int64_t)p.c * p.d) % x_epv) return false;
+    if (t.pd) {
+        // 32-bit element offsets inside a tile: TN rows of x, DD blocks of w
+        if ((int64_t)t.tn * p.a * p.c * p.d + (int64_t)p.c * p.d >= 0xffffffffLL) return false;
+        if ((int64_t)t.dd * p.c * p.b >= 0xffffffffLL) return false;
+    }
     return true;
 }
 
@@ -247,8 +703,8 @@ uint32_t bf_inst_id(int i)
 {
     if (i < 0 || i >= N_BF_INSTS) return 0;
     const BfInst &t = bf_insts[i];
-    const int v[7] = {t.combo, t.dd, t.tm, t.tn, t.tk, t.threads, t.wm};
-    return inst_hash('B', v, 7);
+    const int v[8] = {t.combo, t.dd, t.tm, t.tn, t.tk, t.threads, t.wm, t.pd};
+    return inst_hash('B', v, t.pd ? 8 : 7);  // (ids of the plain instances predate the field)
 }
 
 
@@ -275,6 +731,9 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             }
             const int64_t wgs = (int64_t)p.a * (p.d / t.dd) * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
             int64_t score = (int64_t)t.tm * 1000 + t.tn;
+            // the pipelined 64 x 64 form first (1.1-1.3x the plain instances on (1,192,192,8..16),
+            // (4,128,128,8), (1,64,64,64) at batch 25088)
+            if (t.pd && t.tn == 64 && wgs >= 512) score += 500000;
             if (wgs < 512) score -= 100000;
             if (score > best) {
                 best = score;
