@@ -421,7 +421,9 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int64_t ag = (int64_t)p.a * (p.d / t.dd);  // (a_i, group) pairs
     // one round of workgroups, 8 or more waves per CU
     const int per_cu_lds = 160 * 1024 / t.lds, per_cu_waves = 16 / t.dd > 0 ? 16 / t.dd : 1;
-    if (wgs <= 0) wgs = (256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves) + ag - 1) / ag;
+    // (rounded down: a few workgroups beyond one round would cost a whole second round)
+    if (wgs <= 0) wgs = 256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves) / ag;
+    if (wgs <= 0) wgs = 1;
     if (wgs > n_tiles) wgs = n_tiles;
     const int64_t grid = ag * wgs;
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;

@@ -722,11 +722,16 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             if (!bf_fits(t, p, combo)) continue;
             // Groups out of a larger d: every line of x is shared by d/DD groups x b/TM tiles, and
             // the loads are 16-byte pieces d elements apart.  Against the transposed route (two
-            // extra passes, but the fastest kernels in between) this wins for moderate d and b:
-            // measured over 178 patterns at batch 25088, mean time ratio 0.6-0.9 inside these
-            // bounds and 1.1-1.4 outside (large b re-reads x too often, large d scatters it).
+            // extra passes, but the fastest kernels in between) this wins while b x d stays
+            // moderate: measured at batch 25088 on 33 patterns around these bounds with the
+            // pipelined instances, time ratio 0.5-0.9 inside (fp16 (1,64,256,128) 1277 -> 765 us,
+            // (1,512,128,16) 333 -> 257; fp32 (1,512,128,8) 466 -> 328) and 1.0-1.3 outside
+            // ((1,768,192,24) fp16, (1,192,192,32) fp32, very long c).
             if (p.d != t.dd) {
-                const bool pays = combo == 0 ? (p.d <= 16 && p.b <= 192) : (p.d <= 32 && p.b <= 384 && t.tm >= 64);
+                const int64_t bd = (int64_t)p.b * p.d;
+                const bool pays = combo == 0 ? ((p.d <= 16 && p.b <= 192) || (bd <= 8192 && (p.d <= 16 || p.c <= 128)))
+                                             : (t.tm >= 64 && ((p.d <= 32 && p.b <= 384) ||
+                                                               (p.c <= 256 && (p.b <= 192 ? p.d <= 128 : bd <= 12288))));
                 if (!pays) continue;
             }
             const int64_t wgs = (int64_t)p.a * (p.d / t.dd) * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
