@@ -938,7 +938,7 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbf_kernel(const CT *
 // two neighbouring 32-column blocks for fp16, one for fp32) and stores whole lines.  The pieces
 // are private, so a tile switch needs no workgroup barrier: waves that finish their part of
 // the tile early start on the next tile's first slab while the others still store.
-template <typename CT, typename TY, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool EPI>
+template <typename CT, typename TY, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool MTAIL, bool EPI>
 __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT *__restrict__ x,
                                                                 const CT *__restrict__ w,
                                                                 TY *__restrict__ y, int batch, int a,
@@ -995,13 +995,14 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT
     constexpr int SWZ_ROWS = C::ES == 1 ? 8 : C::ES == 2 ? 4 : 2;  // rows after which the chunk swizzle repeats
     static_assert(LOADERS % C::W_CPR == 0 && W_ROWS_PER % SWZ_ROWS == 0 && W_ROWS_PER * LW == TK, "uniform weight chunk strides");
     static_assert(LOADERS % C::X_CPR == 0 && X_ROWS_PER % SWZ_ROWS == 0 && X_ROWS_PER * LX == TK, "uniform input chunk strides");
-    uint32_t wvoff0, xvoff0, xrow_off;
-    int xcol;
+    uint32_t wvoff0, xvoff0, xrow_off, wrow_off;
+    int xcol, wcol;
     {
         const int q = tid & (LOADERS - 1);
         const int row = q / C::W_CPR, pc = q % C::W_CPR;
-        const int col = (pc ^ swz_outer<CT, C::W_CPR>(row)) * C::EPC;
-        wvoff0 = (uint32_t)(((size_t)row * b + col) * C::ES);
+        wcol = (pc ^ swz_outer<CT, C::W_CPR>(row)) * C::EPC;
+        wrow_off = (uint32_t)((size_t)row * b * C::ES);
+        wvoff0 = wrow_off + (uint32_t)(wcol * C::ES);
         const int xrow = q / C::X_CPR, xpc = q % C::X_CPR;
         xcol = (xpc ^ swz_outer<CT, C::X_CPR>(xrow)) * C::EPC;
         xrow_off = (uint32_t)((size_t)xrow * d * batch * C::ES);
@@ -1015,6 +1016,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT
         i_x = (const char *)(x + ((size_t)q.a_i * c * d + q.d_i) * batch + q.n0);
         // the last batch tile repeats its last 16 bytes instead of reading past the end of a row
         xvoff0 = xrow_off + (uint32_t)(min(xcol, batch - C::EPC - q.n0) * C::ES);
+        // MTAIL: so does a last TM-tile that reaches beyond b (its rows behind b are not stored)
+        if constexpr (MTAIL) wvoff0 = wrow_off + (uint32_t)(min(wcol, b - C::EPC - q.m0) * C::ES);
     };
     // next slab of the stream; after the last one the load side stays there (the ring then
     // receives repeats of it, which keeps the number of loads per slab constant)
@@ -1169,7 +1172,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT
 #pragma unroll
             for (int i = 0; i < C::MT; ++i) {
                 const int mb = (wm * C::MT + i) * 32;
-                const float bl = epi_bias<TY>(ep, ((size_t)cur.a_i * b + cur.m0 + mb + l32) * d + cur.d_i);
+                const float bl = epi_bias<TY>(ep, ((size_t)cur.a_i * b + min(cur.m0 + mb + l32, b - 1)) * d + cur.d_i);
 #pragma unroll
                 for (int j = 0; j < C::NT; ++j)
 #pragma unroll
@@ -1210,12 +1213,14 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
                         const uint4_t v = *(const uint4_t *)(rd + 8 * t * OP);
-                        if (n < batch) __builtin_nontemporal_store(v, (uint4_t *)(dstp + (size_t)8 * t * d * batch));
+                        if (n < batch && (!MTAIL || row + 8 * t < b))
+                            __builtin_nontemporal_store(v, (uint4_t *)(dstp + (size_t)8 * t * d * batch));
                     }
                     __builtin_amdgcn_wave_barrier();
                 }
         }
-        stores_behind = cur.n0 + TN <= batch;  // a ragged tile skips stores: then wait the safe way
+        // a ragged tile skips stores: then wait the safe way
+        stores_behind = cur.n0 + TN <= batch && (!MTAIL || cur.m0 + TM <= b);
         if (c_t + 1 < my_tiles) {
             clear_acc();
             cur = decode(c_t + 1);
@@ -1233,6 +1238,7 @@ struct GemmInst {
     int wm;     // waves along the TM side
     int pers;   // persistent workgroups (per CU) with split memory roles (ks_gemm_pbf_kernel, ks_gemm_pbl_kernel)
     const void *fn[2];  // plain, with bias/activation
+    int mtail;  // takes b that is not a multiple of tm (the last TM-tile is partly masked)
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
 // so that one multiplies while the other stores its output tile)
@@ -1246,13 +1252,15 @@ struct GemmInst {
     {1, false, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
      8, 0, WM_, 1, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, false>, \
                     (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
-// OCC_: persistent workgroups per CU (4-wave tiles: two)
-#define GEMM_INST_PL(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                            \
+// OCC_: persistent workgroups per CU (4-wave tiles: two); MT_: partial last TM-tile
+#define GEMM_INST_PLM(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, MT_)                      \
     {COMBO_, true, 1, TM_, TN_, TK_, 64 * WM_ * WN_,                                                  \
      GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES + WM_ * WN_ * 32 * 144,           \
      GemmCfg<CT_, true, 1, TM_, TN_, TK_, WM_, WN_, ST_>::EPC, 0, WM_, OCC_,                          \
-     {(const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false>,         \
-      (const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, true>}}
+     {(const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, MT_, false>,    \
+      (const void *)ks_gemm_pbl_kernel<CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, MT_, true>}, MT_}
+#define GEMM_INST_PL(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                            \
+    GEMM_INST_PLM(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_T(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                   \
     GEMM_INST_K(COMBO_, CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false)
 #define GEMM_INST_O(COMBO_, CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                        \
@@ -1322,6 +1330,11 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_PL(1, half_t, half_t, 64, 128, 32, 2, 2, 5, 2),
     GEMM_INST_PL(0, float, float, 64, 256, 16, 1, 4, 3, 2),
     GEMM_INST_PL(0, float, float, 64, 128, 16, 2, 2, 5, 2),
+    // the same with a partly masked last TM-tile: b = 48, 80, 96, ... (named by the table only)
+    GEMM_INST_PLM(1, half_t, half_t, 64, 256, 32, 1, 4, 3, 2, true),
+    GEMM_INST_PLM(1, half_t, half_t, 64, 128, 32, 2, 2, 5, 2, true),
+    GEMM_INST_PLM(0, float, float, 64, 256, 16, 1, 4, 3, 2, true),
+    GEMM_INST_PLM(0, float, float, 64, 128, 16, 2, 2, 5, 2, true),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
@@ -1329,7 +1342,7 @@ constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
 bool gemm_fits(const GemmInst &t, const Problem &p, int combo)
 {
     if (t.combo != combo || t.bs_last != p.bs_last) return false;
-    if (p.b % t.tm || (p.c % t.tk && !t.ktail)) return false;
+    if ((p.b % t.tm && !t.mtail) || (p.c % t.tk && !t.ktail)) return false;
     if (p.b % t.epc) return false;  // 16-byte weight vectors
     if (p.bs_last) {
         if (p.batch % t.epc || p.batch < t.epc) return false;
@@ -1356,8 +1369,8 @@ uint32_t gemm_inst_id(int i)
     if (i < 0 || i >= N_GEMM_INSTS) return 0;
     const GemmInst &t = gemm_insts[i];
     // threads and the LDS footprint stand for the wave grid and the ring depth
-    const int v[11] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm, t.pers};
-    return inst_hash('G', v, 11);
+    const int v[12] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm, t.pers, t.mtail};
+    return inst_hash('G', v, t.mtail ? 12 : 11);  // (ids of the other instances predate the field)
 }
 
 // variant: index into the instance table; -1: first that fits with enough workgroups to fill
@@ -1374,7 +1387,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         // kernels) and partial K slabs; otherwise the stream and weight-stationary tiles come
         // first, then these (variant -4: 15-25 % faster than the k-loop tiles on 180 patterns
         // of the reference's list), then the k-loop tiles
-        if (variant < 0 && t.pers) continue;  // measured choices only (the table names them)
+        if (variant < 0 && (t.pers || t.mtail)) continue;  // measured choices only (the table names them)
         if (variant == -1 && t.tm < 128 && t.combo != 2 && !(t.ktail && p.c % t.tk)) continue;
         if (variant == -4 && t.tm >= 128) continue;  // -4: the TM = 64 tiles, after stream / weight-stationary
         // few K slabs: the 8-wave 256 x 256 tiles spend their time in prologue and epilogue; two
@@ -1399,7 +1412,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         const GemmInst &o = gemm_insts[pick];
         for (int i = 0; i < N_GEMM_INSTS; ++i) {
             const GemmInst &q = gemm_insts[i];
-            if (!q.pers || q.combo != o.combo || q.bs_last != o.bs_last || q.dd != o.dd) continue;
+            if (!q.pers || q.mtail || q.combo != o.combo || q.bs_last != o.bs_last || q.dd != o.dd) continue;
             if (!q.bs_last && (q.tm != o.tm || q.tn != o.tn || q.tk != o.tk)) continue;
             if (!gemm_fits(q, p, combo)) continue;
             const int64_t groups = q.dd == 1 ? (int64_t)p.a * p.d : p.a;
@@ -1409,7 +1422,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         }
     }
     const GemmInst &t = gemm_insts[pick];
-    const int m_tiles = p.b / t.tm;
+    const int m_tiles = (p.b + t.tm - 1) / t.tm;
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
     const int64_t groups = t.dd == 1 ? (int64_t)p.a * p.d : p.a;
     const int64_t blocks = groups * m_tiles * n_tiles;
