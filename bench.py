@@ -223,6 +223,35 @@ def copy_reference(steps, warmup):
             "bytes": nbytes, "kernel": "torch.add(x, 1, out=y) elementwise kernel"}
 
 
+def tiled_copy_reference(steps, warmup):
+    """A copy with the tile access pattern of the headline factor (1,48,48,16), fp32, bs_last:
+    48 rows of a block 16 rows apart, moved in pieces of 256 B .. 4 KB per row by one workgroup
+    per tile, no arithmetic.  What that access pattern reaches on this GPU, next to the linear
+    copy: the gap between the two is the price of the layout, not of the kernel."""
+    import ctypes
+
+    from ksmm_amd import _lib
+
+    lib = _lib.load()
+    n_sets = 4
+    src = [torch.randn(768, BATCH, device="cuda") for _ in range(n_sets)]
+    dst = [torch.zeros_like(t) for t in src]
+    nbytes = 2 * src[0].numel() * 4
+    res = {"bytes": nbytes, "kernel": "ksmm_tilecopy_probe: tiles of 48 rows x tile_bytes, rows 16 apart"}
+    for tile_bytes in (256, 1024, 4096):
+        def run(j):
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            _lib.check(lib.ksmm_tilecopy_probe(src[j].data_ptr(), dst[j].data_ptr(), BATCH * 4, 1, 48, 16, tile_bytes, stream))
+
+        run(0)
+        torch.cuda.synchronize()
+        if not torch.equal(src[0], dst[0]):
+            raise RuntimeError("tile copy probe: output differs from input")
+        sec = time_launches(run, n_sets, steps, warmup)
+        res["tile_%dB" % tile_bytes] = {"us": sec * 1e6, "gbs": nbytes / sec / 1e9, "frac_of_8tbs": nbytes / sec / 8e12}
+    return res
+
+
 def mfma_reference():
     """Rate at which the matrix cores multiply operands held in registers (no memory traffic at
     all), with all-ones and with random operands: what this GPU sustains next to the datasheet
@@ -352,6 +381,7 @@ def main():
         for cfg in CONFIGS[1:]:
             others.append(bench_config(*cfg, steps=max(20, args.steps // 2), warmup=max(5, args.warmup // 2)))
     copy_ref = copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
+    tiled_ref = tiled_copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     mfma_ref = mfma_reference()
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
     if args.cpu:
@@ -372,6 +402,7 @@ def main():
                      "unit": roof["unit"], "frac": roof["frac"], "traffic": traffic},
         "cpu_baseline": cpu,
         "copy_reference": copy_ref,
+        "tiled_copy_reference": tiled_ref,
         "mfma_reference": mfma_ref,
         "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),
                    "ok": head.get("parity_ok")},

@@ -1375,12 +1375,22 @@ uint32_t gemm_inst_id(int i)
 
 // variant: index into the instance table; -1: first that fits with enough workgroups to fill
 // the chip (TM = 64 tiles only where nothing better exists); -4: the TM = 64 tiles, same
-// condition; -2: first that fits
+// condition; -5: the persistent tiles with a masked last TM-tile, for b beyond one tile and
+// three tiles per persistent workgroup (they beat the k-loop tiles on 72 of 80 such patterns of
+// the reference's list, up to 2x); -2: first that fits
 int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     int pick = -1;
-    for (int i = 0; i < N_GEMM_INSTS; ++i) {
+    for (int i = 0; i < N_GEMM_INSTS && variant == -5; ++i) {
+        const GemmInst &t = gemm_insts[i];
+        if (!t.mtail || p.b <= t.tm || !gemm_fits(t, p, combo)) continue;
+        const int64_t tiles = (int64_t)p.a * p.d * ((p.b + t.tm - 1) / t.tm) * ((p.batch + t.tn - 1) / t.tn);
+        if (tiles < 3 * 256 * t.pers) continue;
+        pick = i;
+        break;
+    }
+    for (int i = 0; i < N_GEMM_INSTS && variant != -5; ++i) {
         if (variant >= 0 && variant != i) continue;
         const GemmInst &t = gemm_insts[i];
         // TM = 64 tiles are a first choice only where nothing better exists: e4m3 (no stream
@@ -1404,7 +1414,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         break;
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
-    if (variant < 0 && !gemm_insts[pick].pers) {
+    if (variant < 0 && variant != -5 && !gemm_insts[pick].pers) {
         // three or more tiles per CU: the persistent forms save the per-tile prologue and keep the
         // load stream running (8 % on (1,1536,384,2) fp16 batch-size-first at batch 25088 with the
         // tile of the pick; batch-size-last: 12 % with the first persistent tile that still

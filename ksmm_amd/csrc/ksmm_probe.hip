@@ -63,6 +63,34 @@ __global__ __launch_bounds__(512, 1) void ks_mfma_probe_kernel(float *__restrict
     out[tid] = s;
 }
 
+
+// A copy with the access pattern of a batch-size-last factor and nothing else: workgroup t moves
+// the `rows` x `tile_bytes` tile of block (a_i, d_i) and batch tile nt from x to the same place
+// in y, rows of a block being d rows apart.  Every load is issued before the first store.  What
+// this reaches is what a factor kernel with that tiling can reach at best.
+constexpr int TC_MAX_PASSES = 24;
+__global__ __launch_bounds__(256) void ks_tilecopy_probe_kernel(const uint4_t *__restrict__ x, uint4_t *__restrict__ y,
+                                                           int rows, int d, int64_t row_chunks, int tile_chunks,
+                                                           int n_tiles)
+{
+    const int tile = blockIdx.x, g = tile / n_tiles, nt = tile - g * n_tiles;
+    const int a_i = g / d, d_i = g - a_i * d;
+    const int rpp = 256 / tile_chunks;  // rows per pass
+    const int rr = threadIdx.x / tile_chunks, cc = threadIdx.x - rr * tile_chunks;
+    const int64_t chunk = (int64_t)nt * tile_chunks + cc;
+    uint4_t v[TC_MAX_PASSES];
+#pragma unroll
+    for (int i = 0; i < TC_MAX_PASSES; ++i) {
+        const int row = i * rpp + rr;
+        if (row < rows && chunk < row_chunks) v[i] = x[((int64_t)(a_i * rows + row) * d + d_i) * row_chunks + chunk];
+    }
+#pragma unroll
+    for (int i = 0; i < TC_MAX_PASSES; ++i) {
+        const int row = i * rpp + rr;
+        if (row < rows && chunk < row_chunks) y[((int64_t)(a_i * rows + row) * d + d_i) * row_chunks + chunk] = v[i];
+    }
+}
+
 }  // namespace
 
 }  // namespace ksmm
@@ -91,6 +119,28 @@ int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_byt
     *flops = per_iter * iters * 256.0 * 8.0;
     void *args[] = {&out, &iters, &random};
     return hipLaunchKernel(fn, dim3(256), dim3(512), args, 0, (hipStream_t)stream) == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+int ksmm_tilecopy_probe(const void *x, void *y, int64_t row_bytes, int a, int rows, int d, int tile_bytes, void *stream)
+{
+    using namespace ksmm;
+    if (!x || !y) return KSMM_ERR_NULL_POINTER;
+    if (((uintptr_t)x | (uintptr_t)y) & 15) return KSMM_ERR_WORKSPACE;
+    if (row_bytes < 16 || row_bytes % 16 || a < 1 || d < 1 || rows < 1) return KSMM_ERR_BAD_PATTERN;
+    // a tile row is 16..4096 bytes, a power of two (256 threads take whole rows per pass)
+    if (tile_bytes < 16 || tile_bytes > 4096 || (tile_bytes & (tile_bytes - 1))) return KSMM_ERR_BAD_PATTERN;
+    const int tile_chunks = tile_bytes / 16;
+    if (rows > TC_MAX_PASSES * (256 / tile_chunks)) return KSMM_ERR_BAD_PATTERN;
+    const int64_t row_chunks = row_bytes / 16;
+    const int64_t n_tiles = (row_chunks + tile_chunks - 1) / tile_chunks;
+    const int64_t grid = (int64_t)a * d * n_tiles;
+    if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    int n_tiles_i = (int)n_tiles, tc = tile_chunks;
+    void *args[] = {(void *)&x, (void *)&y, &rows, &d, (void *)&row_chunks, &tc, &n_tiles_i};
+    return hipLaunchKernel((const void *)ks_tilecopy_probe_kernel, dim3((unsigned)grid), dim3(256), args, 0,
+                           (hipStream_t)stream) == hipSuccess
+               ? KSMM_OK
+               : KSMM_ERR_LAUNCH;
 }
 
 }  // extern "C"

@@ -658,6 +658,8 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
         rc = gemm_run(p, -4, launch, tile);  // GEMM tiles with TM = 64
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        rc = gemm_run(p, -5, launch, tile);  // persistent GEMM tiles with a masked last TM-tile
+        if (rc != KSMM_ERR_BAD_ALGO) return rc;
     }
     int pick = -1;
     if (variant >= 0) {

@@ -280,9 +280,13 @@ def test_every_pattern_shape_class_has_a_kernel_family():
     f16, f32, f8 = torch.float16, torch.float32, torch.float8_e4m3fn
     B = 25088
     for dt in (f32, f16, f8):
-        for bs_last in (True, False):  # ragged b, d = 1: k-loop tiles with a partial last TM-tile
+        for bs_last in (True, False):  # ragged b, d = 1: tiles with a partial last TM-tile
             t = query_tile(B, (64, 460, 64, 1), dt, None, bs_last, variant=-3)
-            assert t["algo"] == 3 and t["grid"] >= 64 * 98 * 4, (dt, bs_last, t)
+            if bs_last and dt == f32:
+                # rows of whole 16-byte vectors (460 floats): the persistent GEMM tiles with a masked last TM-tile
+                assert t["algo"] == 3 and (t["variant"] >> 24) == 4 and t["grid"] == 512 and t["tile_m"] == 64, (dt, t)
+            else:  # k-loop tiles
+                assert t["algo"] == 3 and t["grid"] >= 64 * 98 * 4, (dt, bs_last, t)
         t = query_tile(B, (1, 448, 910, 32), dt, None, True, variant=-3)       # c = 910: partial K slab
         assert t["algo"] == 3 and (t["variant"] >> 24) == 4, (dt, t)
         t = query_tile(B, (1, 2, 4, 7168), dt, None, True, variant=-3)         # tiny block: vector form
