@@ -1330,11 +1330,16 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_PL(1, half_t, half_t, 64, 128, 32, 2, 2, 5, 2),
     GEMM_INST_PL(0, float, float, 64, 256, 16, 1, 4, 3, 2),
     GEMM_INST_PL(0, float, float, 64, 128, 16, 2, 2, 5, 2),
-    // the same with a partly masked last TM-tile: b = 48, 80, 96, ... (named by the table only)
+    // the same with a partly masked last TM-tile: b = 48, 80, 96, ... (variant -5 and the table)
     GEMM_INST_PLM(1, half_t, half_t, 64, 256, 32, 1, 4, 3, 2, true),
     GEMM_INST_PLM(1, half_t, half_t, 64, 128, 32, 2, 2, 5, 2, true),
     GEMM_INST_PLM(0, float, float, 64, 256, 16, 1, 4, 3, 2, true),
     GEMM_INST_PLM(0, float, float, 64, 128, 16, 2, 2, 5, 2, true),
+    // e4m3: the 4-wave tiles, whole and masked
+    GEMM_INST_PL(2, fp8_t, half_t, 64, 256, 64, 1, 4, 3, 2),
+    GEMM_INST_PL(2, fp8_t, half_t, 64, 128, 64, 2, 2, 5, 2),
+    GEMM_INST_PLM(2, fp8_t, half_t, 64, 256, 64, 1, 4, 3, 2, true),
+    GEMM_INST_PLM(2, fp8_t, half_t, 64, 128, 64, 2, 2, 5, 2, true),
 };
 constexpr int GEMM_PF = 4;             // GemmCfg::PF
 constexpr int N_GEMM_INSTS = sizeof(gemm_insts) / sizeof(GemmInst);
@@ -1397,7 +1402,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         // kernels) and partial K slabs; otherwise the stream and weight-stationary tiles come
         // first, then these (variant -4: 15-25 % faster than the k-loop tiles on 180 patterns
         // of the reference's list), then the k-loop tiles
-        if (variant < 0 && (t.pers || t.mtail)) continue;  // measured choices only (the table names them)
+        if (variant < 0 && (t.pers || t.mtail)) continue;  // taken below (persistent form of the pick) or by variant -5
         if (variant == -1 && t.tm < 128 && t.combo != 2 && !(t.ktail && p.c % t.tk)) continue;
         if (variant == -4 && t.tm >= 128) continue;  // -4: the TM = 64 tiles, after stream / weight-stationary
         // few K slabs: the 8-wave 256 x 256 tiles spend their time in prologue and epilogue; two

@@ -86,7 +86,7 @@ def test_tile_bf_groups_of_blocks_forced():
     cases = [("fp16", (1, 128, 64, 16)), ("fp16", (2, 64, 32, 8)), ("fp16", (1, 64, 64, 24)), ("fp16", (1, 128, 32, 2)),
              ("fp16", (2, 64, 32, 4)), ("fp32", (1, 128, 32, 8)), ("fp32", (2, 64, 16, 12)), ("fp32", (1, 64, 32, 4)),
              ("fp32", (1, 128, 32, 2)), ("fp8", (1, 128, 64, 16)),
-             # 5 and 12 slabs of 16: the register pipelines (2 and 3 slabs deep) end in a partial round
+             # 5, 7 and 12 slabs of 16: whole and partial rounds of the two-slab register pipeline
              ("fp16", (1, 64, 80, 8)), ("fp16", (1, 192, 192, 16)), ("fp8", (2, 64, 112, 8)),
              ("fp32", (1, 64, 80, 8)), ("fp32", (1, 192, 192, 4)), ("fp32", (2, 64, 112, 12))]
     ran, strided = 0, 0
@@ -187,8 +187,10 @@ def test_gemm_kernels_forced_e4m3():
     cases = [("fp8", True, (2, 256, 64, 3), 1008), ("fp8", True, (1, 128, 128, 2), 272),
              ("fp8", True, (2, 256, 192, 1), 528), ("fp8", True, (1, 256, 96, 2), 1024),
              ("fp8", True, (1, 128, 70, 2), 1008), ("fp8", True, (2, 256, 40, 1), 272), ("fp8", True, (1, 128, 9, 1), 64),
-             ("fp8", True, (1, 192, 128, 2), 528), ("fp8", True, (2, 64, 72, 1), 1008)]
-    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 48)], 3, 18)
+             ("fp8", True, (1, 192, 128, 2), 528), ("fp8", True, (2, 64, 72, 1), 1008),
+             # partly masked last TM-tile
+             ("fp8", True, (2, 96, 64, 3), 1008), ("fp8", True, (1, 48, 128, 4), 528)]
+    _forced_sweep(cases, [(4 << 24) | i for i in range(21, 64)], 3, 26)
 
 
 def _forced_sweep(cases, variants, algo, min_ran):
@@ -829,7 +831,8 @@ def test_persistent_gemm_batch_size_last():
             assert O.rel_fro_error(y.float().cpu().numpy()[:, cols], z) <= TOL[prec], (prec, pattern, inst)
     assert ran >= 20, ran
     # the e4m3 instances (the persistent ones are the last of the table), whole output against the oracle
-    _forced_sweep([("fp8", True, (1, 512, 128, 2), 20016)], [(4 << 24) | i for i in range(39, 48)], 3, 2)
+    _forced_sweep([("fp8", True, (1, 512, 128, 2), 20016), ("fp8", True, (2, 96, 128, 3), 20016)],
+                  [(4 << 24) | i for i in range(39, 64)], 3, 8)
     # bias + GELU (an instantiation of its own), reached through the automatic choice: three
     # tiles per CU make the heuristic take the persistent form
     import scipy.special
