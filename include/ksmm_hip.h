@@ -267,7 +267,7 @@ int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_byt
  * to the same place in y (the rows of a block are d rows apart), all loads before the first
  * store.  Timed by the caller, it gives the rate a factor kernel with that tiling can reach at
  * best, which a benchmark prints beside the rate of a linear copy.  tile_bytes: a power of two,
- * 16..4096; rows <= 24 * (4096 / tile_bytes). */
+ * 16..4096; rows <= 48 * (4096 / tile_bytes). */
 int ksmm_tilecopy_probe(const void *x, void *y, int64_t row_bytes, int a, int rows, int d, int tile_bytes, void *stream);
 
 #ifdef __cplusplus

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(512, 1) void ks_mfma_probe_kernel(float *__restrict
 // the `rows` x `tile_bytes` tile of block (a_i, d_i) and batch tile nt from x to the same place
 // in y, rows of a block being d rows apart.  Every load is issued before the first store.  What
 // this reaches is what a factor kernel with that tiling can reach at best.
-constexpr int TC_MAX_PASSES = 24;
+constexpr int TC_MAX_PASSES = 48;
 __global__ __launch_bounds__(256) void ks_tilecopy_probe_kernel(const uint4_t *__restrict__ x, uint4_t *__restrict__ y,
                                                            int rows, int d, int64_t row_chunks, int tile_chunks,
                                                            int n_tiles)
