@@ -82,6 +82,39 @@ def time_launches(fn, n_sets, steps, warmup):
     return t0.elapsed_time(t1) / 1e3 / steps
 
 
+def pattern_copy_us(p, bs_last, srcs, dsts, steps, warmup):
+    """Time of a copy that touches memory the way a factor with square blocks does and computes
+    nothing (ksmm_tilecopy_probe), best of the tile widths the probe takes; None where the
+    pattern has no such copy (b != c, input and output element sizes differ, bs_first, whose
+    rows are contiguous)."""
+    import ctypes
+
+    from ksmm_amd import _lib
+
+    a, b, c, d = p
+    es = srcs[0].element_size()
+    if b != c or dsts[0].element_size() != es or srcs[0].shape != dsts[0].shape:
+        return None
+    if bs_last:
+        cases = [(BATCH * es, a, c, d, tb) for tb in (256, 1024, 4096) if c <= 48 * (4096 // tb)]
+    else:
+        return None
+    lib = _lib.load()
+    best = None
+    for row_bytes, pa, rows, pd, tb in cases:
+        def run(j):
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            _lib.check(lib.ksmm_tilecopy_probe(srcs[j].data_ptr(), dsts[j].data_ptr(), row_bytes, pa, rows, pd, tb, stream))
+
+        run(0)
+        torch.cuda.synchronize()
+        if not torch.equal(srcs[0].view(torch.uint8), dsts[0].view(torch.uint8)):
+            raise RuntimeError("tile copy probe: output differs from input")
+        sec = time_launches(run, len(srcs), max(10, steps // 4), max(3, warmup // 4))
+        best = sec if best is None else min(best, sec)
+    return best * 1e6
+
+
 def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True):
     """Per-factor and whole-chain timings of one configuration."""
     from ksmm_amd import Kernel, generate_factor, quantize_fp8, query_tile
@@ -131,6 +164,7 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
         def run(j, cur=cur, outs=outs, sc=sc, i=i, p=p):
             Kernel.forward(cur[j], facs[i], bs_last, *p, scale=sc[j], out=outs[j])
 
+        copy_us = pattern_copy_us(p, bs_last, cur, outs, steps, warmup)
         sec = time_launches(run, n_sets, steps, warmup)
         x_dt = cur[0].dtype
         roof = factor_roofline(BATCH, p, x_dt, facs[i].dtype, out_dt, sec)
@@ -138,7 +172,9 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
         result["factors"].append({
             "pattern": p, "us": sec * 1e6, "gbs": roof["gbs"], "tflops": roof["tflops"],
             "bound": roof["bound"], "roofline_frac": roof["frac"], "floor_us": roof["floor_us"],
-            "x_dtype": str(x_dt).replace("torch.", ""), "algo": tile["algo"], "variant": tile["variant"]})
+            "x_dtype": str(x_dt).replace("torch.", ""), "algo": tile["algo"], "variant": tile["variant"],
+            # a copy with this factor's access pattern and no arithmetic (None: no such copy)
+            "pattern_copy_us": copy_us})
         cur = outs
     # ---- whole KSLinear (chain launcher) ----------------------------------------------------
     if len(patterns) > 1:
