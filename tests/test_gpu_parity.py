@@ -881,3 +881,52 @@ def test_measurement_probes():
     _lib.check(lib.ksmm_mfma_probe(dtype_code(torch.float16), 10, 1, out.data_ptr(), out.numel(), ctypes.byref(flops), stream))
     torch.cuda.synchronize()
     assert flops.value == 16 * 2.0 * 32 * 32 * 16 * 10 * 256 * 8
+
+
+def test_auto_dispatch_at_larger_batches():
+    """The automatic choice at batches where the persistent GEMM tiles, the masked last TM-tile,
+    the pipelined batch-size-first tiles and the measured table take over (the small-batch
+    tests above stay below their thresholds): sampled batch entries against the oracle, and
+    the families that are expected to run must be the ones that do."""
+    from ksmm_amd import Kernel, generate_factor
+    from ksmm_amd.kernel import query_tile
+
+    cases = [  # (prec, bs_last, pattern, batch)
+        ("fp16", True, (3, 192, 64, 4), 33000), ("fp32", True, (2, 192, 64, 3), 33000),
+        ("fp16", True, (1, 96, 384, 6), 25088), ("fp32", True, (2, 452, 64, 1), 18004),
+        ("fp8", True, (2, 192, 128, 3), 33008), ("fp8", True, (1, 96, 128, 8), 25088),
+        ("fp16", False, (1, 192, 192, 16), 9000), ("fp16", False, (2, 64, 64, 64), 9000),
+        ("fp32", False, (1, 192, 192, 8), 9000), ("fp32", False, (3, 64, 64, 16), 25088),
+        ("fp16", False, (1, 1536, 384, 2), 25088), ("fp32", True, (1, 768, 192, 2), 25088),
+        ("fp16", True, (4, 192, 192, 1), 25088), ("fp32", True, (6, 64, 64, 1), 25088),
+        ("fp16", True, (1, 512, 128, 2), 12296), ("fp32", False, (3, 64, 64, 64), 4104),
+    ]
+    seen = set()
+    for prec, bs_last, pattern, batch in cases:
+        a, b, c, d = pattern
+        dt = TORCH_DTYPE[prec]
+        t = query_tile(batch, pattern, dt, None, bs_last)
+        seen.add((t["algo"], t["variant"] >> 24 if t["algo"] == 3 else -1, t["grid"] in (256, 512)))
+        print("auto", prec, bs_last, pattern, batch, t["algo"], hex(t["variant"]), t["grid"], flush=True)
+        (w4,) = seeded_weights([pattern], seed=201)
+        x = seeded_input(a * c * d, batch, bs_last, seed=202)
+        wr, wq, ws = round_to(w4, prec)
+        xr, xq, xs = round_to(x, prec)
+        if prec == "fp8":
+            fac = generate_factor(a, b, c, d, "kernel", wq.to(torch.float32), dt, "cuda")
+            xin, scale = xq.cuda(), ws * xs
+        else:
+            fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+            xin, scale = x.to(dt).cuda(), 1.0
+        y = Kernel.forward(xin, fac, bs_last, a, b, c, d, dtype=dt, scale=scale)
+        torch.cuda.synchronize()
+        assert torch.isfinite(y).all(), (prec, bs_last, pattern, batch)
+        idx = sample_columns(batch, step=211)
+        xs_ = xr[:, idx] if bs_last else xr[idx]
+        z = O.ks_apply_einsum(wr, xs_, bs_last)
+        got = y.float().cpu().numpy()
+        got = got[:, idx] if bs_last else got[idx]
+        err = O.rel_fro_error(got, z)
+        assert err <= TOL[prec], (prec, bs_last, pattern, batch, t, err)
+    # persistent GEMM tiles (one or two workgroups per CU) and the batch-size-first tile kernels ran
+    assert (3, 4, True) in seen and any(s[0] == 3 and s[1] == 3 for s in seen), seen
