@@ -26,29 +26,39 @@ namespace ksmm {
 
 namespace {
 
-template <int BB, int CC, int DD, int TN> struct RowCfg {
+// PL: the LDS tiles are split into one plane per d_i ([d_i][row][k], rows padded by 4, planes
+// padded to 4 floats past a multiple of 64).  With d_i fastest all 64 lanes of an operand read
+// or result write hit the same 4-byte slot of the 16-byte groups (16 banks at most: 4-way
+// conflicts whatever the padding); in planes those accesses are conflict-free, and so are
+// the four 4-byte stores / loads per 16-byte global vector that feed and drain them.
+constexpr int plane_floats(int n) { return n + (68 - n % 64) % 64; }
+template <int BB, int CC, int DD, int TN, bool PL = false> struct RowCfg {
     static constexpr int NW = DD, THREADS = 64 * NW;
     static constexpr int MT = BB / 16, KS = CC / 4, NT = TN / 16;
     static constexpr int XROW = CC * DD, OROW = BB * DD;  // floats per row segment
     static constexpr int LDX = XROW + 4, LDO = OROW + 4;
+    static constexpr int LDK = CC + 4, LDM = BB + 4;      // PL: rows of a plane
+    static constexpr int PLANE_X = plane_floats(TN * LDK), PLANE_O = plane_floats(TN * LDM);
+    static constexpr int X_FLOATS = PL ? DD * PLANE_X : TN * LDX, O_FLOATS = PL ? DD * PLANE_O : TN * LDO;
     static constexpr int X_VECS = TN * XROW / 4, O_VECS = TN * OROW / 4;
     static constexpr int X_PER_T = (X_VECS + THREADS - 1) / THREADS, O_PER_T = (O_VECS + THREADS - 1) / THREADS;
-    static constexpr int LDS_BYTES = (2 * TN * LDX + TN * LDO) * 4;
+    static constexpr int LDS_BYTES = (2 * X_FLOATS + O_FLOATS) * 4;
+    static_assert(!PL || DD % 4 == 0, "planes: a 16-byte vector is 4 d_i of one k");
     static_assert(BB % 16 == 0 && CC % 4 == 0 && TN % 16 == 0, "MFMA tiling");
     static_assert(NW <= 16 && XROW % 4 == 0 && OROW % 4 == 0, "shape");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-template <int BB, int CC, int DD, int TN, bool NT_STORE>
+template <int BB, int CC, int DD, int TN, bool NT_STORE, bool PL = false>
 __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a,
                                                             int d, Epi ep, int wgs_per_a, int n_tiles)
 {
-    typedef RowCfg<BB, CC, DD, TN> C;
+    typedef RowCfg<BB, CC, DD, TN, PL> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    float *const xs = (float *)smem;                // [2][TN][LDX]
-    float *const os = xs + 2 * TN * C::LDX;         // [TN][LDO]
+    float *const xs = (float *)smem;                // [2][TN][LDX]; PL: [2][DD][PLANE_X]
+    float *const os = xs + 2 * C::X_FLOATS;         // [TN][LDO]; PL: [DD][PLANE_O]
     // blockIdx -> (a_i, group of DD d_i, share of the tiles)
     const int groups = d / DD;
     const int ag = blockIdx.x / wgs_per_a;
@@ -98,7 +108,13 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
             const int v = tid + i * C::THREADS;
             if (C::X_VECS % C::THREADS == 0 || v < C::X_VECS) {
                 const int nn = v / (C::XROW / 4), e0 = (v % (C::XROW / 4)) * 4;
-                *(float4_t *)(xs + (buf * TN + nn) * C::LDX + e0) = xreg[decltype(P)::value][i];
+                if constexpr (PL) {
+                    float *dst = xs + buf * C::X_FLOATS + (e0 % DD) * C::PLANE_X + nn * C::LDK + e0 / DD;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) dst[j * C::PLANE_X] = xreg[decltype(P)::value][i][j];
+                } else {
+                    *(float4_t *)(xs + (buf * TN + nn) * C::LDX + e0) = xreg[decltype(P)::value][i];
+                }
             }
         }
     };
@@ -108,7 +124,7 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
     auto do_tile = [&](int t, int buf, auto P) {
         typedef std::integral_constant<int, 1 - decltype(P)::value> Q;
         if (t + 2 * t_step < t_end) gload(t + 2 * t_step, P);
-        const float *xb = xs + buf * TN * C::LDX;
+        const float *xb = xs + buf * C::X_FLOATS;
         float4_t acc[C::MT][C::NT];
 #pragma unroll
         for (int mt = 0; mt < C::MT; ++mt)
@@ -119,7 +135,9 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < C::NT; ++nt) xf[ks][nt] = xb[(16 * nt + r) * C::LDX + (4 * ks + q) * DD + dd];
+            for (int nt = 0; nt < C::NT; ++nt)
+                xf[ks][nt] = PL ? xb[dd * C::PLANE_X + (16 * nt + r) * C::LDK + 4 * ks + q]
+                                : xb[(16 * nt + r) * C::LDX + (4 * ks + q) * DD + dd];
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
@@ -134,7 +152,8 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
+                    os[PL ? dd * C::PLANE_O + (16 * nt + r) * C::LDM + 16 * mt + 4 * q + i
+                          : (16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -143,7 +162,14 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
                 const int nn = v / (C::OROW / 4), e0 = (v % (C::OROW / 4)) * 4;
                 const int row = t * TN + nn;
                 if (row < batch) {
-                    const float4_t o = *(const float4_t *)(os + nn * C::LDO + e0);
+                    float4_t o;
+                    if constexpr (PL) {
+                        const float *src = os + (e0 % DD) * C::PLANE_O + nn * C::LDM + e0 / DD;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) o[j] = src[j * C::PLANE_O];
+                    } else {
+                        o = *(const float4_t *)(os + nn * C::LDO + e0);
+                    }
                     if (NT_STORE)
                         __builtin_nontemporal_store(o, (float4_t *)(yg + (size_t)row * out_size + row_off(e0)));
                     else
@@ -316,7 +342,10 @@ struct RowInst {
     int vec;  // elements per 16-byte vector of the input
     int nt;   // streaming (nontemporal) output stores
     const void *fn;
+    int planes;  // fp32: LDS tiles split into one plane per d_i
 };
+#define ROW_INST_PL(BB_, CC_, DD_, TN_) \
+    {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_, true>::LDS_BYTES, 4, 1, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, true, true>, 1}
 #define ROW_INST(BB_, CC_, DD_, TN_, NT_) \
     {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, 4, NT_, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
 #define ROW_INST_H(BB_, CC_, DD_, TN_)                                                                      \
@@ -362,6 +391,11 @@ const RowInst row_insts[] = {
     // the same for fp16 and e4m3
     ROW_SET_16B(ROW_INST_H),
     ROW_SET_16B(ROW_INST_Q),
+    // fp32 with one LDS plane per d_i (groups of 4, 8, 16)
+    ROW_INST_PL(48, 48, 16, 16), ROW_INST_PL(48, 48, 8, 32), ROW_INST_PL(48, 48, 8, 16), ROW_INST_PL(48, 48, 4, 64),
+    ROW_INST_PL(48, 48, 4, 16), ROW_INST_PL(64, 64, 8, 16), ROW_INST_PL(64, 64, 4, 32), ROW_INST_PL(64, 64, 4, 16),
+    ROW_INST_PL(16, 16, 16, 32), ROW_INST_PL(16, 16, 4, 128), ROW_INST_PL(32, 32, 8, 32), ROW_INST_PL(32, 32, 16, 16),
+    ROW_INST_PL(96, 96, 4, 16), ROW_INST_PL(48, 192, 4, 16), ROW_INST_PL(192, 48, 4, 16),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 constexpr int ROW_INST_BITS = 10, ROW_INST_ANY = (1 << ROW_INST_BITS) - 1;
@@ -375,8 +409,8 @@ uint32_t rows_inst_id(int i)
 {
     if (i < 0 || i >= N_ROW_INSTS) return 0;
     const RowInst &t = row_insts[i];
-    const int v[6] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt};
-    return inst_hash('R', v, 6);
+    const int v[7] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt, t.planes};
+    return inst_hash('R', v, t.planes ? 7 : 6);  // (ids of the other instances predate the field)
 }
 
 // variant: bits 0-9 instance (all ones: first that fits), bits 10.. workgroups per a_i (0: heuristic)
@@ -392,6 +426,7 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         if (want != ROW_INST_ANY && want != i) continue;
         const RowInst &t = row_insts[i];
         if (t.combo != combo || t.bb != p.b || t.cc != p.c) continue;
+        if (want == ROW_INST_ANY && t.planes) continue;  // named by the table (or forced) only
         // row segments start on 16-byte boundaries (output vectors: 4 floats / 8 halves)
         const int ovec = combo == 0 ? 4 : 8;
         if (((int64_t)p.a * p.c * p.d) % t.vec || ((int64_t)p.a * p.b * p.d) % ovec) continue;

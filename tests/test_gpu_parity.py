@@ -255,7 +255,8 @@ def test_row_kernel_instances_forced():
               # d a multiple of the group: several workgroups per a_i, runs of DD floats
               (1, 48, 48, 32), (2, 48, 48, 24), (1, 64, 64, 16), (1, 16, 16, 64), (2, 96, 96, 8), (1, 192, 48, 16)]
     cases = [("fp32", False, p, batch) for p in shapes for batch in (512, 203)]
-    _forced_sweep(cases, [1000 + i for i in list(range(32)) + list(range(97, 110))], 2, 80)
+    # (143..157: the instances whose LDS tiles are split into one plane per d_i)
+    _forced_sweep(cases, [1000 + i for i in list(range(32)) + list(range(97, 110)) + list(range(143, 160))], 2, 120)
     # fp16: the same design with 16-byte vectors of 8 halves (batch a multiple of nothing special)
     shapes16 = [(2, 48, 48, 16), (1, 48, 48, 8), (2, 48, 48, 4), (1, 48, 48, 12), (1, 48, 48, 6), (2, 48, 48, 2),
                 (1, 64, 64, 16), (1, 64, 64, 8), (2, 64, 64, 3), (1, 96, 96, 8), (1, 96, 96, 3), (1, 48, 192, 8),
