@@ -18,6 +18,7 @@
 // (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-286,
 //  template_kernels_half.cuh:103-299), which gather the strided inputs with scalar loads.
 #include "ksmm_mfma.h"
+#include <type_traits>
 
 namespace ksmm {
 
@@ -212,8 +213,8 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
 //  * the planes are unpadded rows of 16 k, their two 16-byte halves swapped for rows 8..15 of
 //    every 16 (the 16 rows a 16-byte operand read covers then fall on distinct banks);
 // which brings LDS to 72 KB: two workgroups per CU, four slabs of 32 KB in flight.
-template <typename TW, int TM, int TN, int WM, int WN, int PDX, int PDW>
-__global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_bf8_kernel(const half_t *__restrict__ x,
+template <typename TX, typename TW, int TM, int TN, int WM, int WN, int PDX, int PDW>
+__global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_bf8_kernel(const TX *__restrict__ x,
                                                                 const TW *__restrict__ w,
                                                                 half_t *__restrict__ y, int batch, int a,
                                                                 int b, int c, int d, Epi ep,
@@ -248,10 +249,11 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
-    const half_t *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
 
     stage<TW, half_t> wreg[PDW][W_PER_T];
-    uint4_t xreg[PDX][XQ_PER_T][2];
+    // one (row, k) of the group: 8 halves = 16 bytes, or 8 e4m3 bytes (decoded when they go to LDS)
+    typedef typename std::conditional<sizeof(TX) == 2, uint4_t, uint2_t>::type xvec_t;
+    xvec_t xreg[PDX][XQ_PER_T][2];
     // The loads of a slab are issued unconditionally: a branch around them would leave the
     // compiler two histories of the load counter to merge, and it would then wait for every
     // load in flight before it touches a register of the pipeline.  Behind the last slab
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     // offsets are masked, not selected, so that no branch comes back.  Addresses are a uniform
     // base per tile plus a 32-bit offset per lane (the host checks that they fit).
     const TW *const wt = w + ((size_t)(a_i * d + dg * DD) * c) * b + m0;
-    const half_t *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DD;
+    const TX *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DD;
     uint32_t woff[W_PER_T], xoff[XQ_PER_T];
 #pragma unroll
     for (int i = 0; i < W_PER_T; ++i) {
@@ -291,7 +293,7 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
         for (int i = 0; i < XQ_PER_T; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                xreg[slot][i][j] = *(const uint4_t *)(xt + ((xoff[i] + (uint32_t)((k0 + 8 * j) * d)) & mk));
+                xreg[slot][i][j] = *(const xvec_t *)(xt + ((xoff[i] + (uint32_t)((k0 + 8 * j) * d)) & mk));
     };
     auto lstore = [&](int wslot, int slot, int buf) {
 #pragma unroll
@@ -309,7 +311,19 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
             // k = k8 and k8 + 8 of row nn: positions 2 * k8 and 2 * k8 + 1, i.e. 4-byte piece k8 & 3
             // of the 16-byte half k8 >> 2 (swapped for rows 8..15 of every 16)
             half_t *const dst = xs(buf, 0) + nn * TK + ((((k8 >> 2) ^ ((nn >> 3) & 1)) << 3) | ((k8 & 3) << 1));
-            const uint4_t c0 = xreg[slot][i][0], c1 = xreg[slot][i][1];
+            uint4_t c0, c1;  // register p: d_i = 2p (low half) and 2p + 1 (high half), as fp16
+            if constexpr (sizeof(TX) == 2) {
+                c0 = xreg[slot][i][0];
+                c1 = xreg[slot][i][1];
+            } else {
+#pragma unroll
+                for (int w2 = 0; w2 < 2; ++w2) {
+                    c0[2 * w2] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(xreg[slot][i][0][w2]));
+                    c0[2 * w2 + 1] = __builtin_bit_cast(uint32_t, fp8x2_hi_to_half2(xreg[slot][i][0][w2]));
+                    c1[2 * w2] = __builtin_bit_cast(uint32_t, fp8x2_to_half2(xreg[slot][i][1][w2]));
+                    c1[2 * w2 + 1] = __builtin_bit_cast(uint32_t, fp8x2_hi_to_half2(xreg[slot][i][1][w2]));
+                }
+            }
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 // register p of a vector holds d_i = 2p (low half) and 2p + 1 (high half)
@@ -648,15 +662,15 @@ struct BfInst {
 #define BF_SET_H8(COMBO_, TW_)                                                                   \
     BF_INST(COMBO_, half_t, TW_, 8, 64, 64, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 8, 64, 64, 16, 2, 2), \
         BF_INST(COMBO_, half_t, TW_, 8, 32, 128, 16, 1, 4), BF_INST(COMBO_, half_t, TW_, 8, 128, 64, 16, 4, 2)
-#define BF8_INST(COMBO_, TW_, TM_, TN_, WM_, WN_, PDX_, PDW_)                                    \
+#define BF8_INST(COMBO_, TX_, TW_, TM_, TN_, WM_, WN_, PDX_, PDW_)                                    \
     {COMBO_, 8, TM_, TN_, 16, 64 * WM_ * WN_,                                                    \
      2 * 2 * (8 * 16 * pads<half_t>::outer(TM_) + 8 * TN_ * 16), WM_,                            \
-     (const void *)ks_tile_bf8_kernel<TW_, TM_, TN_, WM_, WN_, PDX_, PDW_>, PDX_ * 16 + PDW_}
+     (const void *)ks_tile_bf8_kernel<TX_, TW_, TM_, TN_, WM_, WN_, PDX_, PDW_>, PDX_ * 16 + PDW_}
 #define BF4_INST(TM_, TN_, WM_, WN_, PDX_, PDW_)                                                 \
     {0, 4, TM_, TN_, 16, 64 * WM_ * WN_, 2 * 4 * (4 * 16 * TM_ + 4 * TN_ * 16), WM_,                 \
      (const void *)ks_tile_bf4_kernel<TM_, TN_, WM_, WN_, PDX_, PDW_>, PDX_ * 16 + PDW_}
-#define BF8_SET(COMBO_, TW_)                                                                     \
-    BF8_INST(COMBO_, TW_, 64, 64, 2, 2, 2, 2), BF8_INST(COMBO_, TW_, 64, 128, 2, 4, 2, 2)
+#define BF8_SET(COMBO_, TX_, TW_)                                                                \
+    BF8_INST(COMBO_, TX_, TW_, 64, 64, 2, 2, 2, 2), BF8_INST(COMBO_, TX_, TW_, 64, 128, 2, 4, 2, 2)
 const BfInst bf_insts[] = {
     BF_SET_H(1, half_t),
     BF_SET_H(3, fp8_t),
@@ -669,11 +683,13 @@ const BfInst bf_insts[] = {
     BF_SET_H8(1, half_t),
     BF_SET_H8(3, fp8_t),
     // the same groups with a register pipeline (ks_tile_bf8_kernel)
-    BF8_SET(1, half_t),
-    BF8_SET(3, fp8_t),
+    BF8_SET(1, half_t, half_t),
+    BF8_SET(3, half_t, fp8_t),
     // fp32 groups of 4 (ks_tile_bf4_kernel)
     BF4_INST(64, 64, 2, 2, 2, 2),
     BF4_INST(64, 128, 2, 4, 2, 2),
+    // e4m3 input and weights: groups of 8 again (8-byte vectors, decoded on their way to LDS)
+    BF8_SET(2, fp8_t, fp8_t),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
@@ -683,10 +699,12 @@ bool bf_fits(const BfInst &t, const Problem &p, int combo)
     if (p.b % t.tm || p.c % t.tk) return false;
     const int x_epv = 16 / (int)dtype_size(p.x_dtype), w_epv = 16 / (int)dtype_size(p.w_dtype);
     // d > DD: the DD elements of one (row, k) must fill the 16-byte vector
-    if (p.d != t.dd && t.dd != x_epv) return false;
+    // (the pipelined e4m3 instances read 8-byte vectors: groups of 8 out of any multiple of 8)
+    const int vec = (t.pd && combo == 2) ? 8 : x_epv;
+    if (p.d != t.dd && t.dd != vec) return false;
     if (p.b % w_epv) return false;
     // rows of x start at multiples of in_size, slabs at multiples of TK * d: keep 16-byte alignment
-    if (((int64_t)p.a * p.c * p.d) % x_epv || ((int64_t)p.c * p.d) % x_epv) return false;
+    if (((int64_t)p.a * p.c * p.d) % vec || ((int64_t)p.c * p.d) % vec) return false;
     if (t.pd) {
         // 32-bit element offsets inside a tile: TN rows of x, DD blocks of w
         if ((int64_t)t.tn * p.a * p.c * p.d + (int64_t)p.c * p.d >= 0xffffffffLL) return false;

@@ -121,6 +121,10 @@ def test_tile_bf_groups_of_blocks_forced():
             err = O.rel_fro_error(y.float().cpu().numpy(), zb)
             assert err <= TOL[prec], (prec, pattern, batch, "bias", err)
     print("tile_bf forced: ran", ran, "of which d > DD", strided, flush=True)
+    # e4m3 input and weights (8-byte vectors of a group, decoded on their way to LDS)
+    _forced_sweep([("fp8", False, (1, 128, 64, 16), 520), ("fp8", False, (2, 64, 80, 8), 77),
+                   ("fp8", False, (1, 192, 192, 8), 1000), ("fp8", False, (1, 64, 32, 24), 203)],
+                  [(3 << 24) | i for i in range(27, 40)], 3, 8)
     assert ran >= 30 and strided >= 12, (ran, strided)
 
 
