@@ -593,8 +593,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 //    stages already hold the next tile's slabs): every wave turns its 32x32 blocks around in a
 //    private piece of it and stores whole 128-byte lines, without a workgroup barrier.
 // All waves multiply and store their own part of the output.
-template <typename CT, typename TY, int DD, int TM, int TN, int TK, int WM, int WN, int ST, bool EPI>
-__global__ __launch_bounds__(64 * WM * WN, 1) void ks_gemm_pbf_kernel(const CT *__restrict__ x,
+template <typename CT, typename TY, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool EPI>
+__global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT *__restrict__ x,
                                                                 const CT *__restrict__ w,
                                                                 TY *__restrict__ y, int batch, int a,
                                                                 int b, int c, int d, Epi ep,
@@ -1248,10 +1248,11 @@ struct GemmInst {
      GemmCfg<CT_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::EPC,                                       \
      KT_, WM_, 0, {(const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_, false>, \
                    (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_, true>}}
-#define GEMM_INST_P(DD_, TM_, TN_, TK_, WM_, WN_, ST_)                                                \
+#define GEMM_INST_PO(DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                                          \
     {1, false, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
-     8, 0, WM_, 1, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, false>, \
-                    (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, true>}}
+     8, 0, WM_, OCC_, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false>, \
+                       (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, true>}}
+#define GEMM_INST_P(DD_, TM_, TN_, TK_, WM_, WN_, ST_) GEMM_INST_PO(DD_, TM_, TN_, TK_, WM_, WN_, ST_, 1)
 // OCC_: persistent workgroups per CU (4-wave tiles: two); MT_: partial last TM-tile
 #define GEMM_INST_PLM(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, MT_)                      \
     {COMBO_, true, 1, TM_, TN_, TK_, 64 * WM_ * WN_,                                                  \
@@ -1335,6 +1336,8 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_PLM(1, half_t, half_t, 64, 128, 32, 2, 2, 5, 2, true),
     GEMM_INST_PLM(0, float, float, 64, 256, 16, 1, 4, 3, 2, true),
     GEMM_INST_PLM(0, float, float, 64, 128, 16, 2, 2, 5, 2, true),
+    // fp16 bs_first d == 2: 4-wave tile, two persistent workgroups per CU (b = 64, 192, ...)
+    GEMM_INST_PO(2, 64, 128, 32, 1, 4, 3, 2),
     // e4m3: the 4-wave tiles, whole and masked
     GEMM_INST_PL(2, fp8_t, half_t, 64, 256, 64, 1, 4, 3, 2),
     GEMM_INST_PL(2, fp8_t, half_t, 64, 128, 64, 2, 2, 5, 2),
@@ -1382,11 +1385,23 @@ uint32_t gemm_inst_id(int i)
 // the chip (TM = 64 tiles only where nothing better exists); -4: the TM = 64 tiles, same
 // condition; -5: the persistent tiles with a masked last TM-tile, for b beyond one tile and
 // three tiles per persistent workgroup (they beat the k-loop tiles on 72 of 80 such patterns of
-// the reference's list, up to 2x); -2: first that fits
+// the reference's list, up to 2x); -6: the 4-wave persistent batch-size-first tile; -2: first
+// that fits
 int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
 {
     const int combo = combo_of(p.x_dtype, p.w_dtype, p.y_dtype);
     int pick = -1;
+    for (int i = 0; i < N_GEMM_INSTS && variant == -6; ++i) {
+        // -6: the 4-wave persistent batch-size-first tile (d == 2, b a multiple of 64) from half a
+        // chip of tiles: 1.1-2.5x faster than the tile_bf and 64 x 256 GEMM tiles it
+        // replaces ((1,192,192,2) 18.1 -> 12.5 us, (1,64,256,2) 21.5 -> 8.5, (2,320,64,2) 31.9 -> 17.2)
+        const GemmInst &t = gemm_insts[i];
+        if (!t.pers || t.bs_last || t.tm != 64 || !gemm_fits(t, p, combo)) continue;
+        const int64_t tiles = (int64_t)p.a * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
+        if (tiles < 128) continue;  // (measured down to 196 tiles: still 2.5x)
+        pick = i;
+        break;
+    }
     for (int i = 0; i < N_GEMM_INSTS && variant == -5; ++i) {
         const GemmInst &t = gemm_insts[i];
         if (!t.mtail || p.b <= t.tm || !gemm_fits(t, p, combo)) continue;
@@ -1395,7 +1410,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         pick = i;
         break;
     }
-    for (int i = 0; i < N_GEMM_INSTS && variant != -5; ++i) {
+    for (int i = 0; i < N_GEMM_INSTS && variant != -5 && variant != -6; ++i) {
         if (variant >= 0 && variant != i) continue;
         const GemmInst &t = gemm_insts[i];
         // TM = 64 tiles are a first choice only where nothing better exists: e4m3 (no stream
@@ -1419,7 +1434,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         break;
     }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
-    if (variant < 0 && variant != -5 && !gemm_insts[pick].pers) {
+    if (variant < 0 && variant > -5 && !gemm_insts[pick].pers) {
         // three or more tiles per CU: the persistent forms save the per-tile prologue and keep the
         // load stream running (8 % on (1,1536,384,2) fp16 batch-size-first at batch 25088 with the
         // tile of the pick; batch-size-last: 12 % with the first persistent tile that still
@@ -1428,7 +1443,7 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         for (int i = 0; i < N_GEMM_INSTS; ++i) {
             const GemmInst &q = gemm_insts[i];
             if (!q.pers || q.mtail || q.combo != o.combo || q.bs_last != o.bs_last || q.dd != o.dd) continue;
-            if (!q.bs_last && (q.tm != o.tm || q.tn != o.tn || q.tk != o.tk)) continue;
+            if (!q.bs_last && (q.tm != o.tm || q.tk != o.tk || (q.tn != o.tn && q.tm > 64))) continue;
             if (!gemm_fits(q, p, combo)) continue;
             const int64_t groups = q.dd == 1 ? (int64_t)p.a * p.d : p.a;
             if (groups * (p.b / q.tm) * ((p.batch + q.tn - 1) / q.tn) < 3 * 256 * q.pers) continue;

@@ -651,6 +651,10 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     } else {
         int rc = gemm_run(p, -1, launch, tile);  // large blocks: matrix-core-bound
         if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        if (!p.bs_last && p.d == 2) {
+            rc = gemm_run(p, -6, launch, tile);  // 4-wave persistent GEMM tile, two workgroups per CU
+            if (rc != KSMM_ERR_BAD_ALGO) return rc;
+        }
         if (!p.bs_last && p.d > 1) return tile_bf_run(p, -1, launch, tile);
         rc = stream_run(p, -1, launch, tile);
         if (rc != KSMM_ERR_BAD_ALGO) return rc;

@@ -758,11 +758,11 @@ def test_persistent_gemm_walks_several_tiles_per_workgroup():
         rows = sample_columns(batch, step=389)
         z = O.ks_apply_einsum(round_to(w4, "fp16")[0], round_to(x, "fp16")[0][rows], False)
         assert O.rel_fro_error(ref.float().cpu().numpy()[rows], z) <= TOL["fp16"]
-        for inst in range(32, 48):
+        for inst in range(32, 64):
             try:
                 variant_id(3, (4 << 24) | inst, 1, False)
             except _lib.KsmmError:
-                break
+                continue
             try:
                 y = Kernel.forward(xin, fac, False, a, b, c, d, algo=3, variant=(4 << 24) | inst)
             except _lib.KsmmError as e:
@@ -773,7 +773,7 @@ def test_persistent_gemm_walks_several_tiles_per_workgroup():
             assert torch.isfinite(y).all(), (pattern, inst)
             err = ((y.float() - ref.float()).norm() / ref.float().norm()).item()
             assert err <= 1e-6, (pattern, inst, err)
-    assert ran >= 5, ran
+    assert ran >= 7, ran
     # bias + GELU on the persistent kernel (its epilogue is an instantiation of its own): forced
     # instances take no epilogue, so a problem with three tiles per CU, where the heuristic picks
     # the persistent form by itself
