@@ -734,8 +734,9 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
     struct XPairs {
         uint4_t lo, hi;
     };
+    typedef typename std::conditional<DD == 2, XPairs, frag_t>::type xraw_t;  // d == 1: the operand itself
     auto read_frags = [&](const uint32_t(&wa)[C::MT], const uint32_t(&xa)[C::NT], int k0, frag_t(&fw)[DD][C::MT],
-                          XPairs(&xr)[C::NT]) {
+                          xraw_t(&xr)[C::NT]) {
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
@@ -743,15 +744,23 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
                 fw[dd][i] = outer_frag<CT, TM>::read(wa[i] + dd * (TK * TM * C::ES), k0);
 #pragma unroll
         for (int j = 0; j < C::NT; ++j) {
-            typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
-            const uint32_t pa = xa[j] ^ ((k0 >> 2) << 4);
-            xr[j].lo = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa);
-            xr[j].hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ 16);
+            if constexpr (DD == 2) {
+                typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
+                const uint32_t pa = xa[j] ^ ((k0 >> 2) << 4);
+                xr[j].lo = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa);
+                xr[j].hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ 16);
+            } else {
+                typedef __attribute__((address_space(3))) half8_t *lds_ptr;
+                xr[j] = *(lds_ptr)(lds_bytes_t)(uintptr_t)(xa[j] ^ ((k0 >> 3) << 4));
+            }
         }
     };
-    auto split_x = [&](const XPairs(&xr)[C::NT], frag_t(&fx)[DD][C::NT]) {
+    auto split_x = [&](const xraw_t(&xr)[C::NT], frag_t(&fx)[DD][C::NT]) {
 #pragma unroll
         for (int j = 0; j < C::NT; ++j) {
+            if constexpr (DD == 1) {
+                fx[0][j] = xr[j];
+            } else {
             const uint4_t lo = xr[j].lo, hi = xr[j].hi;
             uint4_t e, o;
             e[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100u);
@@ -763,7 +772,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
             o[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07060302u);
             o[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07060302u);
             fx[0][j] = __builtin_bit_cast(half8_t, e);
-            fx[1][j] = __builtin_bit_cast(half8_t, o);
+            fx[DD - 1][j] = __builtin_bit_cast(half8_t, o);
+            }
         }
     };
     constexpr int K0 = TK / C::KSTEP;           // MFMA sub-steps per slab
@@ -772,7 +782,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
     constexpr int SLOTS = (K0 - 1) * PER_K0;
     constexpr int STRIDE = SLOTS / L > 0 ? SLOTS / L : 1;  // MFMAs per load issued (loader waves)
     frag_t fw[2][DD][C::MT], fx[DD][C::NT];
-    XPairs xr[2][C::NT];
+    xraw_t xr[2][C::NT];
     uint32_t wa[C::MT], xa[C::NT];
     auto stage_addrs = [&](int stg) {
         const uint32_t base = lds_base + stg * C::STAGE_BYTES;
@@ -794,9 +804,12 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
 
     const int l32 = lane & 31, lq = lane >> 5;
     constexpr int OP = 128 + 16;  // bytes per row of a wave's output piece
-    static_assert(DD == 2 && NWAVES * 32 * OP <= C::STAGE_BYTES, "output pieces fit the consumed stage");
+    static_assert(NWAVES * 32 * OP <= C::STAGE_BYTES, "output pieces fit the consumed stage");
+    // d == 1: a block row is 32 outputs = 64 bytes, so two neighbouring TM-blocks share a line
+    constexpr int IP = DD == 2 ? 1 : 2;
+    static_assert(C::MT % IP == 0, "TM-blocks pair up into whole lines");
 
-    constexpr int TILE_STORES = C::MT * C::NT * 4;  // stores of a wave per full tile
+    constexpr int TILE_STORES = (C::MT / IP) * C::NT * 4;  // stores of a wave per full tile
     static_assert(N_WAIT + TILE_STORES <= 63, "counter range");
     bool stores_behind = false;  // the previous tile issued exactly TILE_STORES stores (uniform)
     Tile cur = decode(0);
@@ -869,16 +882,17 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
                 const size_t f0 = ((size_t)cur.a_i * b + cur.m0 + (wm * C::MT + i) * 32 + 4 * lq) * DD;
 #pragma unroll
                 for (int eg = 0; eg < 4; ++eg) {
-                    // the lane's 8 bias values of this group: (4 outputs) x (2 d_i), one 16-byte load
-                    half8_t bb = {0, 0, 0, 0, 0, 0, 0, 0};
-                    if (ep.bias) bb = *(const half8_t *)((const TY *)ep.bias + f0 + 16 * eg);
+                    // the lane's bias values of this group: (4 outputs) x (DD d_i), one vector load
+                    typedef TY bias_v __attribute__((ext_vector_type(4 * DD)));
+                    bias_v bb = {};
+                    if (ep.bias) bb = *(const bias_v *)((const TY *)ep.bias + f0 + 8 * DD * eg);
 #pragma unroll
                     for (int j = 0; j < C::NT; ++j)
 #pragma unroll
                         for (int u = 0; u < 4; ++u)
 #pragma unroll
                             for (int dd = 0; dd < DD; ++dd) {
-                                const float v = fmaf(acc[dd][i][j][4 * eg + u], scale, (float)bb[2 * u + dd]);
+                                const float v = fmaf(acc[dd][i][j][4 * eg + u], scale, (float)bb[DD * u + dd]);
                                 acc[dd][i][j][4 * eg + u] = ep.act == KSMM_ACT_GELU ? gelu_erf(v) : v;
                             }
                 }
@@ -887,22 +901,33 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
         const float st_scale = has_epi ? 1.f : scale;
         {
             unsigned char *const piece = smem + stg * C::STAGE_BYTES + wave * (32 * OP);
-            unsigned char *const wr = piece + l32 * OP + 16 * lq;           // + 32 * eg
+            unsigned char *const wr = piece + l32 * OP + (8 * DD) * lq;     // + 16 * DD * eg (+ 64 * second block)
             const unsigned char *const rd = piece + (lane >> 3) * OP + 16 * (lane & 7);  // + 8 * t rows
 #pragma unroll
-            for (int i = 0; i < C::MT; ++i)
+            for (int ip = 0; ip < C::MT / IP; ++ip)
 #pragma unroll
                 for (int j = 0; j < C::NT; ++j) {
+                    const int i = ip * IP;
                     const int mb = (wm * C::MT + i) * 32, nb = (wn * C::NT + j) * 32;
 #pragma unroll
                     for (int eg = 0; eg < 4; ++eg) {
-                        half8_t v;
+                        if constexpr (DD == 2) {
+                            half8_t v;
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            v[2 * u] = (half_t)(acc[0][i][j][4 * eg + u] * st_scale);
-                            v[2 * u + 1] = (half_t)(acc[1][i][j][4 * eg + u] * st_scale);
+                            for (int u = 0; u < 4; ++u) {
+                                v[2 * u] = (half_t)(acc[0][i][j][4 * eg + u] * st_scale);
+                                v[2 * u + 1] = (half_t)(acc[DD - 1][i][j][4 * eg + u] * st_scale);
+                            }
+                            *(half8_t *)(wr + 32 * eg) = v;
+                        } else {
+#pragma unroll
+                            for (int ii = 0; ii < IP; ++ii) {
+                                const float16_t &ac = acc[0][i + ii][j];
+                                const half4_t v = {(half_t)(ac[4 * eg] * st_scale), (half_t)(ac[4 * eg + 1] * st_scale),
+                                                   (half_t)(ac[4 * eg + 2] * st_scale), (half_t)(ac[4 * eg + 3] * st_scale)};
+                                *(half4_t *)(wr + 64 * ii + 16 * eg) = v;
+                            }
                         }
-                        *(half8_t *)(wr + 32 * eg) = v;
                     }
                     __builtin_amdgcn_wave_barrier();
                     const int n = cur.n0 + nb + (lane >> 3);  // + 8 * t
@@ -1338,6 +1363,9 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_PLM(0, float, float, 64, 128, 16, 2, 2, 5, 2, true),
     // fp16 bs_first d == 2: 4-wave tile, two persistent workgroups per CU (b = 64, 192, ...)
     GEMM_INST_PO(2, 64, 128, 32, 1, 4, 3, 2),
+    // fp16 bs_first d == 1: 4-wave tiles of 64 and 128 rows
+    GEMM_INST_PO(1, 64, 256, 32, 1, 4, 3, 2),
+    GEMM_INST_PO(1, 128, 256, 32, 2, 2, 3, 2),
     // e4m3: the 4-wave tiles, whole and masked
     GEMM_INST_PL(2, fp8_t, half_t, 64, 256, 64, 1, 4, 3, 2),
     GEMM_INST_PL(2, fp8_t, half_t, 64, 128, 64, 2, 2, 5, 2),
