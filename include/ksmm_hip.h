@@ -172,7 +172,12 @@ int ksmm_factor_forward_algo(const void *x, const void *w, void *y, int64_t batc
  * direct kernel exists, the workspace is ignored).  With a smaller workspace (or NULL) it
  * returns KSMM_ERR_WORKSPACE; ksmm_factor_forward (no workspace) falls back to the generic
  * kernel for such shapes.  The reference has no counterpart: its batch-size-first kernels
- * gather with strided scalar loads (template_kernels_float.cuh:156-161). */
+ * gather with strided scalar loads (template_kernels_float.cuh:156-161).
+ * The same pair serves batch-size-last problems whose batch is not a multiple of the 16-byte
+ * vector (rows that are not vector-aligned): the workspace holds the input and the output with
+ * rows zero-filled to the next multiple of 16 columns, the factor runs there with the kernel of
+ * the padded batch, and the result rows are cut back.  The reference refuses batch sizes its
+ * hyper-parameters do not divide (kernel.py:241-244). */
 int64_t ksmm_factor_workspace(int64_t batch, int a, int b, int c, int d, int x_dtype, int w_dtype,
                               int y_dtype, int bs_last);
 int ksmm_factor_forward_ws(const void *x, const void *w, void *y, int64_t batch, int a, int b,
@@ -197,7 +202,9 @@ int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int
 /* The same for a given layout and input type: a batch-size-first chain with a factor that
  * needs the transposed route asks for room for the transposed input and for ping-pong buffers
  * that also hold the (transposed) final output.  ksmm_chain_forward takes that route when the
- * workspace it is given is at least this large, and the factor-by-factor route otherwise. */
+ * workspace it is given is at least this large, and the factor-by-factor route otherwise.
+ * A batch-size-last chain whose batch is not a multiple of the 16-byte vector asks for the same
+ * buffers with rows padded to a multiple of 16 columns and runs the whole chain there. */
 int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
                                     int x_dtype, int y_dtype, int bs_last);
 

@@ -245,6 +245,25 @@ bool wants_transposed(const Problem &p)
     return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && (t.algo != KSMM_ALGO_GENERIC || t.variant == 1);
 }
 
+// Batch-size-last rows are `batch` elements long: when that is not a multiple of the 16-byte
+// vector only the one-thread-per-output kernel takes the problem.  With a workspace it runs on a
+// copy whose rows are zero-filled to the next multiple of 16 columns (the vector of every type)
+// and the result rows are cut back: two copies more, but on the kernel of the padded batch.
+int64_t padded_batch(int64_t batch) { return (batch + 15) / 16 * 16; }
+
+bool wants_padded(const Problem &p)
+{
+    if (!p.bs_last || p.batch % 16 == 0) return false;
+    ksmm_tile t;
+    memset(&t, 0, sizeof(t));
+    if (dispatch(p, KSMM_ALGO_AUTO, -1, false, &t) != KSMM_OK || t.algo != KSMM_ALGO_GENERIC || t.variant == 1)
+        return false;
+    Problem q = p;
+    q.batch = padded_batch(p.batch);
+    memset(&t, 0, sizeof(t));
+    return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && (t.algo != KSMM_ALGO_GENERIC || t.variant == 1);
+}
+
 int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 bool overlaps(const void *p, int64_t p_bytes, const void *q, int64_t q_bytes)
@@ -304,6 +323,18 @@ int factor_forward_ws_impl(const void *x, const void *w, void *y, int64_t batch,
     if (overlaps(x, xbytes, y, ybytes) || overlaps(workspace, need, x, xbytes) || overlaps(workspace, need, y, ybytes))
         return KSMM_ERR_ALIAS;
     if (((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
+    if (bs_last) {
+        // rows padded to the vector (see wants_padded)
+        const int64_t bp = padded_batch(batch);
+        char *xp = (char *)workspace;
+        char *yp = xp + align256(in_size * bp * (int64_t)dtype_size(x_dtype));
+        int rc = repitch_run(x, xp, in_size, batch, bp, (int)dtype_size(x_dtype), (hipStream_t)stream);
+        if (rc != KSMM_OK) return rc;
+        rc = factor_forward_impl(xp, w, yp, bp, a, b, c, d, x_dtype, w_dtype, y_dtype, 1, scale, KSMM_ALGO_AUTO, -1,
+                                 ep, stream);
+        if (rc != KSMM_OK) return rc;
+        return repitch_run(yp, y, out_size, bp, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+    }
     char *xt = (char *)workspace;
     char *yt = xt + align256(xbytes);
     int rc = transpose_run(x, xt, batch, in_size, (int)dtype_size(x_dtype), (hipStream_t)stream);
@@ -342,6 +373,19 @@ bool chain_wants_transposed(const ksmm_factor_desc *f, int n, int64_t batch, int
     return false;
 }
 
+// batch-size-last chain whose batch is not a multiple of the vector, with at least one factor
+// that has a real kernel at the padded batch
+bool chain_wants_padded(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype, int bs_last)
+{
+    if (!bs_last || batch % 16 == 0) return false;
+    for (int i = 0; i < n; ++i) {
+        Problem p{nullptr, nullptr, nullptr, batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
+                  f[i].w_dtype, y_dtype, 1, 1.f, nullptr};
+        if (wants_padded(p)) return true;
+    }
+    return false;
+}
+
 // The chain launcher behind ksmm_chain_forward, ksmm_chain_forward_ep and
 // ksmm_chain_forward_static: `ep` (may be null) belongs to the last factor.
 int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y, void *workspace,
@@ -366,37 +410,57 @@ int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const voi
         if (((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
     }
     auto ep_of = [&](int i) { return i == n_factors - 1 ? ep : nullptr; };
+    // The whole chain in batch-size-last layout on workspace buffers: input x0 (nb columns), two
+    // ping-pong buffers of `one` bytes at pp; *result = where the last factor's output is.
+    auto run_bs_last = [&](const void *x0, char *pp, int64_t one, int64_t nb, const void **result) -> int {
+        int rc2 = KSMM_ERR_BAD_ALGO;
+        if (fuse)
+            rc2 = chain16_run(factors, n_factors, x0, pp, nb, x_dtype, y_dtype, 1, true, (hipStream_t)stream, ep);
+        if (rc2 == KSMM_OK) {
+            *result = pp;
+            return KSMM_OK;
+        }
+        if (rc2 != KSMM_ERR_BAD_ALGO) return rc2;
+        const void *cur = x0;
+        int cur_dtype = x_dtype;
+        for (int i = 0; i < n_factors; ++i) {
+            void *dst = pp + (i & 1) * one;
+            rc2 = factor_forward_impl(cur, factors[i].w, dst, nb, factors[i].a, factors[i].b, factors[i].c,
+                                      factors[i].d, cur_dtype, factors[i].w_dtype, y_dtype, 1, factors[i].scale,
+                                      KSMM_ALGO_AUTO, -1, ep_of(i), stream);
+            if (rc2 != KSMM_OK) return rc2;
+            cur = dst;
+            cur_dtype = y_dtype;
+        }
+        *result = cur;
+        return KSMM_OK;
+    };
     if (chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
         // transpose once, run the whole chain in batch-size-last layout, transpose back
         const int64_t need_t = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 0);
         if (workspace && workspace_bytes >= need_t) {
             const int64_t xt_bytes = align256(xbytes);
             char *xt = (char *)workspace;
-            char *pp = xt + xt_bytes;
-            const int64_t one = (need_t - xt_bytes) / 2;
             rc = transpose_run(x, xt, batch, in0, (int)dtype_size(x_dtype), (hipStream_t)stream);
             if (rc != KSMM_OK) return rc;
-            const void *cur = xt;
-            int cur_dtype = x_dtype;
-            rc = KSMM_ERR_BAD_ALGO;
-            if (fuse)
-                rc = chain16_run(factors, n_factors, xt, pp, batch, x_dtype, y_dtype, 1, true, (hipStream_t)stream, ep);
-            if (rc == KSMM_OK) {
-                cur = pp;
-            } else if (rc != KSMM_ERR_BAD_ALGO) {
-                return rc;
-            } else {
-                for (int i = 0; i < n_factors; ++i) {
-                    void *dst = pp + (i & 1) * one;
-                    rc = factor_forward_impl(cur, factors[i].w, dst, batch, factors[i].a, factors[i].b, factors[i].c,
-                                             factors[i].d, cur_dtype, factors[i].w_dtype, y_dtype, 1, factors[i].scale,
-                                             KSMM_ALGO_AUTO, -1, ep_of(i), stream);
-                    if (rc != KSMM_OK) return rc;
-                    cur = dst;
-                    cur_dtype = y_dtype;
-                }
-            }
+            const void *cur = nullptr;
+            rc = run_bs_last(xt, xt + xt_bytes, (need_t - xt_bytes) / 2, batch, &cur);
+            if (rc != KSMM_OK) return rc;
             return transpose_run(cur, y, out_n, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+        }
+    } else if (chain_wants_padded(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
+        // pad the rows once, run the whole chain at the padded batch, cut the result rows back
+        const int64_t need_p = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 1);
+        if (workspace && workspace_bytes >= need_p) {
+            const int64_t bp = padded_batch(batch);
+            const int64_t xp_bytes = align256(in0 * bp * (int64_t)dtype_size(x_dtype));
+            char *xp = (char *)workspace;
+            rc = repitch_run(x, xp, in0, batch, bp, (int)dtype_size(x_dtype), (hipStream_t)stream);
+            if (rc != KSMM_OK) return rc;
+            const void *cur = nullptr;
+            rc = run_bs_last(xp, xp + xp_bytes, (need_p - xp_bytes) / 2, bp, &cur);
+            if (rc != KSMM_OK) return rc;
+            return repitch_run(cur, y, out_n, bp, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
         }
     }
     if (fuse) {
@@ -553,9 +617,11 @@ int64_t ksmm_factor_workspace(int64_t batch, int a, int b, int c, int d, int x_d
     if (rc != KSMM_OK) return rc;
     Problem p{nullptr, nullptr, nullptr, batch, a, b, c, d, x_dtype, w_dtype, y_dtype,
               bs_last ? 1 : 0, 1.f, nullptr};
-    if (!wants_transposed(p)) return 0;
-    return align256((int64_t)a * c * d * batch * (int64_t)dtype_size(x_dtype)) +
-           align256((int64_t)a * b * d * batch * (int64_t)dtype_size(y_dtype));
+    // both routes stage the input and the output: transposed, or with rows padded to the vector
+    const int64_t nb = wants_transposed(p) ? batch : wants_padded(p) ? padded_batch(batch) : 0;
+    if (nb == 0) return 0;
+    return align256((int64_t)a * c * d * nb * (int64_t)dtype_size(x_dtype)) +
+           align256((int64_t)a * b * d * nb * (int64_t)dtype_size(y_dtype));
 }
 
 int ksmm_factor_forward_ws(const void *x, const void *w, void *y, int64_t batch, int a, int b,
@@ -598,16 +664,19 @@ int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_facto
 {
     int rc = check_chain(factors, n_factors, batch, x_dtype, y_dtype);
     if (rc != KSMM_OK) return rc;
-    if (!chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last))
-        return ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
+    const int64_t nb = chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)
+                           ? batch
+                           : chain_wants_padded(factors, n_factors, batch, x_dtype, y_dtype, bs_last)
+                                 ? padded_batch(batch) : 0;
+    if (nb == 0) return ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
     int64_t widest = 0;
     for (int i = 0; i < n_factors; ++i) {
         int64_t o = (int64_t)factors[i].a * factors[i].b * factors[i].d;
         if (o > widest) widest = o;
     }
     const int64_t in0 = (int64_t)factors[0].a * factors[0].c * factors[0].d;
-    return align256(in0 * batch * (int64_t)dtype_size(x_dtype)) +
-           2 * align256(widest * batch * (int64_t)dtype_size(y_dtype));
+    return align256(in0 * nb * (int64_t)dtype_size(x_dtype)) +
+           2 * align256(widest * nb * (int64_t)dtype_size(y_dtype));
 }
 
 int ksmm_chain_forward(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,

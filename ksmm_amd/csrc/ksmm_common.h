@@ -175,6 +175,9 @@ int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch
 
 // Fused radix-16 chain (intermediates in LDS); KSMM_ERR_BAD_ALGO when the chain does not qualify.
 int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream);
+// out (rows x cols_out) = the rows of in (rows x cols_in) cut or zero-filled to cols_out columns
+int repitch_run(const void *in, void *out, int64_t rows, int64_t cols_in, int64_t cols_out, int elem_bytes,
+                hipStream_t stream);
 int chain16_run(const ksmm_factor_desc *f, int n, const void *x, void *y, int64_t batch, int x_dtype,
                 int y_dtype, int bs_last, bool launch, hipStream_t stream, const ksmm_epilogue *ep);
 

@@ -11,6 +11,10 @@
 // an odd stride in 4-byte words, so that the column reads of the store phase spread over the
 // 64 banks.
 //
+// The same file holds the row re-pitch copy (rows cut or zero-filled to another length), which
+// serves batch-size-last problems whose batch is not a multiple of the 16-byte vector: they run
+// on a copy whose rows are padded to the vector, and the result is copied back.
+//
 // Reference counterpart: none as a kernel (the reference's batch-size-first kernels gather with
 // strided scalar loads, template_kernels_float.cuh:156-161); KSLinear permutes activations with
 // torch in its 'bmm' path (interface.py:213-267).
@@ -106,7 +110,80 @@ template <int ES> const void *transpose_fn(bool vin, bool vout)
     return (const void *)ks_transpose_kernel<ES, false, false>;
 }
 
+// out (rows x cols_out) <- in (rows x cols_in): the first min(cols_in, cols_out) columns of
+// every row, zeros behind them.  A thread moves one 16-byte vector: aligned on the side whose
+// row length is a multiple of the vector (VOUT: widening, VIN: narrowing), at element alignment
+// on the other, element by element where the vector straddles the end of the row.
+template <int ES, bool VIN, bool VOUT>
+__global__ __launch_bounds__(256) void ks_repitch_kernel(const void *__restrict__ in_, void *__restrict__ out_,
+                                                        int64_t rows, int cols_in, int cols_out, int vec_per_row)
+{
+    typedef typename elem_of<ES>::type T;
+    constexpr int V = 16 / ES;
+    const T *in = (const T *)in_;
+    T *out = (T *)out_;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t r = id / vec_per_row;
+    const int c0 = (int)(id - r * vec_per_row) * V;
+    if (r >= rows) return;
+    const T *src = in + r * cols_in + c0;
+    T *dst = out + r * cols_out + c0;
+    union {
+        uint4_t v;
+        T e[V];
+    } u;
+    u.v = uint4_t{0u, 0u, 0u, 0u};
+    if (VIN) {  // cols_in % V == 0 and c0 < cols_out <= cols_in: a whole, aligned vector
+        u.v = *(const uint4_t *)src;
+    } else if (c0 + V <= cols_in) {
+        // a whole vector at element alignment (global memory takes unaligned vector accesses)
+        __builtin_memcpy(&u.v, src, 16);
+    } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+            if (c0 + j < cols_in) u.e[j] = src[j];
+    }
+    if (VOUT) {  // cols_out % V == 0
+        *(uint4_t *)dst = u.v;
+    } else if (c0 + V <= cols_out) {
+        __builtin_memcpy(dst, &u.v, 16);
+    } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+            if (c0 + j < cols_out) dst[j] = u.e[j];
+    }
+}
+
+template <int ES> const void *repitch_fn(bool vin, bool vout)
+{
+    if (vin && vout) return (const void *)ks_repitch_kernel<ES, true, true>;
+    if (vin) return (const void *)ks_repitch_kernel<ES, true, false>;
+    if (vout) return (const void *)ks_repitch_kernel<ES, false, true>;
+    return (const void *)ks_repitch_kernel<ES, false, false>;
+}
+
 }  // namespace
+
+// out (rows x cols_out) = the rows of in (rows x cols_in) cut or zero-filled to cols_out columns
+int repitch_run(const void *in, void *out, int64_t rows, int64_t cols_in, int64_t cols_out, int elem_bytes,
+                hipStream_t stream)
+{
+    if (rows < 1 || cols_in < 1 || cols_out < 1 || cols_in > 0x7fffffffLL || cols_out > 0x7fffffffLL)
+        return KSMM_ERR_TOO_LARGE;
+    const int v = 16 / elem_bytes;
+    // threads cover the output's columns; input vectors only where those all lie inside the input
+    const bool vin = cols_in % v == 0 && cols_out <= cols_in && ((uintptr_t)in & 15) == 0;
+    const bool vout = cols_out % v == 0 && ((uintptr_t)out & 15) == 0;
+    const int64_t vec_per_row = (cols_out + v - 1) / v;
+    const int64_t blocks = (rows * vec_per_row + 255) / 256;
+    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    const void *fn = elem_bytes == 4 ? repitch_fn<4>(vin, vout)
+                                     : elem_bytes == 2 ? repitch_fn<2>(vin, vout) : repitch_fn<1>(vin, vout);
+    int ci = (int)cols_in, co = (int)cols_out, vpr = (int)vec_per_row;
+    void *args[] = {(void *)&in, (void *)&out, &rows, &ci, &co, &vpr};
+    hipError_t e = hipLaunchKernel(fn, dim3((unsigned)blocks), dim3(256), args, 0, stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
 
 // out (cols x rows) = transpose of in (rows x cols); elem_bytes in {1, 2, 4}
 int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream)

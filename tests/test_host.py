@@ -230,6 +230,39 @@ def test_workspace_queries_need_no_gpu():
     assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 0) == 3 * (3072 * 512 * 2)
 
 
+def test_unaligned_batch_asks_for_room_for_padded_rows():
+    """Batch-size-last rows are `batch` elements long; when that is not a multiple of the
+    16-byte vector the library asks for room for the input and the output with rows padded to a
+    multiple of 16 columns (the reference refuses shapes without hyper-parameters,
+    kernel.py:241-244).  Aligned batches, and batch-size-first, ask for nothing."""
+    from ksmm_amd import _lib
+
+    lib = _lib.load()
+    F32, F16, F8 = _lib.KSMM_F32, _lib.KSMM_F16, _lib.KSMM_FP8_E4M3
+    pad = lambda n: (n + 255) // 256 * 256
+    for a, b, c, d in [(1, 48, 48, 16), (6, 64, 64, 1), (1, 768, 192, 2)]:
+        assert lib.ksmm_factor_workspace(25088, a, b, c, d, F32, F32, F32, 1) == 0
+        assert lib.ksmm_factor_workspace(25092, a, b, c, d, F32, F32, F32, 1) == 0      # 4 floats
+        assert lib.ksmm_factor_workspace(25087, a, b, c, d, F32, F32, F32, 0) == 0
+        assert lib.ksmm_factor_workspace(25087, a, b, c, d, F32, F32, F32, 1) == \
+            pad(a * c * d * 25088 * 4) + pad(a * b * d * 25088 * 4)
+        assert lib.ksmm_factor_workspace(25090, a, b, c, d, F16, F16, F16, 1) == \
+            pad(a * c * d * 25104 * 2) + pad(a * b * d * 25104 * 2)
+        assert lib.ksmm_factor_workspace(25096, a, b, c, d, F16, F16, F16, 1) == 0      # 8 halves
+        assert lib.ksmm_factor_workspace(25090, a, b, c, d, F8, F8, F16, 1) == \
+            pad(a * c * d * 25104) + pad(a * b * d * 25104 * 2)
+    descs = (_lib.KsmmFactorDesc * 2)()
+    for i, (a, b, c, d) in enumerate([(6, 64, 64, 1), (1, 768, 192, 2)]):
+        descs[i].w = 0
+        descs[i].a, descs[i].b, descs[i].c, descs[i].d = a, b, c, d
+        descs[i].w_dtype = F32
+        descs[i].scale = 1.0
+    assert lib.ksmm_chain_workspace_layout(descs, 2, 2000, F32, F32, 1) == lib.ksmm_chain_workspace(descs, 2, 2000, F32)
+    assert lib.ksmm_chain_workspace_layout(descs, 2, 2003, F32, F32, 1) == \
+        pad(384 * 2016 * 4) + 2 * pad(1536 * 2016 * 4)
+    assert lib.ksmm_chain_workspace_layout(descs, 2, 2003, F32, F32, 0) == lib.ksmm_chain_workspace(descs, 2, 2003, F32)
+
+
 def test_tuned_table_is_sorted_and_every_row_names_a_kernel_that_fits():
     """The measured table (the counterpart of the reference's *.best files, kernel.py:151-257):
     keys strictly ascending (binary search), every row a forced instance that takes the problem
