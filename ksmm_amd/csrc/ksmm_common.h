@@ -87,19 +87,24 @@ struct Epi {
 };
 static inline Epi epi_of(const Problem &p) { return Epi{p.scale, p.act, p.bias}; }
 
-// GELU, erf form: x * Phi(x).  erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7, branch-free:
-// one reciprocal, one exponential, a degree-5 polynomial), far inside fp32 storage rounding of
-// the result for the value range of activations.
+// GELU, erf form: x * Phi(x) = max(x, 0) - |x| * erfc(|x| / sqrt 2) / 2.  erfc by Abramowitz &
+// Stegun 7.1.26 (|error| <= 1.5e-7, branch-free: one reciprocal, one exponential, a degree-4
+// polynomial in t = 1 / (1 + p z)), far inside fp32 storage rounding of the result for the
+// value range of activations.  The constants carry the factors the formula would multiply by:
+// with z' = |x| sqrt(log2(e) / 2) the exponential is 2^(-z'^2), p is divided by sqrt(log2 e),
+// and the polynomial's coefficients are halved: 12 vector instructions per value, two of them
+// transcendental, which is what an epilogue with GELU costs next to the multiplications.
 __device__ __forceinline__ float gelu_erf(float x)
 {
-    const float z = fabsf(x) * 0.70710678118654752f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
-    float poly = fmaf(1.061405429f, t, -1.453152027f);
-    poly = fmaf(poly, t, 1.421413741f);
-    poly = fmaf(poly, t, -0.284496736f);
-    poly = fmaf(poly, t, 0.254829592f);
-    const float tail = 0.5f * poly * t * __builtin_amdgcn_exp2f(-z * z * 1.44269504088896341f);  // 0.5 * erfc(z)
-    return x * (x >= 0.f ? 1.0f - tail : tail);
+    const float ax = fabsf(x);
+    const float z = ax * 0.84932180028801907f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.2727374808792225f, z, 1.0f));
+    float poly = fmaf(0.5307027145f, t, -0.7265760135f);
+    poly = fmaf(poly, t, 0.7107068705f);
+    poly = fmaf(poly, t, -0.142248368f);
+    poly = fmaf(poly, t, 0.127414796f);
+    const float tail = (poly * t) * __builtin_amdgcn_exp2f(-(z * z));  // erfc(|x| / sqrt 2) / 2
+    return fmaf(-ax, tail, fmaxf(x, 0.f));
 }
 
 template <typename TY> __device__ __forceinline__ float epi_bias(const Epi &e, size_t feature)

@@ -230,6 +230,37 @@ def test_workspace_queries_need_no_gpu():
     assert lib.ksmm_chain_workspace_layout(descs, 2, 512, F16, F16, 0) == 3 * (3072 * 512 * 2)
 
 
+def test_gelu_constants_of_the_kernel_epilogue():
+    """The epilogue's GELU (gelu_erf in ksmm_common.h) is x * Phi(x) with erfc by Abramowitz &
+    Stegun 7.1.26 and the formula's factors folded into its constants.  The constants are read
+    from the header and the same arithmetic, in float32, is compared with the erf form of
+    torch.nn.functional.gelu evaluated in float64 (the ViT feed-forward's activation,
+    src/ksmm_py/model/vit.py:416-431): a wrong or mis-folded constant fails this."""
+    import math
+    import os
+    import re
+
+    import torch
+
+    src = open(os.path.join(os.path.dirname(__file__), "..", "ksmm_amd", "csrc", "ksmm_common.h")).read()
+    body = src[src.index("float gelu_erf(float x)"):]
+    body = body[:body.index("\n}\n")]
+    k, p, a5, a4, a3, a2, a1 = [np.float32(v) for v in re.findall(r"(-?\d+\.\d{6,})f", body)]
+    assert abs(float(k) - math.sqrt(math.log2(math.e) / 2)) < 1e-7
+    x = np.concatenate([np.linspace(-12, 12, 240001), [0.0, -0.0, 1e-20, -1e-20, 60.0, -60.0]]).astype(np.float32)
+    ax = np.abs(x)
+    z = ax * k
+    t = np.float32(1) / (p * z + np.float32(1))
+    poly = a5 * t + a4
+    for coef in (a3, a2, a1):
+        poly = poly * t + coef
+    got = np.maximum(x, np.float32(0)) - ax * ((poly * t) * np.exp2(-(z * z)))
+    want = torch.nn.functional.gelu(torch.from_numpy(x).double()).numpy()
+    assert got.dtype == np.float32
+    assert np.abs(got - want).max() <= 5e-7
+    assert np.linalg.norm(got - want) <= 1e-7 * np.linalg.norm(want)
+
+
 def test_unaligned_batch_asks_for_room_for_padded_rows():
     """Batch-size-last rows are `batch` elements long; when that is not a multiple of the
     16-byte vector the library asks for room for the input and the output with rows padded to a
