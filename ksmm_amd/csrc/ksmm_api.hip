@@ -230,8 +230,13 @@ int dispatch(const Problem &p, int algo, int variant, bool launch, ksmm_tile *ti
     }
 }
 
+// Rows of a batch-size-last workspace copy are padded to a multiple of 16 columns (the 16-byte
+// vector of every type).
+int64_t padded_batch(int64_t batch) { return (batch + 15) / 16 * 16; }
+
 // A batch-size-first problem that only the generic kernel takes, while its batch-size-last
-// twin has a real kernel: worth two transposes.
+// twin has a real kernel: worth two transposes.  (The transposed copy has padded rows, so the
+// twin runs at the padded batch.)
 bool wants_transposed(const Problem &p)
 {
     if (p.bs_last) return false;
@@ -240,6 +245,7 @@ bool wants_transposed(const Problem &p)
     if (dispatch(p, KSMM_ALGO_AUTO, -1, false, &t) != KSMM_OK || t.algo != KSMM_ALGO_GENERIC) return false;
     Problem q = p;
     q.bs_last = 1;
+    q.batch = padded_batch(p.batch);
     memset(&t, 0, sizeof(t));
     // (the vector form of the generic kernel counts as a real kernel: variant 1)
     return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && (t.algo != KSMM_ALGO_GENERIC || t.variant == 1);
@@ -249,8 +255,6 @@ bool wants_transposed(const Problem &p)
 // vector only the one-thread-per-output kernel takes the problem.  With a workspace it runs on a
 // copy whose rows are zero-filled to the next multiple of 16 columns (the vector of every type)
 // and the result rows are cut back: two copies more, but on the kernel of the padded batch.
-int64_t padded_batch(int64_t batch) { return (batch + 15) / 16 * 16; }
-
 bool wants_padded(const Problem &p)
 {
     if (!p.bs_last || p.batch % 16 == 0) return false;
@@ -335,14 +339,16 @@ int factor_forward_ws_impl(const void *x, const void *w, void *y, int64_t batch,
         if (rc != KSMM_OK) return rc;
         return repitch_run(yp, y, out_size, bp, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
     }
+    // transposed copies with rows of bp columns (bp = batch when that is a multiple of 16)
+    const int64_t bp = padded_batch(batch);
     char *xt = (char *)workspace;
-    char *yt = xt + align256(xbytes);
-    int rc = transpose_run(x, xt, batch, in_size, (int)dtype_size(x_dtype), (hipStream_t)stream);
+    char *yt = xt + align256(in_size * bp * (int64_t)dtype_size(x_dtype));
+    int rc = transpose_run(x, xt, batch, in_size, (int)dtype_size(x_dtype), (hipStream_t)stream, 0, bp);
     if (rc != KSMM_OK) return rc;
-    rc = factor_forward_impl(xt, w, yt, batch, a, b, c, d, x_dtype, w_dtype, y_dtype, 1, scale, KSMM_ALGO_AUTO, -1,
+    rc = factor_forward_impl(xt, w, yt, bp, a, b, c, d, x_dtype, w_dtype, y_dtype, 1, scale, KSMM_ALGO_AUTO, -1,
                              ep, stream);
     if (rc != KSMM_OK) return rc;
-    return transpose_run(yt, y, out_size, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+    return transpose_run(yt, y, out_size, batch, (int)dtype_size(y_dtype), (hipStream_t)stream, bp, 0);
 }
 
 int check_chain(const ksmm_factor_desc *f, int n, int64_t batch, int x_dtype, int y_dtype)
@@ -439,14 +445,15 @@ int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const voi
         // transpose once, run the whole chain in batch-size-last layout, transpose back
         const int64_t need_t = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 0);
         if (workspace && workspace_bytes >= need_t) {
-            const int64_t xt_bytes = align256(xbytes);
+            const int64_t bp = padded_batch(batch);  // row length of the transposed copies
+            const int64_t xt_bytes = align256(in0 * bp * (int64_t)dtype_size(x_dtype));
             char *xt = (char *)workspace;
-            rc = transpose_run(x, xt, batch, in0, (int)dtype_size(x_dtype), (hipStream_t)stream);
+            rc = transpose_run(x, xt, batch, in0, (int)dtype_size(x_dtype), (hipStream_t)stream, 0, bp);
             if (rc != KSMM_OK) return rc;
             const void *cur = nullptr;
-            rc = run_bs_last(xt, xt + xt_bytes, (need_t - xt_bytes) / 2, batch, &cur);
+            rc = run_bs_last(xt, xt + xt_bytes, (need_t - xt_bytes) / 2, bp, &cur);
             if (rc != KSMM_OK) return rc;
-            return transpose_run(cur, y, out_n, batch, (int)dtype_size(y_dtype), (hipStream_t)stream);
+            return transpose_run(cur, y, out_n, batch, (int)dtype_size(y_dtype), (hipStream_t)stream, bp, 0);
         }
     } else if (chain_wants_padded(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
         // pad the rows once, run the whole chain at the padded batch, cut the result rows back
@@ -618,7 +625,7 @@ int64_t ksmm_factor_workspace(int64_t batch, int a, int b, int c, int d, int x_d
     Problem p{nullptr, nullptr, nullptr, batch, a, b, c, d, x_dtype, w_dtype, y_dtype,
               bs_last ? 1 : 0, 1.f, nullptr};
     // both routes stage the input and the output: transposed, or with rows padded to the vector
-    const int64_t nb = wants_transposed(p) ? batch : wants_padded(p) ? padded_batch(batch) : 0;
+    const int64_t nb = wants_transposed(p) || wants_padded(p) ? padded_batch(batch) : 0;
     if (nb == 0) return 0;
     return align256((int64_t)a * c * d * nb * (int64_t)dtype_size(x_dtype)) +
            align256((int64_t)a * b * d * nb * (int64_t)dtype_size(y_dtype));
@@ -664,10 +671,9 @@ int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_facto
 {
     int rc = check_chain(factors, n_factors, batch, x_dtype, y_dtype);
     if (rc != KSMM_OK) return rc;
-    const int64_t nb = chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)
-                           ? batch
-                           : chain_wants_padded(factors, n_factors, batch, x_dtype, y_dtype, bs_last)
-                                 ? padded_batch(batch) : 0;
+    const int64_t nb = chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last) ||
+                               chain_wants_padded(factors, n_factors, batch, x_dtype, y_dtype, bs_last)
+                           ? padded_batch(batch) : 0;
     if (nb == 0) return ksmm_chain_workspace(factors, n_factors, batch, y_dtype);
     int64_t widest = 0;
     for (int i = 0; i < n_factors; ++i) {

@@ -179,7 +179,9 @@ int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch
               int dtype, int bs_last, float scale, hipStream_t stream, int *kernel_used);
 
 // Fused radix-16 chain (intermediates in LDS); KSMM_ERR_BAD_ALGO when the chain does not qualify.
-int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream);
+// out (cols x rows) = transpose of in (rows x cols); pitches in elements per row, 0 = dense
+int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream,
+                  int64_t in_pitch = 0, int64_t out_pitch = 0);
 // out (rows x cols_out) = the rows of in (rows x cols_in) cut or zero-filled to cols_out columns
 int repitch_run(const void *in, void *out, int64_t rows, int64_t cols_in, int64_t cols_out, int elem_bytes,
                 hipStream_t stream);

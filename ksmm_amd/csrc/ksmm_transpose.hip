@@ -31,10 +31,14 @@ template <> struct elem_of<1> { typedef uint8_t type; };
 template <> struct elem_of<2> { typedef uint16_t type; };
 template <> struct elem_of<4> { typedef uint32_t type; };
 
-// in: rows x cols, row-major; out: cols x rows.  VIN / VOUT: 16-byte vectors on that side.
+// in: rows x cols, row-major with in_pitch elements per row; out: cols x rows with out_pitch
+// elements per row.  VIN / VOUT: 16-byte vectors on that side (the pitch is a multiple of the
+// vector there; a vector may reach past the last column into the padding of its row: what it
+// reads there is never stored inside the matrix, what it writes there is never read).
 template <int ES, bool VIN, bool VOUT>
 __global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restrict__ in_, void *__restrict__ out_,
-                                                          int rows, int cols, int tiles_c)
+                                                          int rows, int cols, int tiles_c, int in_pitch,
+                                                          int out_pitch)
 {
     typedef typename elem_of<ES>::type T;
     constexpr int V = 16 / ES;             // elements per vector
@@ -52,8 +56,8 @@ __global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restric
 #pragma unroll
         for (int i = 0; i < TT * VPR / 256; ++i) {
             const int q = tid + i * 256, r = q / VPR, cv = (q % VPR) * V;
-            if (r0 + r < rows && c0 + cv < cols) {  // cols % V == 0: whole vectors
-                const uint4_t v = *(const uint4_t *)(in + (size_t)(r0 + r) * cols + c0 + cv);
+            if (r0 + r < rows && c0 + cv < cols) {  // in_pitch % V == 0: whole vectors
+                const uint4_t v = *(const uint4_t *)(in + (size_t)(r0 + r) * in_pitch + c0 + cv);
                 // 4-byte LDS writes (the odd stride leaves rows only 4-byte aligned)
                 uint32_t *dst = (uint32_t *)(tile + r * LD + cv);
                 dst[0] = v[0];
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restric
     } else {
         for (int q = tid; q < TT * TT; q += 256) {
             const int r = q / TT, c = q % TT;
-            if (r0 + r < rows && c0 + c < cols) tile[r * LD + c] = in[(size_t)(r0 + r) * cols + c0 + c];
+            if (r0 + r < rows && c0 + c < cols) tile[r * LD + c] = in[(size_t)(r0 + r) * in_pitch + c0 + c];
         }
     }
     __syncthreads();
@@ -75,7 +79,7 @@ __global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restric
 #pragma unroll
         for (int i = 0; i < TT * VPR / 256; ++i) {
             const int q = tid + i * 256, c = q / VPR, rv = (q % VPR) * V;
-            if (c0 + c < cols && r0 + rv < rows) {  // rows % V == 0
+            if (c0 + c < cols && r0 + rv < rows) {  // out_pitch % V == 0
                 T e[V];
 #pragma unroll
                 for (int j = 0; j < V; ++j) e[j] = tile[(rv + j) * LD + c];
@@ -91,13 +95,13 @@ __global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restric
                         v[j] = (uint32_t)e[4 * j] | ((uint32_t)e[4 * j + 1] << 8) | ((uint32_t)e[4 * j + 2] << 16) |
                                ((uint32_t)e[4 * j + 3] << 24);
                 }
-                *(uint4_t *)(out + (size_t)(c0 + c) * rows + r0 + rv) = v;
+                *(uint4_t *)(out + (size_t)(c0 + c) * out_pitch + r0 + rv) = v;
             }
         }
     } else {
         for (int q = tid; q < TT * TT; q += 256) {
             const int c = q / TT, r = q % TT;
-            if (r0 + r < rows && c0 + c < cols) out[(size_t)(c0 + c) * rows + r0 + r] = tile[r * LD + c];
+            if (r0 + r < rows && c0 + c < cols) out[(size_t)(c0 + c) * out_pitch + r0 + r] = tile[r * LD + c];
         }
     }
 }
@@ -185,19 +189,25 @@ int repitch_run(const void *in, void *out, int64_t rows, int64_t cols_in, int64_
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
-// out (cols x rows) = transpose of in (rows x cols); elem_bytes in {1, 2, 4}
-int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream)
+// out (cols x rows, out_pitch elements per row) = transpose of in (rows x cols, in_pitch elements
+// per row); elem_bytes in {1, 2, 4}; a pitch of 0 means the dense one
+int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream,
+                  int64_t in_pitch, int64_t out_pitch)
 {
-    if (rows < 1 || cols < 1 || rows > 0x7fffffffLL || cols > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    if (in_pitch == 0) in_pitch = cols;
+    if (out_pitch == 0) out_pitch = rows;
+    if (rows < 1 || cols < 1 || in_pitch < cols || out_pitch < rows || in_pitch > 0x7fffffffLL ||
+        out_pitch > 0x7fffffffLL)
+        return KSMM_ERR_TOO_LARGE;
     const int v = 16 / elem_bytes;
-    const bool vin = cols % v == 0 && ((uintptr_t)in & 15) == 0;
-    const bool vout = rows % v == 0 && ((uintptr_t)out & 15) == 0;
+    const bool vin = in_pitch % v == 0 && ((uintptr_t)in & 15) == 0;
+    const bool vout = out_pitch % v == 0 && ((uintptr_t)out & 15) == 0;
     const void *fn = elem_bytes == 4 ? transpose_fn<4>(vin, vout)
                                      : elem_bytes == 2 ? transpose_fn<2>(vin, vout) : transpose_fn<1>(vin, vout);
     const int64_t tiles_r = (rows + TT - 1) / TT, tiles_c = (cols + TT - 1) / TT;
     if (tiles_r * tiles_c > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
-    int rows_i = (int)rows, cols_i = (int)cols, tiles_c_i = (int)tiles_c;
-    void *args[] = {(void *)&in, (void *)&out, &rows_i, &cols_i, &tiles_c_i};
+    int rows_i = (int)rows, cols_i = (int)cols, tiles_c_i = (int)tiles_c, ip = (int)in_pitch, op = (int)out_pitch;
+    void *args[] = {(void *)&in, (void *)&out, &rows_i, &cols_i, &tiles_c_i, &ip, &op};
     hipError_t e = hipLaunchKernel(fn, dim3((unsigned)(tiles_r * tiles_c)), dim3(256), args, 0, stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }

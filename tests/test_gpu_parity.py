@@ -459,7 +459,8 @@ def test_bs_first_strided_blocks_take_the_transposed_route(prec):
     lib = _lib.load()
     dt = TORCH_DTYPE[prec]
     for pattern, batch in [((1, 192, 192, 16), 512), ((2, 128, 128, 8), 328), ((4, 64, 64, 8), 1000),
-                           ((1, 96, 96, 6), 77), ((2, 64, 256, 8), 256)]:
+                           ((1, 96, 96, 6), 77), ((2, 64, 256, 8), 256), ((1, 192, 192, 12), 1001),
+                           ((2, 128, 128, 6), 3)]:
         a, b, c, d = pattern
         ydt = torch.float16 if prec == "fp8" else dt
         need = lib.ksmm_factor_workspace(batch, a, b, c, d, dtype_code(dt), dtype_code(dt), dtype_code(ydt), 0)
@@ -468,7 +469,8 @@ def test_bs_first_strided_blocks_take_the_transposed_route(prec):
         y, z = _run_factor(pattern, batch, prec, False, "auto")
         assert O.rel_fro_error(y, z) <= TOL[prec], (pattern, batch)
         direct = query_tile(batch, pattern, dt, dt, False)["algo"] != 1   # e.g. the fp32 row kernel
-        twin = query_tile(batch, pattern, dt, dt, True)["algo"] != 1      # batch-size-last kernel
+        # batch-size-last kernel (the transposed copy has rows padded to 16 columns)
+        twin = query_tile((batch + 15) // 16 * 16, pattern, dt, dt, True)["algo"] != 1
         if direct or not twin:
             assert need == 0, pattern
             continue
@@ -485,7 +487,9 @@ def test_bs_first_strided_blocks_take_the_transposed_route(prec):
         assert rc == -9
     # chains: butterfly (fused between the transposes) and a mixed one
     for patterns, batch in [([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], 400),
-                            ([(2, 64, 64, 8), (16, 64, 64, 1)], 264)]:
+                            ([(2, 64, 64, 8), (16, 64, 64, 1)], 264),
+                            ([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], 203),
+                            ([(2, 128, 128, 6), (12, 128, 128, 1)], 77)]:
         if prec == "fp32" and patterns[0][1] == 16:
             continue
         ws4 = seeded_weights(patterns, seed=41, bound=0.25)
