@@ -745,10 +745,11 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             // pipelined instances, time ratio 0.5-0.9 inside (fp16 (1,64,256,128) 1277 -> 765 us,
             // (1,512,128,16) 333 -> 257; fp32 (1,512,128,8) 466 -> 328) and 1.0-1.3 outside
             // ((1,768,192,24) fp16, (1,192,192,32) fp32, very long c).
-            // 16-bit blocks of 768 x 768 and more are matrix-core-bound: there the batch-size-last
-            // GEMM tiles between two transposes beat this kernel (the transposes move each
-            // operand once more, the GEMM tiles run at 2-3x its matrix-core rate)
-            if (p.d == t.dd && combo != 0 && p.b >= 768 && p.c >= 768) continue;
+            // 16-bit blocks of 512 x 512 and more (b at least 512) are matrix-core-bound: there
+            // the batch-size-last GEMM tiles between two transposes beat this kernel (the
+            // transposes move each operand once more, the GEMM tiles run at 2-3x its
+            // matrix-core rate)
+            if (p.d == t.dd && combo != 0 && p.b >= 512 && (int64_t)p.b * p.c >= 512 * 512) continue;
             if (p.d != t.dd) {
                 const int64_t bd = (int64_t)p.b * p.d;
                 const bool pays = combo == 0 ? ((p.d <= 16 && p.b <= 192) || (bd <= 8192 && (p.d <= 16 || p.c <= 128)))
