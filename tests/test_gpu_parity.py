@@ -966,6 +966,10 @@ def test_auto_dispatch_at_larger_batches():
         ("fp16", False, (1, 1536, 384, 2), 25088), ("fp32", True, (1, 768, 192, 2), 25088),
         ("fp16", True, (4, 192, 192, 1), 25088), ("fp32", True, (6, 64, 64, 1), 25088),
         ("fp16", True, (1, 512, 128, 2), 12296), ("fp32", False, (3, 64, 64, 64), 4104),
+        # big 16-bit blocks with d = 4 in batch-size-first: the transposed route (algo 1 here)
+        ("fp16", False, (1, 512, 512, 4), 4100), ("fp16", False, (1, 1024, 256, 4), 4096),
+        # batch-size-last batches off the vector: the padded-rows route
+        ("fp16", True, (4, 192, 192, 1), 25083), ("fp32", True, (1, 768, 192, 2), 9001),
     ]
     seen = set()
     for prec, bs_last, pattern, batch in cases:
