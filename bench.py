@@ -83,8 +83,8 @@ def time_launches(fn, n_sets, steps, warmup):
 
 
 def pattern_copy_us(p, bs_last, srcs, dsts, steps, warmup):
-    """Time of a copy that touches memory the way a factor with square blocks does and computes
-    nothing (ksmm_tilecopy_probe), best of the tile widths the probe takes; None where the
+    """Time of a tile-at-a-time copy that touches memory the way a factor with square blocks does
+    and computes nothing (ksmm_tilecopy_probe), best of the tile widths the probe takes; None where the
     pattern has no such copy (b != c, input and output element sizes differ, bs_first, whose
     rows are contiguous)."""
     import ctypes
@@ -173,7 +173,7 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
             "pattern": p, "us": sec * 1e6, "gbs": roof["gbs"], "tflops": roof["tflops"],
             "bound": roof["bound"], "roofline_frac": roof["frac"], "floor_us": roof["floor_us"],
             "x_dtype": str(x_dt).replace("torch.", ""), "algo": tile["algo"], "variant": tile["variant"],
-            # a copy with this factor's access pattern and no arithmetic (None: no such copy)
+            # a tile-at-a-time copy with this factor's addresses and no arithmetic (None: no such copy)
             "pattern_copy_us": copy_us})
         cur = outs
     # ---- whole KSLinear (chain launcher) ----------------------------------------------------
@@ -260,10 +260,13 @@ def copy_reference(steps, warmup):
 
 
 def tiled_copy_reference(steps, warmup):
-    """A copy with the tile access pattern of the headline factor (1,48,48,16), fp32, bs_last:
-    48 rows of a block 16 rows apart, moved in pieces of 256 B .. 4 KB per row by one workgroup
-    per tile, no arithmetic.  What that access pattern reaches on this GPU, next to the linear
-    copy: the gap between the two is the price of the layout, not of the kernel."""
+    """A tile-at-a-time copy of the headline operand (ksmm_tilecopy_probe, no arithmetic): one
+    workgroup per tile of 48 rows, every load of the tile issued before its first store, which is
+    what a register-stationary block kernel has to do.  Timed with the tile addresses of the
+    headline factor (1,48,48,16), fp32, bs_last (48 rows 16 apart, pieces of 256 B .. 4 KB per
+    row) and, with the same tile size, on linear memory (48 consecutive 1 KB pieces): the two
+    differ little, both are well above the streaming copy (`copy_reference`), so the gap is the
+    price of moving whole tiles, not of the strided layout."""
     import ctypes
 
     from ksmm_amd import _lib
@@ -273,18 +276,23 @@ def tiled_copy_reference(steps, warmup):
     src = [torch.randn(768, BATCH, device="cuda") for _ in range(n_sets)]
     dst = [torch.zeros_like(t) for t in src]
     nbytes = 2 * src[0].numel() * 4
-    res = {"bytes": nbytes, "kernel": "ksmm_tilecopy_probe: tiles of 48 rows x tile_bytes, rows 16 apart"}
-    for tile_bytes in (256, 1024, 4096):
+    res = {"bytes": nbytes, "kernel": "ksmm_tilecopy_probe: tiles of 48 rows x tile_bytes, rows 16 apart; "
+                                      "linear: the same tiles as 48 consecutive pieces of linear memory"}
+    cases = [("tile_%dB" % tb, (BATCH * 4, 1, 48, 16, tb)) for tb in (256, 1024, 4096)]
+    cases.append(("linear_tile_1024B", (1024, 768 * BATCH * 4 // 1024 // 48, 48, 1, 1024)))
+    for key, (row_bytes, pa, rows, pd, tile_bytes) in cases:
         def run(j):
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            _lib.check(lib.ksmm_tilecopy_probe(src[j].data_ptr(), dst[j].data_ptr(), BATCH * 4, 1, 48, 16, tile_bytes, stream))
+            _lib.check(lib.ksmm_tilecopy_probe(src[j].data_ptr(), dst[j].data_ptr(), row_bytes, pa, rows, pd,
+                                               tile_bytes, stream))
 
+        dst[0].zero_()
         run(0)
         torch.cuda.synchronize()
         if not torch.equal(src[0], dst[0]):
             raise RuntimeError("tile copy probe: output differs from input")
         sec = time_launches(run, n_sets, steps, warmup)
-        res["tile_%dB" % tile_bytes] = {"us": sec * 1e6, "gbs": nbytes / sec / 1e9, "frac_of_8tbs": nbytes / sec / 8e12}
+        res[key] = {"us": sec * 1e6, "gbs": nbytes / sec / 1e9, "frac_of_8tbs": nbytes / sec / 8e12}
     return res
 
 

@@ -272,8 +272,9 @@ int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_byt
  * batch-size-last factor with square blocks.  x and y are (a * rows * d) rows of `row_bytes` bytes;
  * one workgroup moves the `rows` x `tile_bytes` tile of block (a_i, d_i) and one batch tile from x
  * to the same place in y (the rows of a block are d rows apart), all loads before the first
- * store.  Timed by the caller, it gives the rate a factor kernel with that tiling can reach at
- * best, which a benchmark prints beside the rate of a linear copy.  tile_bytes: a power of two,
+ * store.  Timed by the caller, it gives the rate of a copy that moves whole tiles with those
+ * addresses, which a benchmark prints beside the rate of a streaming copy (with d = 1 and
+ * row_bytes = tile_bytes the same tiles lie in linear memory).  tile_bytes: a power of two,
  * 16..4096; rows <= 48 * (4096 / tile_bytes). */
 int ksmm_tilecopy_probe(const void *x, void *y, int64_t row_bytes, int a, int rows, int d, int tile_bytes, void *stream);
 

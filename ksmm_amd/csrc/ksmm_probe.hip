@@ -66,8 +66,10 @@ __global__ __launch_bounds__(512, 1) void ks_mfma_probe_kernel(float *__restrict
 
 // A copy with the access pattern of a batch-size-last factor and nothing else: workgroup t moves
 // the `rows` x `tile_bytes` tile of block (a_i, d_i) and batch tile nt from x to the same place
-// in y, rows of a block being d rows apart.  Every load is issued before the first store.  What
-// this reaches is what a factor kernel with that tiling can reach at best.
+// in y, rows of a block being d rows apart.  Every load is issued before the first store, as in
+// a kernel that needs the whole tile before it can produce an output row.  (With d = 1 and
+// row_bytes = tile_bytes the same tiles lie in linear memory: the two rates differ little, and
+// both are below a streaming copy with a few vectors per thread.)
 constexpr int TC_MAX_PASSES = 48;
 __global__ __launch_bounds__(256) void ks_tilecopy_probe_kernel(const uint4_t *__restrict__ x, uint4_t *__restrict__ y,
                                                            int rows, int d, int64_t row_chunks, int tile_chunks,
