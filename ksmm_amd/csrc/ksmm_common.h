@@ -107,14 +107,25 @@ __device__ __forceinline__ float gelu_erf(float x)
     return fmaf(-ax, tail, fmaxf(x, 0.f));
 }
 
+// GELU of v when `on` (uniform over the wave), v otherwise: a branch, never a select, so that a
+// bias-only or plain epilogue does not pay for the GELU of every output (the empty asm keeps the
+// compiler from computing both sides and choosing).
+__device__ __forceinline__ float gelu_if(bool on, float v)
+{
+    if (on) {
+        asm volatile("");
+        v = gelu_erf(v);
+    }
+    return v;
+}
+
 template <typename TY> __device__ __forceinline__ float epi_bias(const Epi &e, size_t feature)
 {
     return e.bias ? (float)((const TY *)e.bias)[feature] : 0.f;
 }
 __device__ __forceinline__ float epi_finish(const Epi &e, float acc, float bias_value)
 {
-    const float v = fmaf(acc, e.scale, bias_value);
-    return e.act == KSMM_ACT_GELU ? gelu_erf(v) : v;
+    return gelu_if(e.act == KSMM_ACT_GELU, fmaf(acc, e.scale, bias_value));
 }
 
 // dtype combination index: 0 f32, 1 f16, 2 fp8*fp8->f16, 3 f16*fp8->f16, -1 unsupported

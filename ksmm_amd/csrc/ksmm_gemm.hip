@@ -498,7 +498,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
                         for (int e = 0; e < 16; ++e) {
                             const float v = fmaf(acc[0][i][j][e], scale, bl);
-                            acc[0][i][j][e] = gelu ? gelu_erf(v) : v;
+                            acc[0][i][j][e] = gelu_if(gelu, v);
                         }
                 } else {
                     // element u of group eg is output m0 + mb + 4*lq + 8*eg + u (x DD interleaved
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 #pragma unroll
                                 for (int dd = 0; dd < DD; ++dd) {
                                     const float v = fmaf(acc[dd][i][j][4 * eg + u], scale, (float)bb[u * DD + dd]);
-                                    acc[dd][i][j][4 * eg + u] = gelu ? gelu_erf(v) : v;
+                                    acc[dd][i][j][4 * eg + u] = gelu_if(gelu, v);
                                 }
                     }
                 }
@@ -893,7 +893,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
 #pragma unroll
                             for (int dd = 0; dd < DD; ++dd) {
                                 const float v = fmaf(acc[dd][i][j][4 * eg + u], scale, (float)bb[DD * u + dd]);
-                                acc[dd][i][j][4 * eg + u] = ep.act == KSMM_ACT_GELU ? gelu_erf(v) : v;
+                                acc[dd][i][j][4 * eg + u] = gelu_if(ep.act == KSMM_ACT_GELU, v);
                             }
                 }
             }
@@ -1203,7 +1203,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbl_kernel(const CT
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const float v = fmaf(acc[i][j][e], scale, bl);
-                        acc[i][j][e] = gelu ? gelu_erf(v) : v;
+                        acc[i][j][e] = gelu_if(gelu, v);
                     }
             }
         }
