@@ -30,6 +30,9 @@ def _descs(patterns, facs, scales):
     ([(12, 64, 64, 1), (1, 1536, 384, 2)], "fp16", False, 0, 1000, 203),    # batch-size-first chain
     ([(2, 64, 64, 8), (16, 64, 64, 1)], "fp16", False, 1, 520, 264),        # transposed route
     ([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], "fp8", True, 0, 1008, 528),
+    # second batch off the 16-byte vector: rows padded inside the scratch array
+    ([(6, 64, 64, 1), (1, 768, 192, 2)], "fp16", True, 0, 1000, 203),
+    ([(1, 16, 16, 64), (16, 16, 16, 4), (64, 16, 16, 1)], "fp8", True, 1, 1008, 333),
 ])
 def test_static_scratch_entry_point_matches_the_workspace_one(case):
     from ksmm_amd import _lib, generate_factor, quantize_fp8
