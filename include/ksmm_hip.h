@@ -247,7 +247,7 @@ int ksmm_factor_backward_weight(const void *dy, const void *x, void *dw, int64_t
 
 /* ksmm_chain_forward_ep for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): the ping-pong intermediates
- * and the transposed-route buffers live in a fixed device array inside the library,
+ * and the transposed-route and padded-rows buffers live in a fixed device array inside the library,
  * ksmm_static_scratch_bytes() = 32 MiB per GPU, instead of a caller's workspace.  It has no
  * counterpart in the reference (whose Python loop lets torch allocate every intermediate,
  * interface.py:269-291).  Chains whose ksmm_chain_workspace_layout() exceeds the array return
