@@ -84,12 +84,12 @@ def time_launches(fn, n_sets, steps, warmup):
 
 def pattern_copy_us(p, bs_last, srcs, dsts, steps, warmup):
     """Time of a tile-at-a-time copy that touches memory the way a factor with square blocks does
-    and computes nothing (ksmm_tilecopy_probe), best of the tile widths the probe takes; None where the
+    and computes nothing (ksbench_tilecopy_probe), best of the tile widths the probe takes; None where the
     pattern has no such copy (b != c, input and output element sizes differ, bs_first, whose
     rows are contiguous)."""
     import ctypes
 
-    from ksmm_amd import _lib
+    from ksmm_amd import _lib, bench_lib
 
     a, b, c, d = p
     es = srcs[0].element_size()
@@ -99,12 +99,12 @@ def pattern_copy_us(p, bs_last, srcs, dsts, steps, warmup):
         cases = [(BATCH * es, a, c, d, tb) for tb in (256, 1024, 4096) if c <= 48 * (4096 // tb)]
     else:
         return None
-    lib = _lib.load()
+    lib = bench_lib.load()
     best = None
     for row_bytes, pa, rows, pd, tb in cases:
         def run(j):
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            _lib.check(lib.ksmm_tilecopy_probe(srcs[j].data_ptr(), dsts[j].data_ptr(), row_bytes, pa, rows, pd, tb, stream))
+            _lib.check(lib.ksbench_tilecopy_probe(srcs[j].data_ptr(), dsts[j].data_ptr(), row_bytes, pa, rows, pd, tb, stream))
 
         run(0)
         torch.cuda.synchronize()
@@ -259,8 +259,42 @@ def copy_reference(steps, warmup):
             "bytes": nbytes, "kernel": "torch.add(x, 1, out=y) elementwise kernel"}
 
 
+def stream_copy_reference(steps, warmup):
+    """A hand-written streaming copy of the headline workload's bytes (ksbench_stream_copy: a
+    persistent grid, four 16-byte vectors per thread and round, non-temporal loads and stores),
+    best of a few grid sizes: the fastest way found to move these bytes on this GPU, i.e. the
+    ceiling a bandwidth-bound factor is measured against next to the 8 TB/s datasheet figure."""
+    import ctypes
+
+    from ksmm_amd import _lib, bench_lib
+
+    lib = bench_lib.load()
+    n_sets = 4
+    src = [torch.randn(768, BATCH, device="cuda") for _ in range(n_sets)]
+    dst = [torch.zeros_like(t) for t in src]
+    nbytes = 2 * src[0].numel() * 4
+    res = {"bytes": nbytes, "kernel": "ksbench_stream_copy: persistent grid x 256 threads, 4 x 16 B per thread "
+                                      "and round, non-temporal loads and stores"}
+    best = None
+    for wgs in (1024, 2048, 4096):
+        def run(j):
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            _lib.check(lib.ksbench_stream_copy(src[j].data_ptr(), dst[j].data_ptr(), src[j].numel() * 4, wgs, stream))
+
+        dst[0].zero_()
+        run(0)
+        torch.cuda.synchronize()
+        if not torch.equal(src[0], dst[0]):
+            raise RuntimeError("stream copy: output differs from input")
+        sec = time_launches(run, n_sets, steps, warmup)
+        res["workgroups_%d_us" % wgs] = sec * 1e6
+        best = sec if best is None else min(best, sec)
+    res.update({"us": best * 1e6, "gbs": nbytes / best / 1e9, "frac_of_8tbs": nbytes / best / 8e12})
+    return res
+
+
 def tiled_copy_reference(steps, warmup):
-    """A tile-at-a-time copy of the headline operand (ksmm_tilecopy_probe, no arithmetic): one
+    """A tile-at-a-time copy of the headline operand (ksbench_tilecopy_probe, no arithmetic): one
     workgroup per tile of 48 rows, every load of the tile issued before its first store, which is
     what a register-stationary block kernel has to do.  Timed with the tile addresses of the
     headline factor (1,48,48,16), fp32, bs_last (48 rows 16 apart, pieces of 256 B .. 4 KB per
@@ -269,21 +303,21 @@ def tiled_copy_reference(steps, warmup):
     price of moving whole tiles, not of the strided layout."""
     import ctypes
 
-    from ksmm_amd import _lib
+    from ksmm_amd import _lib, bench_lib
 
-    lib = _lib.load()
+    lib = bench_lib.load()
     n_sets = 4
     src = [torch.randn(768, BATCH, device="cuda") for _ in range(n_sets)]
     dst = [torch.zeros_like(t) for t in src]
     nbytes = 2 * src[0].numel() * 4
-    res = {"bytes": nbytes, "kernel": "ksmm_tilecopy_probe: tiles of 48 rows x tile_bytes, rows 16 apart; "
+    res = {"bytes": nbytes, "kernel": "ksbench_tilecopy_probe: tiles of 48 rows x tile_bytes, rows 16 apart; "
                                       "linear: the same tiles as 48 consecutive pieces of linear memory"}
     cases = [("tile_%dB" % tb, (BATCH * 4, 1, 48, 16, tb)) for tb in (256, 1024, 4096)]
     cases.append(("linear_tile_1024B", (1024, 768 * BATCH * 4 // 1024 // 48, 48, 1, 1024)))
     for key, (row_bytes, pa, rows, pd, tile_bytes) in cases:
         def run(j):
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            _lib.check(lib.ksmm_tilecopy_probe(src[j].data_ptr(), dst[j].data_ptr(), row_bytes, pa, rows, pd,
+            _lib.check(lib.ksbench_tilecopy_probe(src[j].data_ptr(), dst[j].data_ptr(), row_bytes, pa, rows, pd,
                                                tile_bytes, stream))
 
         dst[0].zero_()
@@ -302,11 +336,11 @@ def mfma_reference():
     peaks the MFMA-bound rooflines are priced against (fp16 2516.6, fp32 157.3 TFLOP/s)."""
     import ctypes
 
-    from ksmm_amd import _lib
+    from ksmm_amd import _lib, bench_lib
     from ksmm_amd.kernel import dtype_code
 
-    lib = _lib.load()
-    out = torch.empty(lib.ksmm_mfma_probe_bytes(), dtype=torch.uint8, device="cuda")
+    lib = bench_lib.load()
+    out = torch.empty(lib.ksbench_mfma_probe_bytes(), dtype=torch.uint8, device="cuda")
     res = {}
     for name, dt, iters in (("f16_32x32x16", dtype_code(torch.float16), 20000),
                             ("f32_16x16x4", dtype_code(torch.float32), 20000)):
@@ -315,7 +349,7 @@ def mfma_reference():
 
             def run(_):
                 stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-                _lib.check(lib.ksmm_mfma_probe(dt, iters, random, out.data_ptr(), out.numel(), ctypes.byref(flops), stream))
+                _lib.check(lib.ksbench_mfma_probe(dt, iters, random, out.data_ptr(), out.numel(), ctypes.byref(flops), stream))
 
             sec = time_launches(run, 1, 3, 1)
             res["%s_%s_tflops" % (name, "random" if random else "ones")] = flops.value / sec / 1e12
@@ -425,6 +459,7 @@ def main():
         for cfg in CONFIGS[1:]:
             others.append(bench_config(*cfg, steps=max(20, args.steps // 2), warmup=max(5, args.warmup // 2)))
     copy_ref = copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
+    stream_ref = stream_copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     tiled_ref = tiled_copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     mfma_ref = mfma_reference()
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
@@ -446,6 +481,7 @@ def main():
                      "unit": roof["unit"], "frac": roof["frac"], "traffic": traffic},
         "cpu_baseline": cpu,
         "copy_reference": copy_ref,
+        "stream_copy_reference": stream_ref,
         "tiled_copy_reference": tiled_ref,
         "mfma_reference": mfma_ref,
         "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),

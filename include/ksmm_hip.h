@@ -201,8 +201,9 @@ int64_t ksmm_chain_workspace(const ksmm_factor_desc *factors, int n_factors, int
 
 /* The same for a given layout and input type: a batch-size-first chain with a factor that
  * needs the transposed route asks for room for the transposed input and for ping-pong buffers
- * that also hold the (transposed) final output.  ksmm_chain_forward takes that route when the
- * workspace it is given is at least this large, and the factor-by-factor route otherwise.
+ * that also hold the (transposed) final output.  ksmm_chain_forward returns
+ * KSMM_ERR_WORKSPACE when the workspace it is given is smaller than this (or NULL while this
+ * is not 0), like ksmm_factor_forward_ws: it never falls back to a slower route silently.
  * A batch-size-last chain whose batch is not a multiple of the 16-byte vector asks for the same
  * buffers with rows padded to a multiple of 16 columns and runs the whole chain there. */
 int64_t ksmm_chain_workspace_layout(const ksmm_factor_desc *factors, int n_factors, int64_t batch,
@@ -249,8 +250,8 @@ int ksmm_factor_backward_weight(const void *dy, const void *x, void *dw, int64_t
  * capture, tight serving loops, harnesses that forbid hipMalloc): the ping-pong intermediates
  * and the transposed-route and padded-rows buffers live in a fixed device array inside the library,
  * ksmm_static_scratch_bytes() = 32 MiB per GPU, instead of a caller's workspace.  It has no
- * counterpart in the reference (whose Python loop lets torch allocate every intermediate,
- * interface.py:269-291).  Chains whose ksmm_chain_workspace_layout() exceeds the array return
+ * counterpart in the reference: it exists for the callers named above, those that cannot
+ * allocate.  Chains whose ksmm_chain_workspace_layout() exceeds the array return
  * KSMM_ERR_WORKSPACE.  Allocates nothing and frees nothing.  All calls on one GPU share the
  * array (every intermediate is fully written before it is read, so nothing has to be cleared
  * between calls): calls that overlap in time on one GPU race. */
@@ -258,25 +259,6 @@ int64_t ksmm_static_scratch_bytes(void);
 int ksmm_chain_forward_static(const ksmm_factor_desc *factors, int n_factors, const void *x, void *y,
                               int64_t batch, int x_dtype, int y_dtype, int bs_last, int fuse,
                               const ksmm_epilogue *epilogue, void *stream);
-
-/* Measurement aid, no counterpart in the reference: launches a kernel of 256 workgroups x 8 waves
- * that only issues matrix-core instructions on register operands (KSMM_F16: 32x32x16 fp16,
- * KSMM_F32: 16x16x4 fp32; `random` != 0: operands uniform in [-1, 1], else all ones) and
- * returns the flops it performs in *flops; timed by the caller, it gives the rate the matrix
- * cores sustain, which a benchmark prints beside the published peak.  `out` receives
- * ksmm_mfma_probe_bytes() bytes of checksums (so that the work cannot be optimised away). */
-int64_t ksmm_mfma_probe_bytes(void);
-int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_bytes, double *flops, void *stream);
-
-/* Measurement aid, no counterpart in the reference: a copy with the access pattern of a
- * batch-size-last factor with square blocks.  x and y are (a * rows * d) rows of `row_bytes` bytes;
- * one workgroup moves the `rows` x `tile_bytes` tile of block (a_i, d_i) and one batch tile from x
- * to the same place in y (the rows of a block are d rows apart), all loads before the first
- * store.  Timed by the caller, it gives the rate of a copy that moves whole tiles with those
- * addresses, which a benchmark prints beside the rate of a streaming copy (with d = 1 and
- * row_bytes = tile_bytes the same tiles lie in linear memory).  tile_bytes: a power of two,
- * 16..4096; rows <= 48 * (4096 / tile_bytes). */
-int ksmm_tilecopy_probe(const void *x, void *y, int64_t row_bytes, int a, int rows, int d, int tile_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -53,9 +53,6 @@ SIGNATURES = {
                                 ctypes.POINTER(c_int)]),
     "ksmm_variant_from_id": (c_int, [c_int, ctypes.c_uint32, c_int, c_int, c_int, c_int, c_int,
                                      ctypes.POINTER(c_int)]),
-    "ksmm_mfma_probe_bytes": (c_i64, []),
-    "ksmm_mfma_probe": (c_int, [c_int, c_int, c_int, c_vp, c_i64, ctypes.POINTER(ctypes.c_double), c_vp]),
-    "ksmm_tilecopy_probe": (c_int, [c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_vp]),
     "ksmm_factor_forward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, ctypes.c_float, c_vp]),
     "ksmm_factor_forward_algo": (c_int, [c_vp, c_vp, c_vp, c_i64, c_int, c_int, c_int, c_int, c_int,

@@ -246,6 +246,8 @@ bool wants_transposed(const Problem &p)
     Problem q = p;
     q.bs_last = 1;
     q.batch = padded_batch(p.batch);
+    // (a batch whose padded copies would pass the size limit stays on the kernel it has)
+    if (check_shape(q.batch, p.a, p.b, p.c, p.d, p.x_dtype, p.w_dtype, p.y_dtype) != KSMM_OK) return false;
     memset(&t, 0, sizeof(t));
     // (the vector form of the generic kernel counts as a real kernel: variant 1)
     return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && (t.algo != KSMM_ALGO_GENERIC || t.variant == 1);
@@ -264,6 +266,7 @@ bool wants_padded(const Problem &p)
         return false;
     Problem q = p;
     q.batch = padded_batch(p.batch);
+    if (check_shape(q.batch, p.a, p.b, p.c, p.d, p.x_dtype, p.w_dtype, p.y_dtype) != KSMM_OK) return false;
     memset(&t, 0, sizeof(t));
     return dispatch(q, KSMM_ALGO_AUTO, -1, false, &t) == KSMM_OK && (t.algo != KSMM_ALGO_GENERIC || t.variant == 1);
 }
@@ -443,8 +446,12 @@ int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const voi
     };
     if (chain_wants_transposed(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
         // transpose once, run the whole chain in batch-size-last layout, transpose back
+        // (a workspace below what ksmm_chain_workspace_layout() asks for is an error, as it is for
+        // ksmm_factor_forward_ws: the factor-by-factor route would land on the one-thread-per-output
+        // kernel without a word)
         const int64_t need_t = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 0);
-        if (workspace && workspace_bytes >= need_t) {
+        if (!workspace || workspace_bytes < need_t) return KSMM_ERR_WORKSPACE;
+        {
             const int64_t bp = padded_batch(batch);  // row length of the transposed copies
             const int64_t xt_bytes = align256(in0 * bp * (int64_t)dtype_size(x_dtype));
             char *xt = (char *)workspace;
@@ -458,7 +465,8 @@ int chain_forward_impl(const ksmm_factor_desc *factors, int n_factors, const voi
     } else if (chain_wants_padded(factors, n_factors, batch, x_dtype, y_dtype, bs_last)) {
         // pad the rows once, run the whole chain at the padded batch, cut the result rows back
         const int64_t need_p = ksmm_chain_workspace_layout(factors, n_factors, batch, x_dtype, y_dtype, 1);
-        if (workspace && workspace_bytes >= need_p) {
+        if (!workspace || workspace_bytes < need_p) return KSMM_ERR_WORKSPACE;
+        {
             const int64_t bp = padded_batch(batch);
             const int64_t xp_bytes = align256(in0 * bp * (int64_t)dtype_size(x_dtype));
             char *xp = (char *)workspace;

@@ -593,7 +593,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_kernel(const CT *__
 //    stages already hold the next tile's slabs): every wave turns its 32x32 blocks around in a
 //    private piece of it and stores whole 128-byte lines, without a workgroup barrier.
 // All waves multiply and store their own part of the output.
-template <typename CT, typename TY, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool EPI>
+template <typename CT, typename TY, int DD, int TM, int TN, int TK, int WM, int WN, int ST, int OCC, bool EPI, bool SP>
 __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT *__restrict__ x,
                                                                 const CT *__restrict__ w,
                                                                 TY *__restrict__ y, int batch, int a,
@@ -607,6 +607,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
     static_assert(NWAVES % 2 == 0 && C::W_CHUNKS % LOADERS == 0 && C::X_CHUNKS % LOADERS == 0, "loader split");
     static_assert(ST >= 3 && N_WAIT <= 63, "ring");
     static_assert(sizeof(CT) == 2 && sizeof(TY) == 2, "fp16 only");
+    static_assert(!SP || DD == 2, "the sparse-MFMA form is for (k, d_i) pairs");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const float scale = ep.scale;
     // bias and activation live in an instantiation of their own: next to the accumulators their
@@ -702,7 +703,9 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
 #pragma unroll
     for (int j = 0; j < C::NT; ++j) {
         const int row = (wn * C::NT + j) * 32 + (lane & 31), lq = lane >> 5;
-        xoff[j] = C::W_BYTES + row * (TK * DD * 2) + (((DD == 2 ? 2 * lq : lq) ^ swz_inner<C::X_CPR>(row)) << 4);
+        // (k, d_i) pairs: a lane's 16 halves are chunks 2 lq and 2 lq + 1 of the 4 chunks of a
+        // sub-step; the sparse MFMA wants chunks lq and lq + 2 (see the multiplication below)
+        xoff[j] = C::W_BYTES + row * (TK * DD * 2) + (((DD == 2 && !SP ? 2 * lq : lq) ^ swz_inner<C::X_CPR>(row)) << 4);
     }
     float16_t acc[DD][C::MT][C::NT];
     auto clear_acc = [&]() {
@@ -748,7 +751,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
                 typedef __attribute__((address_space(3))) uint4_t *lds_ptr;
                 const uint32_t pa = xa[j] ^ ((k0 >> 2) << 4);
                 xr[j].lo = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa);
-                xr[j].hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ 16);
+                xr[j].hi = *(lds_ptr)(lds_bytes_t)(uintptr_t)(pa ^ (SP ? 32 : 16));
             } else {
                 typedef __attribute__((address_space(3))) half8_t *lds_ptr;
                 xr[j] = *(lds_ptr)(lds_bytes_t)(uintptr_t)(xa[j] ^ ((k0 >> 3) << 4));
@@ -760,6 +763,8 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
         for (int j = 0; j < C::NT; ++j) {
             if constexpr (DD == 1) {
                 fx[0][j] = xr[j];
+            } else if constexpr (SP) {
+                // nothing to split: the sparse MFMA takes the 16 interleaved halves as they are
             } else {
             const uint4_t lo = xr[j].lo, hi = xr[j].hi;
             uint4_t e, o;
@@ -850,7 +855,31 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void ks_gemm_pbf_kernel(const CT
                     for (int i = 0; i < C::MT; ++i)
 #pragma unroll
                         for (int j = 0; j < C::NT; ++j) {
-                            acc[dd][i][j] = frag<CT>::mfma(fw[kk & 1][dd][i], fx[dd][j], acc[dd][i][j]);
+                            if constexpr (SP) {
+                                // Over the interleaved (k, d_i) axis of an input row (position
+                                // P = 2 k + d_i, 32 positions per sub-step of 16 k) the weights of
+                                // block d_i are 2:4 sparse: they sit at positions d_i and d_i + 2 of
+                                // every four.  v_smfmac_f32_32x32x32_f16 takes 16 halves per lane of
+                                // the dense operand and 8 of the compressed one; the index register
+                                // names the positions (two bits per weight: 0,2 for d_i = 0 in its
+                                // low half, 1,3 for d_i = 1 in its high half, chosen by the abid
+                                // field).  Measured operand layout (lane half h = lane / 32): the
+                                // dense operand's elements 0-7 are positions 8 h .. 8 h + 7 and its
+                                // elements 8-15 positions 16 + 8 h .., the compressed operand's
+                                // elements 0-3 go with positions 16 h .. 16 h + 7 and 4-7 with
+                                // 16 h + 8 .. 16 h + 15, i.e. they are k = 8 h .. 8 h + 7 in order,
+                                // exactly the lane's operand of the dense 32x32x16 MFMA; the input
+                                // lane reads chunks h and h + 2 of the sub-step's four.
+                                const half16_t xb = __builtin_bit_cast(half16_t, xr[kk & 1][j]);
+                                if (dd == 0)
+                                    acc[dd][i][j] = __builtin_amdgcn_smfmac_f32_32x32x32_f16(fw[kk & 1][dd][i], xb, acc[dd][i][j],
+                                                                                           (int)0xDDDD8888u, 0, 0);
+                                else
+                                    acc[dd][i][j] = __builtin_amdgcn_smfmac_f32_32x32x32_f16(fw[kk & 1][dd][i], xb, acc[dd][i][j],
+                                                                                           (int)0xDDDD8888u, 0, 1);
+                            } else {
+                                acc[dd][i][j] = frag<CT>::mfma(fw[kk & 1][dd][i], fx[dd][j], acc[dd][i][j]);
+                            }
                             const int m = kk * PER_K0 + (dd * C::MT + i) * C::NT + j;  // MFMA index in the slab
                             if (kk + 1 < K0 && (m + 1) % STRIDE == 0 && m / STRIDE < L) {
                                 if (loader) issue_one(wsrc, xsrc, dst, m / STRIDE);
@@ -1264,6 +1293,7 @@ struct GemmInst {
     int pers;   // persistent workgroups (per CU) with split memory roles (ks_gemm_pbf_kernel, ks_gemm_pbl_kernel)
     const void *fn[2];  // plain, with bias/activation
     int mtail;  // takes b that is not a multiple of tm (the last TM-tile is partly masked)
+    int sp;     // d == 2 operands go to the 2:4 sparse MFMA as (k, d_i) pairs
 };
 // OCC_: waves per SIMD the register allocation must allow (2 lets two workgroups share a CU,
 // so that one multiplies while the other stores its output tile)
@@ -1275,9 +1305,14 @@ struct GemmInst {
                    (const void *)ks_gemm_kernel<CT_, TY_, BL_, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, KT_, true>}}
 #define GEMM_INST_PO(DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                                          \
     {1, false, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, DD_, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
-     8, 0, WM_, OCC_, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false>, \
-                       (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, true>}}
+     8, 0, WM_, OCC_, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false, false>, \
+                       (const void *)ks_gemm_pbf_kernel<half_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, true, false>}}
 #define GEMM_INST_P(DD_, TM_, TN_, TK_, WM_, WN_, ST_) GEMM_INST_PO(DD_, TM_, TN_, TK_, WM_, WN_, ST_, 1)
+// d == 2 through the 2:4 sparse MFMA (no operand split); `sp` tells the instances apart
+#define GEMM_INST_PS(TM_, TN_, TK_, WM_, WN_, ST_, OCC_)                                               \
+    {1, false, 2, TM_, TN_, TK_, 64 * WM_ * WN_, GemmCfg<half_t, false, 2, TM_, TN_, TK_, WM_, WN_, ST_>::LDS_BYTES, \
+     8, 0, WM_, OCC_, {(const void *)ks_gemm_pbf_kernel<half_t, half_t, 2, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, false, true>, \
+                       (const void *)ks_gemm_pbf_kernel<half_t, half_t, 2, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, true, true>}, 0, 1}
 // OCC_: persistent workgroups per CU (4-wave tiles: two); MT_: partial last TM-tile
 #define GEMM_INST_PLM(COMBO_, CT_, TY_, TM_, TN_, TK_, WM_, WN_, ST_, OCC_, MT_)                      \
     {COMBO_, true, 1, TM_, TN_, TK_, 64 * WM_ * WN_,                                                  \
@@ -1363,6 +1398,10 @@ const GemmInst gemm_insts[] = {
     GEMM_INST_PLM(0, float, float, 64, 128, 16, 2, 2, 5, 2, true),
     // fp16 bs_first d == 2: 4-wave tile, two persistent workgroups per CU (b = 64, 192, ...)
     GEMM_INST_PO(2, 64, 128, 32, 1, 4, 3, 2),
+    // the d == 2 persistent tiles on the sparse MFMA
+    GEMM_INST_PS(256, 128, 32, 4, 2, 3, 1),
+    GEMM_INST_PS(128, 256, 32, 2, 4, 3, 1),
+    GEMM_INST_PS(64, 128, 32, 1, 4, 3, 2),
     // fp16 bs_first d == 1: 4-wave tiles of 64 and 128 rows
     GEMM_INST_PO(1, 64, 256, 32, 1, 4, 3, 2),
     GEMM_INST_PO(1, 128, 256, 32, 2, 2, 3, 2),
@@ -1405,8 +1444,8 @@ uint32_t gemm_inst_id(int i)
     if (i < 0 || i >= N_GEMM_INSTS) return 0;
     const GemmInst &t = gemm_insts[i];
     // threads and the LDS footprint stand for the wave grid and the ring depth
-    const int v[12] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm, t.pers, t.mtail};
-    return inst_hash('G', v, t.mtail ? 12 : 11);  // (ids of the other instances predate the field)
+    const int v[13] = {t.combo, t.bs_last, t.dd, t.tm, t.tn, t.tk, t.threads, t.lds, t.ktail, t.wm, t.pers, t.mtail, t.sp};
+    return inst_hash('G', v, t.sp ? 13 : t.mtail ? 12 : 11);  // (ids of the other instances predate the fields)
 }
 
 // variant: index into the instance table; -1: first that fits with enough workgroups to fill

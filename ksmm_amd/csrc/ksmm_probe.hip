@@ -1,9 +1,12 @@
-// Measurement aid: the rate at which the matrix cores multiply operands that are already in
-// registers.  A benchmark prints it beside the kernels' own figures, as a copy kernel's rate is
-// printed beside bandwidth-bound ones: with random operands the rate an MI355X sustains is well
-// under the published peak (clock and power management), and no kernel can beat it.
+// Measurement aids of the benchmark, built into a library of their own (libksmm_bench.so): they
+// are not part of the drop-in ABI.  (1) The rate at which the matrix cores multiply operands that
+// are already in registers: with random operands the rate an MI355X sustains is well under the
+// published peak (clock and power management), and no kernel can beat it.  (2) A copy that moves
+// whole tiles with the addresses of a batch-size-last factor.  (3) A streaming copy with
+// non-temporal loads and stores, the fastest way found to move bytes through this memory system.
 // No counterpart in the reference.
 #include "ksmm_mfma.h"
+#include "ksmm_probe.h"
 
 namespace ksmm {
 
@@ -93,19 +96,55 @@ __global__ __launch_bounds__(256) void ks_tilecopy_probe_kernel(const uint4_t *_
     }
 }
 
+// Streaming copy: a persistent grid, every thread moves VPT 16-byte vectors per round (all loads
+// of a round before its stores), consecutive threads consecutive vectors, non-temporal both ways.
+constexpr int SC_VPT = 4;
+__global__ __launch_bounds__(256) void ks_stream_copy_kernel(const uint4_t *__restrict__ x, uint4_t *__restrict__ y,
+                                                        int64_t n_vec)
+{
+    const int64_t per_round = (int64_t)gridDim.x * 256 * SC_VPT;
+    for (int64_t base = (int64_t)blockIdx.x * 256 * SC_VPT; base < n_vec; base += per_round) {
+        uint4_t v[SC_VPT];
+#pragma unroll
+        for (int i = 0; i < SC_VPT; ++i) {
+            const int64_t q = base + i * 256 + threadIdx.x;
+            if (q < n_vec) v[i] = __builtin_nontemporal_load(x + q);
+        }
+#pragma unroll
+        for (int i = 0; i < SC_VPT; ++i) {
+            const int64_t q = base + i * 256 + threadIdx.x;
+            if (q < n_vec) __builtin_nontemporal_store(v[i], y + q);
+        }
+    }
+}
+
 }  // namespace
 
 }  // namespace ksmm
 
 extern "C" {
 
-int64_t ksmm_mfma_probe_bytes(void) { return 256ll * 512 * (int64_t)sizeof(float); }
+int ksbench_stream_copy(const void *x, void *y, int64_t bytes, int workgroups, void *stream)
+{
+    using namespace ksmm;
+    if (!x || !y) return KSMM_ERR_NULL_POINTER;
+    if ((((uintptr_t)x | (uintptr_t)y) & 15) || bytes < 16 || bytes % 16) return KSMM_ERR_WORKSPACE;
+    if (workgroups < 1 || workgroups > 65536) return KSMM_ERR_BAD_PATTERN;
+    int64_t n_vec = bytes / 16;
+    void *args[] = {(void *)&x, (void *)&y, &n_vec};
+    return hipLaunchKernel((const void *)ks_stream_copy_kernel, dim3((unsigned)workgroups), dim3(256), args, 0,
+                           (hipStream_t)stream) == hipSuccess
+               ? KSMM_OK
+               : KSMM_ERR_LAUNCH;
+}
 
-int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_bytes, double *flops, void *stream)
+int64_t ksbench_mfma_probe_bytes(void) { return 256ll * 512 * (int64_t)sizeof(float); }
+
+int ksbench_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_bytes, double *flops, void *stream)
 {
     using namespace ksmm;
     if (!out || !flops) return KSMM_ERR_NULL_POINTER;
-    if (out_bytes < ksmm_mfma_probe_bytes() || ((uintptr_t)out & 3)) return KSMM_ERR_WORKSPACE;
+    if (out_bytes < ksbench_mfma_probe_bytes() || ((uintptr_t)out & 3)) return KSMM_ERR_WORKSPACE;
     if (iters < 1 || iters > (1 << 24)) return KSMM_ERR_BAD_BATCH;
     const void *fn;
     double per_iter;  // flops per wave and iteration
@@ -123,7 +162,7 @@ int ksmm_mfma_probe(int dtype, int iters, int random, void *out, int64_t out_byt
     return hipLaunchKernel(fn, dim3(256), dim3(512), args, 0, (hipStream_t)stream) == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
-int ksmm_tilecopy_probe(const void *x, void *y, int64_t row_bytes, int a, int rows, int d, int tile_bytes, void *stream)
+int ksbench_tilecopy_probe(const void *x, void *y, int64_t row_bytes, int a, int rows, int d, int tile_bytes, void *stream)
 {
     using namespace ksmm;
     if (!x || !y) return KSMM_ERR_NULL_POINTER;

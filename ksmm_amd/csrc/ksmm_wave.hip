@@ -251,6 +251,229 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
 }
 
 // ------------------------------------------------------------------------------------------
+// fp32 "ring" form: the same wave-per-block design, with the input rows of the next tile
+// arriving by direct-to-LDS loads (global_load_lds_dwordx4) instead of into registers.
+//
+// What bounds the register form is the number of bytes a CU keeps in flight: a wave owns one
+// tile of staging registers next to the weight block and the accumulators, and a CU runs four
+// such waves.  Here a wave owns a private piece of LDS of KS kilobytes, one per k-step: the load
+// of k-step ks of the next tile is issued into slot ks as soon as the current tile has read
+// that slot, and the lane that requested 16 bytes is the lane that reads them back
+// (ds_read_b128 of its own 16 bytes: conflict-free, and no barrier, the waves stay
+// independent).  The registers that held the staged tile now hold a second set of accumulators:
+// the stores of tile t are issued one by one between the k-steps of tile t + 1 instead of in a
+// burst behind it.  Up to eight such waves share a CU (LDS: KS KB per wave).
+//
+// Vector-memory operations of a wave complete in the order they were issued, and the counter
+// behind s_waitcnt vmcnt(N) counts loads and stores alike: "the load of slot ks has landed" is
+// "at most N operations younger than it are outstanding", with N the number of operations
+// issued after it, which the loop structure fixes: per k-step one load (while there is a next
+// tile) followed by that step's share of the previous tile's stores.  A count that is too
+// small only waits longer, so the first two tiles of a wave (whose loads were not yet followed
+// by a full tile of stores) use the count without stores.
+// ------------------------------------------------------------------------------------------
+constexpr int vmcnt_enc(int n)
+{
+    const int m = n > 63 ? 63 : n;
+    return (m & 15) | (7 << 4) | (15 << 8) | (((m >> 4) & 3) << 14);
+}
+
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+__device__ __forceinline__ void ring_dma16(const void *sbase, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+// the lane's own 16 bytes of a slot, complete when the function returns
+template <int OFF> __device__ __forceinline__ float4_t ring_read16(uint32_t lds_addr)
+{
+    float4_t v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr), "n"(OFF) : "memory");
+    return v;
+}
+
+template <int MT, int KS, bool DEFER, bool EPI>
+__global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restrict__ x,
+                                                            const float *__restrict__ w,
+                                                            float *__restrict__ y, int batch, int a, int b,
+                                                            int c, int d, Epi ep, int n_slabs,
+                                                            int iters, int rr)
+{
+    (void)iters;
+    (void)rr;
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring_smem[];
+    const float scale = ep.scale;
+    constexpr int VEC = 4, TN = 16 * VEC;
+    constexpr int NST = 4 * MT;  // store instructions per tile (4 rows x 256 bytes each)
+    static_assert(KS * 1024 + 1023 < 65536, "slot offsets are 16-bit immediates");
+    const int lane = threadIdx.x & 63;
+    const int q = lane >> 4, r = lane & 15;
+    const int wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + wave_in_wg);
+    const int m_split = b / (16 * MT);
+    const int gh = wave / n_slabs;
+    const int g = gh / m_split;  // block index a_i * d + d_i
+    if (g >= a * d) return;
+    const int m_off = (gh - g * m_split) * (16 * MT);
+    const int slab = wave - gh * n_slabs;
+    const int a_i = g / d, d_i = g - a_i * d;
+    // tiles of this wave: every n_slabs-th tile of the block's row of tiles, so that the waves of
+    // a workgroup read neighbouring 256-byte pieces of the same rows at any one time
+    const int n_tiles_row = (batch + TN - 1) / TN;
+    const int count = slab < n_tiles_row ? (n_tiles_row - slab + n_slabs - 1) / n_slabs : 0;
+    if (count <= 0) return;
+
+    float areg[MT][KS];
+    {
+        const float *wg = w + (size_t)g * c * b;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) areg[mt][ks] = wg[(4 * ks + q) * b + m_off + 16 * mt + r];
+    }
+    const size_t row_stride = (size_t)d * batch;  // elements between consecutive c_i (or b_i)
+    const char *const xg = (const char *)(x + ((size_t)a_i * c * d + d_i) * batch);
+    char *const yg = (char *)(y + (((size_t)a_i * b + m_off) * d + d_i) * batch);
+    const uint32_t x_lane = (uint32_t)(q * row_stride) * 4u;      // + column offset
+    const uint32_t y_lane = (uint32_t)(4 * q * row_stride) * 4u;  // + column offset
+    const size_t x_step = row_stride * 16;                        // bytes per k-step (4 rows)
+    const int last_vec = batch - VEC;
+    // Columns past the end are clamped to the last valid vector (batch % VEC == 0): such a lane
+    // computes the outputs of that vector and stores them there, a second copy of the same values.
+    auto col_off = [&](int k) { return (uint32_t)min((slab + k * n_slabs) * TN + VEC * r, last_vec) * 4u; };
+    float bv[EPI ? MT : 1][4];
+    if constexpr (EPI) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * b + m_off + 16 * mt + 4 * q + i) * d + d_i);
+    }
+    const uint32_t lds_wave = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)ring_smem +
+                              (uint32_t)wave_in_wg * (KS * 1024);
+    const uint32_t lds_lane = lds_wave + (uint32_t)lane * 16u;
+    __builtin_amdgcn_s_waitcnt(0);  // weights and bias are here: the counter starts clean
+    {
+        const uint32_t off = x_lane + col_off(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ring_dma16(xg + ks * x_step, off, lds_wave + ks * 1024);
+    }
+    auto store_one = [&](const float4_t(&acc)[MT][VEC], int s, uint32_t off) {
+        const int mt = s >> 2, i = s & 3;
+        float4_t o;
+        if constexpr (EPI)
+            o = float4_t{epi_finish(ep, acc[mt][0][i], bv[mt][i]), epi_finish(ep, acc[mt][1][i], bv[mt][i]),
+                         epi_finish(ep, acc[mt][2][i], bv[mt][i]), epi_finish(ep, acc[mt][3][i], bv[mt][i])};
+        else
+            o = float4_t{acc[mt][0][i] * scale, acc[mt][1][i] * scale, acc[mt][2][i] * scale, acc[mt][3][i] * scale};
+        *(float4_t *)(yg + (size_t)(16 * mt + i) * row_stride * 4 + off) = o;
+    };
+    // One tile: k-step ks waits for slot ks, reads it, hands the slot to the next tile's load,
+    // multiplies, and issues the stores of the previous tile that fall to this step.
+    //  has_prev: `prev` holds a finished tile whose stores go out between the k-steps
+    //  steady:   the tile before the previous one existed as well, so a full tile of stores was
+    //            issued behind each load this tile waits for: exact counts
+    //  has_next: there is a next tile to request
+    auto do_tile = [&](float4_t(&cur)[MT][VEC], const float4_t(&prev)[MT][VEC], uint32_t next_off, uint32_t prev_off,
+                       auto has_prev, auto steady, auto has_next) {
+        constexpr bool HAS_PREV = decltype(has_prev)::value, STEADY = decltype(steady)::value,
+                       HAS_NEXT = decltype(has_next)::value;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) cur[mt][v] = float4_t{0.f, 0.f, 0.f, 0.f};
+        const uint32_t noff = x_lane + next_off;
+        const uint32_t poff = y_lane + prev_off;
+        static_for<0, KS>([&](auto ks_c) {
+            constexpr int ks = decltype(ks_c)::value;
+            // operations issued after the load of (this tile, ks): the loads of the later k-steps
+            // of the tile it was issued in, the loads of the earlier k-steps of this tile, and in
+            // the steady state one tile's worth of stores
+            constexpr int after = (KS - 1 - ks) + (HAS_NEXT ? ks : 0) + (STEADY ? NST : 0);
+            __builtin_amdgcn_s_waitcnt(vmcnt_enc(after));
+            const float4_t xv = ring_read16<ks * 1024>(lds_lane);
+            if constexpr (HAS_NEXT) ring_dma16(xg + ks * x_step, noff, lds_wave + ks * 1024);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    cur[mt][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[mt][ks], xv[v], cur[mt][v], 0, 0, 0);
+            if constexpr (HAS_PREV) {
+                // stores s with s * KS / NST == ks: spread evenly over the k-steps
+#pragma unroll
+                for (int s = 0; s < NST; ++s)
+                    if (s * KS / NST == ks) store_one(prev, s, poff);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto flush = [&](const float4_t(&acc)[MT][VEC], uint32_t off) {
+#pragma unroll
+        for (int s = 0; s < NST; ++s) store_one(acc, s, y_lane + off);
+    };
+    float4_t acc_a[MT][VEC];
+    const std::true_type yes{};
+    const std::false_type no{};
+    if constexpr (!DEFER) {
+        // one set of accumulators (blocks whose weights leave no room for two): a tile's stores
+        // follow its last k-step in a burst, so from the second tile on every load waited for
+        // has a tile of stores behind it
+        if (count == 1) {
+            do_tile(acc_a, acc_a, 0u, 0u, no, no, no);
+            flush(acc_a, col_off(0));
+            return;
+        }
+        do_tile(acc_a, acc_a, col_off(1), 0u, no, no, yes);
+        flush(acc_a, col_off(0));
+        int k = 1;
+        for (; k + 1 < count; ++k) {
+            do_tile(acc_a, acc_a, col_off(k + 1), 0u, no, yes, yes);
+            flush(acc_a, col_off(k));
+        }
+        do_tile(acc_a, acc_a, 0u, 0u, no, yes, no);
+        flush(acc_a, col_off(k));
+    } else {
+    float4_t acc_b[MT][VEC];
+    // tile k of the wave uses acc_a for even k, acc_b for odd k
+    if (count == 1) {
+        do_tile(acc_a, acc_b, 0u, 0u, no, no, no);
+        flush(acc_a, col_off(0));
+        return;
+    }
+    do_tile(acc_a, acc_b, col_off(1), 0u, no, no, yes);
+    if (count == 2) {
+        do_tile(acc_b, acc_a, 0u, col_off(0), yes, no, no);
+        flush(acc_b, col_off(1));
+        return;
+    }
+    do_tile(acc_b, acc_a, col_off(2), col_off(0), yes, no, yes);
+    int k = 2;
+    for (; k + 2 < count; k += 2) {
+        do_tile(acc_a, acc_b, col_off(k + 1), col_off(k - 1), yes, yes, yes);
+        do_tile(acc_b, acc_a, col_off(k + 2), col_off(k), yes, yes, yes);
+    }
+    if (count - k == 2) {
+        do_tile(acc_a, acc_b, col_off(k + 1), col_off(k - 1), yes, yes, yes);
+        do_tile(acc_b, acc_a, 0u, col_off(k), yes, yes, no);
+        flush(acc_b, col_off(k + 1));
+    } else {
+        do_tile(acc_a, acc_b, 0u, col_off(k - 1), yes, yes, no);
+        flush(acc_a, col_off(k));
+    }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // 16-bit MFMA path: x is fp16 or e4m3fn (decoded to fp16, exact), w is fp16 or e4m3fn,
 // y is fp16.  MT = b / 16, KS = c / (4 * KL).  Each wave iteration covers 16 * VEC columns.
 // ------------------------------------------------------------------------------------------
@@ -411,6 +634,7 @@ struct WaveInst {
     // [0]: several tiles per wave, rolling register pipeline; [1]: one tile per wave (nothing is
     // reloaded); [2], [3]: the same with bias / activation
     const void *fn[4];
+    int ring = 0;  // > 0: the ring form, with at most this many waves per workgroup (LDS: c / 4 KB each)
 };
 
 typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, Epi, int, int, int);
@@ -422,6 +646,11 @@ using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int,
 #define F32_INST(B_, C_, OCC_) \
     {B_, C_, 4, 1, OCC_, {F32_FN(B_, C_, OCC_, true, false), F32_FN(B_, C_, OCC_, false, false), \
                           F32_FN(B_, C_, OCC_, true, true), F32_FN(B_, C_, OCC_, false, true)}}
+// DEFER_: a second set of accumulators, the stores of a tile spread over the next one
+#define F32_RING_FN(B_, C_, DEFER_, EPI_) (const void *)(f32_fn)ks_wave_ring_f32<B_ / 16, C_ / 4, DEFER_, EPI_>
+#define F32_RING(B_, C_, DEFER_, WAVES_) \
+    {B_, C_, 4, 1, DEFER_ ? 1 : 2, {F32_RING_FN(B_, C_, DEFER_, false), F32_RING_FN(B_, C_, DEFER_, false), \
+                                    F32_RING_FN(B_, C_, DEFER_, true), F32_RING_FN(B_, C_, DEFER_, true)}, WAVES_}
 const WaveInst f32_insts[] = {
     F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
     F32_INST(16, 16, 4), F32_INST(32, 32, 3), F32_INST(48, 192, 1),
@@ -429,6 +658,9 @@ const WaveInst f32_insts[] = {
     // weight registers, three waves per SIMD; 6 % faster than the whole block per wave on
     // (6,64,64,1) at batch 25088 (groups of 16 rows were 15-40 % slower there and on 48 x 48)
     F32_INST(32, 64, 3),
+    // ring form (input through a per-wave LDS ring, stores spread over the next tile)
+    F32_RING(48, 48, true, 8), F32_RING(64, 64, false, 8), F32_RING(32, 64, true, 8), F32_RING(16, 16, true, 8),
+    F32_RING(32, 32, true, 8), F32_RING(48, 48, false, 8),
 };
 
 #define H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, ROLL_, EPI_) \
@@ -452,6 +684,9 @@ const WaveInst q_insts[] = {
     H_INST(fp8_t, fp8_t, 16, 16, 4, 16, 3), H_INST(fp8_t, fp8_t, 32, 32, 8, 16, 2),
     H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),  H_INST(fp8_t, fp8_t, 48, 192, 8, 8, 1),
 };
+
+// whether the automatic choice may take ring instances (listed behind the register forms)
+constexpr bool RING_BY_DEFAULT = false;
 
 const WaveInst *wave_table(int combo, int *n)
 {
@@ -478,8 +713,8 @@ uint32_t wave_inst_id(int combo, int i)
     int n;
     const WaveInst *t = wave_table(combo, &n);
     if (i < 0 || i >= n) return 0;
-    const int v[6] = {combo, t[i].b, t[i].c, t[i].vec, t[i].kl, t[i].occ};
-    return inst_hash('W', v, 6);
+    const int v[7] = {combo, t[i].b, t[i].c, t[i].vec, t[i].kl, t[i].occ, t[i].ring};
+    return inst_hash('W', v, t[i].ring ? 7 : 6);  // (ids of the register-form instances predate the field)
 }
 
 int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
@@ -506,6 +741,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         if (!rows_ok || insts[i].c != p.c) continue;
         if (p.batch % insts[i].vec) continue;
         if (want != 0xff && want != i) continue;
+        if (want == 0xff && insts[i].ring && !RING_BY_DEFAULT) continue;
         pick = i;
         break;
     }
@@ -522,6 +758,53 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     }
     const int tn = 16 * in.vec;
     const int64_t n_tiles = (p.batch + tn - 1) / tn;
+    if (in.ring) {
+        // Ring form: every wave takes every n_slabs-th tile of its block's row of tiles.  Tiles per
+        // wave (bits 8-15, 0: automatic): the smallest number with which all waves are resident at
+        // once (at most in.ring waves per CU, and what the LDS holds: c / 4 KB per wave), so that
+        // all of them share the work evenly; bits 18-21: waves per workgroup (0: as many as spread
+        // the waves over one workgroup per CU).
+        const int64_t groups = (int64_t)p.a * p.d * (p.b / in.b);
+        const int ks = p.c / 4;
+        int wmax = in.ring;
+        if (wmax * ks > 160) wmax = 160 / ks;
+        int wpw = variant < 0 ? 0 : ((variant >> 18) & 15);
+        if (wpw > wmax || wmax < 1) return KSMM_ERR_BAD_ALGO;
+        if (iters == 0) {
+            iters = 1;
+            while (iters < 255 && groups * ((n_tiles + iters - 1) / iters) > 256 * (int64_t)(wpw ? wpw : wmax)) ++iters;
+        }
+        const int64_t n_slabs = (n_tiles + iters - 1) / iters;
+        const int64_t waves = groups * n_slabs;
+        if (wpw == 0) {
+            wpw = (int)((waves + 255) / 256);
+            if (wpw < 4) wpw = 4;  // (small problems: fewer, fuller workgroups)
+            if (wpw > wmax) wpw = wmax;
+        }
+        const int64_t blocks = (waves + wpw - 1) / wpw;
+        if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+        const int lds = wpw * ks * 1024;
+        if (tile) {
+            tile->algo = KSMM_ALGO_WAVE;
+            tile->variant = pick | (iters << 8) | (wpw << 18);
+            tile->tile_m = in.b;
+            tile->tile_n = tn;
+            tile->tile_k = p.c;
+            tile->tile_d = 1;
+            tile->threads = 64 * wpw;
+            tile->lds_bytes = lds;
+            tile->grid = blocks;
+        }
+        if (!launch) return KSMM_OK;
+        Epi ep = epi_of(p);
+        const void *fn = in.fn[p.bias || p.act ? 2 : 0];
+        if (ensure_dynamic_lds(fn, wmax * ks * 1024) != KSMM_OK) return KSMM_ERR_LAUNCH;
+        int batch_i = (int)p.batch, n_slabs_i = (int)n_slabs, rr_i = 1;
+        void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.b,
+                        (void *)&p.c, (void *)&p.d, &ep, &n_slabs_i, &iters, &rr_i};
+        hipError_t e = hipLaunchKernel(fn, dim3((unsigned)blocks), dim3(64 * wpw), args, lds, p.stream);
+        return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+    }
     // Tiles per wave.  Small blocks (16x16, 32x32) have little matrix work per byte: one tile
     // per wave and many waves in flight measured best.  Larger blocks keep a SIMD's matrix pipe
     // busy for microseconds per tile; there a single round of workgroups (at most one per CU,

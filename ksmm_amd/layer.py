@@ -104,6 +104,14 @@ class KSLinear(nn.Module):
     """Drop-in for the reference's ``KSLinear`` on the ``kernel``/``dense``/``bmm``/``einsum``
     algorithms.
 
+    ``algo='kernel'`` has two modes.  Without gradients (``torch.no_grad()``, which is how the
+    reference runs it, utils.py:6-8, or when neither the input nor a factor requires a gradient)
+    the whole layer is one call of the chain launcher: intermediates in a workspace or in LDS,
+    bias and activation inside the last factor's kernel.  With gradients enabled and trainable
+    factors (the state of a freshly built layer, ``eval()`` included) it runs factor by factor
+    through an autograd function that keeps the intermediates for the backward pass, and bias
+    and activation are PyTorch operations; both modes compute the same function.
+
     Beyond the reference's signature: ``fuse`` lets the chain launcher keep intermediates in
     LDS where it has a kernel for the chain, and ``act='gelu'`` applies GELU (erf form) after
     the bias, as the feed-forward block of the reference's ViT does between its two
@@ -244,13 +252,17 @@ class KSLinear(nn.Module):
         return self.post_process(tensor, output)
 
     # -- helpers -----------------------------------------------------------------------------
-    def get_dense_product(self):
-        """Dense matrix of the whole layer, K_L ... K_1 (interface.py:363-437)."""
+    def get_dense_product(self, dtype=None):
+        """Dense matrix of the whole layer, K_L ... K_1 (interface.py:363-437), multiplied in the
+        factors' own type like the reference does, or in ``dtype`` when one is given (e4m3
+        factors are dequantised to fp32 first either way)."""
         mats = []
         for factor, pattern, s in zip(self.factors, self.patterns, self.w_scales):
             f = factor.detach()
             if f.dtype == FP8:
                 f = f.to(torch.float32) * s
+            if dtype is not None:
+                f = f.to(dtype)
             if self.algo == "bmm":
                 mats.append(from_bmm_format_to_dense(f, pattern))
             elif self.algo == "kernel":

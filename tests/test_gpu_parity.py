@@ -923,28 +923,36 @@ def test_persistent_gemm_batch_size_last():
 
 
 def test_measurement_probes():
-    """The two measurement aids of the library: the tile copy must reproduce its input exactly
-    (ragged last batch tile, several blocks, every supported tile width) and refuse tiles it
-    cannot hold; the matrix-core probe must report the flops it was asked to perform."""
+    """The measurement aids of the benchmark (libksmm_bench.so, not part of the drop-in ABI): the
+    tile copy and the streaming copy must reproduce their input exactly (ragged last batch tile,
+    several blocks, every supported tile width; a size that is not a multiple of a round) and
+    refuse what they cannot hold; the matrix-core probe must report the flops it was asked to
+    perform."""
     import ctypes
 
-    from ksmm_amd import _lib
+    from ksmm_amd import _lib, bench_lib
     from ksmm_amd.kernel import dtype_code
 
-    lib = _lib.load()
+    lib = bench_lib.load()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     a, rows, d, batch = 2, 48, 3, 1000  # 4000-byte rows: 250 vectors, ragged for every tile width
     x = torch.randn(a * rows * d, batch, device="cuda")
     for tile_bytes in (16, 256, 1024, 4096):
         y = torch.zeros_like(x)
-        _lib.check(lib.ksmm_tilecopy_probe(x.data_ptr(), y.data_ptr(), batch * 4, a, rows, d, tile_bytes, stream))
+        _lib.check(lib.ksbench_tilecopy_probe(x.data_ptr(), y.data_ptr(), batch * 4, a, rows, d, tile_bytes, stream))
         torch.cuda.synchronize()
         assert torch.equal(x, y), tile_bytes
-    assert lib.ksmm_tilecopy_probe(x.data_ptr(), y.data_ptr(), batch * 4, a, 49, d, 4096, stream) == -2  # 49 rows of 4 KB
-    assert lib.ksmm_tilecopy_probe(x.data_ptr(), y.data_ptr(), batch * 4, a, rows, d, 48, stream) == -2  # not a power of two
-    out = torch.empty(lib.ksmm_mfma_probe_bytes(), dtype=torch.uint8, device="cuda")
+    assert lib.ksbench_tilecopy_probe(x.data_ptr(), y.data_ptr(), batch * 4, a, 49, d, 4096, stream) == -2  # 49 rows of 4 KB
+    assert lib.ksbench_tilecopy_probe(x.data_ptr(), y.data_ptr(), batch * 4, a, rows, d, 48, stream) == -2  # not a power of two
+    for wgs in (1, 7, 512):
+        y = torch.zeros_like(x)
+        _lib.check(lib.ksbench_stream_copy(x.data_ptr(), y.data_ptr(), x.numel() * 4, wgs, stream))
+        torch.cuda.synchronize()
+        assert torch.equal(x, y), wgs
+    assert lib.ksbench_stream_copy(x.data_ptr(), y.data_ptr(), 24, 8, stream) == -9  # not whole vectors
+    out = torch.empty(lib.ksbench_mfma_probe_bytes(), dtype=torch.uint8, device="cuda")
     flops = ctypes.c_double(0.0)
-    _lib.check(lib.ksmm_mfma_probe(dtype_code(torch.float16), 10, 1, out.data_ptr(), out.numel(), ctypes.byref(flops), stream))
+    _lib.check(lib.ksbench_mfma_probe(dtype_code(torch.float16), 10, 1, out.data_ptr(), out.numel(), ctypes.byref(flops), stream))
     torch.cuda.synchronize()
     assert flops.value == 16 * 2.0 * 32 * 32 * 16 * 10 * 256 * 8
 

@@ -108,6 +108,21 @@ def test_chain_argument_checks(lib):
     assert lib.ksmm_static_scratch_bytes() == 32 << 20
     assert lib.ksmm_chain_workspace_layout(d, 2, 1 << 20, 0, 0, 1) > lib.ksmm_static_scratch_bytes()
     assert lib.ksmm_chain_forward_static(d, 2, x, 1 << 40, 1 << 20, 0, 0, 1, 1, None, None) == -9
+    # chains that take the transposed (batch-size-first, strided blocks) or the padded-rows route
+    # (batch-size-last, batch off the vector) ask for more than ksmm_chain_workspace(): with less
+    # they are refused, like ksmm_factor_forward_ws, instead of falling back to a slow kernel
+    t = (_lib.KsmmFactorDesc * 1)()
+    t[0].w, t[0].w_dtype, t[0].scale = 4096, 1, 1.0
+    t[0].a, t[0].b, t[0].c, t[0].d = 1, 192, 192, 12
+    big = lib.ksmm_chain_workspace_layout(t, 1, 1024, 1, 1, 0)
+    assert big > 0 and lib.ksmm_chain_workspace(t, 1, 1024, 1) == 0
+    x2, y2, ws2 = 1 << 30, 2 << 30, 3 << 30
+    assert lib.ksmm_chain_forward(t, 1, x2, y2, None, 0, 1024, 1, 1, 0, 1, None) == -9
+    assert lib.ksmm_chain_forward(t, 1, x2, y2, ws2, big - 256, 1024, 1, 1, 0, 1, None) == -9
+    t[0].a, t[0].b, t[0].c, t[0].d = 1, 48, 48, 16
+    pad = lib.ksmm_chain_workspace_layout(t, 1, 1003, 1, 1, 1)
+    assert pad > 0
+    assert lib.ksmm_chain_forward(t, 1, x2, y2, ws2, pad - 256, 1003, 1, 1, 1, 1, None) == -9
     d[1].c = 5  # 3*5*2 = 30 != 24
     assert lib.ksmm_chain_forward(d, 2, x, y, ws, need, 100, 0, 0, 1, 1, None) == -8
     assert lib.ksmm_chain_forward(d, 17, x, y, ws, need, 100, 0, 0, 1, 1, None) == -10

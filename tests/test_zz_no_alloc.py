@@ -77,11 +77,14 @@ def test_static_scratch_entry_point_matches_the_workspace_one(case):
         print("no-alloc case", patterns, prec, bs_last, batch, "workspace", need, flush=True)
         _lib.check(lib.ksmm_chain_forward_ep(d, len(patterns), xin.data_ptr(), y_ref.data_ptr(), ws.data_ptr(), need,
                                              batch, xd, yd, int(bs_last), fuse, ctypes.byref(ep), stream))
+        torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
+        free_before = torch.cuda.mem_get_info()[0]  # device memory: a hipMalloc in the library would show here
         _lib.check(lib.ksmm_chain_forward_static(d, len(patterns), xin.data_ptr(), y_sta.data_ptr(), batch, xd, yd,
                                                  int(bs_last), fuse, ctypes.byref(ep), stream))
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before
         # same kernels on the same inputs: bit-identical
         assert torch.equal(y_ref.view(torch.uint8), y_sta.view(torch.uint8)), (patterns, prec, batch)
     # a chain whose intermediates exceed the fixed array is refused, not truncated
