@@ -242,6 +242,51 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
     return result
 
 
+def bench_backward(name, pattern, prec, bs_last, steps, warmup):
+    """µs of the input gradient (dX = K^T dY, on the forward kernels with transposed blocks) and of
+    the weight gradient (dW = sum over the batch of dY x X^T per block, per-split partial sums added
+    in a fixed order) of one factor at B = 25 088, each against its own roofline: both move the two
+    batch-sized operands once and do the forward's 2*B*a*b*c*d flops."""
+    from ksmm_amd import Kernel, generate_factor, _lib
+    from ksmm_amd.kernel import dtype_code
+    from ksmm_amd.roofline import HBM_PEAK_GBS, MFMA_PEAK_TFLOPS
+
+    HBM_BW = HBM_PEAK_GBS * 1e9
+    peak = MFMA_PEAK_TFLOPS[prec] * 1e12
+
+    a, b, c, d = pattern
+    dt = DT[prec]
+    es = torch.empty(0, dtype=dt).element_size()
+    gen = torch.Generator().manual_seed(SEED + 7)
+    (w4,) = make_weights([pattern], None, gen)
+    fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+    n_sets = max(2, min(8, int(math.ceil(1.2e9 / (2 * max(a * c * d, a * b * d) * BATCH * 4)))))
+    shape_x = (a * c * d, BATCH) if bs_last else (BATCH, a * c * d)
+    shape_y = (a * b * d, BATCH) if bs_last else (BATCH, a * b * d)
+    xs = [torch.randn(shape_x, generator=gen).to(dt).cuda() for _ in range(n_sets)]
+    dys = [torch.randn(shape_y, generator=gen).to(dt).cuda() for _ in range(n_sets)]
+    lib = _lib.load()
+    need = lib.ksmm_factor_backward_workspace(BATCH, a, b, c, d, dtype_code(dt), int(bs_last))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    nnz = a * b * c * d
+    flops = 2.0 * BATCH * nnz
+    nbytes = BATCH * (a * c * d + a * b * d) * es + nnz * es
+    floor = max(nbytes / HBM_BW, flops / peak)
+    out = {"name": name, "pattern": pattern, "precision": prec, "bs_last": bs_last, "workspace_bytes": int(need),
+           "bytes": nbytes, "flops": flops, "floor_us": floor * 1e6,
+           "bound": "hbm" if nbytes / HBM_BW >= flops / peak else "mfma"}
+    for key, kw in (("dx", {"need_weight": False}), ("dw", {"need_input": False})):
+        def run(j):
+            Kernel.backward(dys[j], xs[j], fac, bs_last, a, b, c, d, workspace=ws, **kw)
+
+        sec = time_launches(run, n_sets, steps, warmup)
+        out[key + "_us"] = sec * 1e6
+        out[key + "_roofline_frac"] = floor / sec
+        out[key + "_gbs"] = nbytes / sec / 1e9
+        out[key + "_tflops"] = flops / sec / 1e12
+    return out
+
+
 def copy_reference(steps, warmup):
     """Plain elementwise stream (y = x + 1) over the headline workload's bytes (77 MB in, 77 MB out) with
     the same buffer rotation and timing: what this particular GPU sustains for the simplest
@@ -356,10 +401,12 @@ def mfma_reference():
     return res
 
 
-def cpu_baseline(patterns, bs_last, budget_s=12.0, min_run_time=0.25):
-    """The reference's algo='bmm' CPU algorithm (restated in oracle/), fp32, on all host
-    cores; protocol of the reference's ksmm_time.py: blocked_autorange(min_run_time=0.25),
-    re-run with 11*max(mean, median) when fewer than 10 runs fit."""
+def cpu_baseline(patterns, bs_last, budget_s=12.0, min_run_time=0.25, dtype=torch.float32, batch=BATCH, bound=None):
+    """The reference's algo='bmm' CPU algorithm (restated in oracle/) on all host cores;
+    protocol of the reference's ksmm_time.py: blocked_autorange(min_run_time=0.25), re-run with
+    11*max(mean, median) when fewer than 10 runs fit.  ``dtype``: the type torch.bmm runs in
+    (fp16 is what the reference's CPU path does for dtype=float16); ``batch`` below the full
+    25 088 columns bounds the slow fp16 leg (columns are independent: time scales with them)."""
     import torch.utils.benchmark as tb
     from oracle import ks_oracle as O
 
@@ -367,10 +414,10 @@ def cpu_baseline(patterns, bs_last, budget_s=12.0, min_run_time=0.25):
     cores = min(cores, os.cpu_count() or cores)
     torch.set_num_threads(cores)
     gen = torch.Generator().manual_seed(SEED)
-    ws4 = make_weights(patterns, None, gen)
-    wb = [torch.from_numpy(O.pack_bmm_format(w.numpy())) for w in ws4]
+    ws4 = make_weights(patterns, bound, gen)
+    wb = [torch.from_numpy(O.pack_bmm_format(w.numpy())).to(dtype) for w in ws4]
     in_size = patterns[0][0] * patterns[0][2] * patterns[0][3]
-    x = torch.randn(BATCH, in_size, generator=gen)
+    x = torch.randn(batch, in_size, generator=gen).to(dtype)
     x = x.t().contiguous() if bs_last else x
     with torch.no_grad():
         timer = tb.Timer(stmt="f(wb, x, patterns, bs_last)",
@@ -379,9 +426,20 @@ def cpu_baseline(patterns, bs_last, budget_s=12.0, min_run_time=0.25):
         m = timer.blocked_autorange(min_run_time=min_run_time)
         if m.number_per_run <= 10:
             m = timer.blocked_autorange(min_run_time=min(budget_s, 11 * max(m.mean, m.median)))
+        calls = len(m.times) * m.number_per_run
+        if len(m.times) < 5 and m.median * m.number_per_run * 5 <= budget_s:
+            # blocked_autorange may return one block: time a few more of the same size so that the
+            # spread over blocks (iqr) is a spread
+            per_block = m.number_per_run
+            blocks = [timer.timeit(per_block) for _ in range(5)]
+            m = tb.Measurement.merge(blocks)[0]  # (times become per-call means of each block)
+            calls = 5 * per_block
+    name = str(dtype).replace("torch.", "")
     return {"value": m.median * 1e6, "unit": "us", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "full workload (B=%d, fp32, bs_last=%s, patterns=%s), %d timed calls of torch.bmm "
-                      "+ permute copies; median" % (BATCH, bs_last, patterns, len(m.times) * m.number_per_run),
+            "sample": "%s (B=%d of %d, %s, bs_last=%s, patterns=%s), %d timed calls of torch.bmm "
+                      "+ permute copies in %d blocks; median of the blocks"
+                      % ("full workload" if batch == BATCH else "a share of the batch columns", batch, BATCH, name,
+                         bs_last, patterns, calls, len(m.times)),
             "mean_us": m.mean * 1e6, "iqr_us": m.iqr * 1e6, "host_cpu_count": os.cpu_count()}
 
 
@@ -419,6 +477,9 @@ def main():
     ap.add_argument("--cpu", type=int, default=1, help="time the CPU baseline")
     ap.add_argument("--copy-calib", type=int, default=0,
                     help="also run N plain device copies of 77 MB (counter calibration for profiling runs)")
+    ap.add_argument("--backward", type=int, default=1,
+                    help="also time the backward pass (input and weight gradients) of the headline factor and of "
+                         "the ViT-B up-projection factors")
     ap.add_argument("--factor", default=None,
                     help="time one factor only, e.g. fp16:last:1,768,192,16 (per-kernel profiling runs); "
                          "prints that configuration's JSON instead of the headline line")
@@ -462,14 +523,28 @@ def main():
     stream_ref = stream_copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     tiled_ref = tiled_copy_reference(max(20, args.steps // 2), max(5, args.warmup // 2))
     mfma_ref = mfma_reference()
+    backward = []
+    if args.backward:
+        bsteps, bwarm = max(10, args.steps // 4), max(3, args.warmup // 4)
+        backward.append(bench_backward("C2_bs_last", (1, 48, 48, 16), "fp32", True, bsteps, bwarm))
+        backward.append(bench_backward("C4_vit_b_up_f0", (12, 64, 64, 1), "fp16", False, bsteps, bwarm))
+        backward.append(bench_backward("C4_vit_b_up_f1", (1, 1536, 384, 2), "fp16", False, bsteps, bwarm))
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
     if args.cpu:
         # the same CPU algorithm beside every other configuration (fp32 on the host, whatever the
         # device precision; a short sample each so that the whole run stays within minutes)
         head["cpu_bmm_us"], head["cpu_cores"] = cpu["value"], cpu["cores"]
         for cfg, res in zip(CONFIGS[1:], others):
-            c = cpu_baseline(cfg[1], cfg[3], budget_s=4.0, min_run_time=0.1)
+            c = cpu_baseline(cfg[1], cfg[3], budget_s=4.0, min_run_time=0.1, bound=cfg[4])
             res["cpu_bmm_us"], res["cpu_cores"], res["cpu_sample"] = c["value"], c["cores"], c["sample"]
+            if cfg[2] == "fp16":
+                # the reference's CPU path in the configuration's own type: torch.bmm in fp16, on an
+                # eighth of the batch columns (slow on the host; the time is per call of that share)
+                share = BATCH // 8
+                h = cpu_baseline(cfg[1], cfg[3], budget_s=3.0, min_run_time=0.1, dtype=torch.float16, batch=share)
+                res["cpu_bmm_fp16_us_share"], res["cpu_bmm_fp16_share_columns"] = h["value"], share
+                res["cpu_bmm_fp16_us_scaled_to_full_batch"] = h["value"] * (BATCH / share)
+                res["cpu_fp16_sample"] = h["sample"]
     line = {
         "metric": "us_per_ks_factor", "value": head["factors"][0]["us"], "unit": "us",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
@@ -487,6 +562,7 @@ def main():
         "parity": {"rel_fro_error": head.get("rel_fro_error"), "tolerance": head.get("tolerance"),
                    "ok": head.get("parity_ok")},
         "configs": [head] + others,
+        "backward": backward,
         "wall_s": time.time() - t_start,
     }
     print(json.dumps(line))

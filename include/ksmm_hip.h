@@ -235,8 +235,10 @@ int ksmm_chain_forward_ep(const ksmm_factor_desc *factors, int n_factors, const 
  *   ksmm_factor_backward_weight:  dw[a_i,b_i,c_i,d_i] = scale * sum_n dy[a_i,b_i,d_i,n] x[a_i,c_i,d_i,n],
  *                                 written in kernel format (a*d*c, b) like w.
  * dy has y's shape and layout, dx has x's.  Both need ksmm_factor_backward_workspace() bytes of
- * 16-byte aligned device memory (transposed blocks, an fp32 accumulator for the reduction over
- * the batch, and the forward kernels' own workspace for the transposed factor). */
+ * 16-byte aligned device memory (transposed blocks, fp32 partial sums of the reduction over the
+ * batch, one slice per batch split, and the forward kernels' own workspace for the transposed
+ * factor).  The weight gradient adds its partial sums in a fixed order: two calls on the same
+ * inputs give the same bits. */
 int64_t ksmm_factor_backward_workspace(int64_t batch, int a, int b, int c, int d, int dtype,
                                        int bs_last);
 int ksmm_factor_backward_input(const void *dy, const void *w, void *dx, int64_t batch, int a, int b,

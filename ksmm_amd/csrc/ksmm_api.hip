@@ -273,6 +273,27 @@ bool wants_padded(const Problem &p)
 
 int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
+// Bytes of the weight gradient's partial sums (at the batch as given and at the padded batch of the
+// transposed copies: whichever is larger)
+int64_t wgrad_partial_bytes(int64_t batch, int a, int b, int c, int d, int dtype)
+{
+    const int64_t p0 = wgrad_partial_floats(batch, a, b, c, d, dtype);
+    const int64_t p1 = wgrad_partial_floats(padded_batch(batch), a, b, c, d, dtype);
+    return align256((p0 > p1 ? p0 : p1) * 4);
+}
+
+// Bytes of the transposed copies of dY and X a batch-size-first weight gradient reduces (0: the
+// problem is batch-size-last, or its padded copies would pass the size limit and the tiled
+// kernel takes it as it is).
+int64_t wgrad_transposed_bytes(int64_t batch, int a, int b, int c, int d, int dtype, int bs_last)
+{
+    if (bs_last) return 0;
+    const int64_t bp = padded_batch(batch);
+    if (check_shape(bp, a, b, c, d, dtype, dtype, dtype) != KSMM_OK) return 0;
+    const int64_t es = (int64_t)dtype_size(dtype);
+    return align256((int64_t)a * b * d * bp * es) + align256((int64_t)a * c * d * bp * es);
+}
+
 bool overlaps(const void *p, int64_t p_bytes, const void *q, int64_t q_bytes)
 {
     const char *pb = (const char *)p, *qb = (const char *)q;
@@ -716,11 +737,12 @@ int64_t ksmm_factor_backward_workspace(int64_t batch, int a, int b, int c, int d
     if (rc != KSMM_OK) return rc;
     if (dtype != KSMM_F32 && dtype != KSMM_F16) return KSMM_ERR_BAD_DTYPE;
     const int64_t nnz = (int64_t)a * b * c * d;
-    // transposed blocks (input gradient) | fp32 accumulator (weight gradient) | what the forward
-    // kernels of the transposed factor ask for
+    // transposed blocks (input gradient) | fp32 partial sums, one slice per batch split (weight
+    // gradient) | what the forward kernels of the transposed factor ask for
     const int64_t fwd = ksmm_factor_workspace(batch, a, c, b, d, dtype, dtype, dtype, bs_last);
     if (fwd < 0) return fwd;
-    return align256(nnz * (int64_t)dtype_size(dtype)) + align256(nnz * 4) + fwd;
+    return align256(nnz * (int64_t)dtype_size(dtype)) + wgrad_partial_bytes(batch, a, b, c, d, dtype) + align256(fwd) +
+           wgrad_transposed_bytes(batch, a, b, c, d, dtype, bs_last);
 }
 
 int ksmm_factor_backward_input(const void *dy, const void *w, void *dx, int64_t batch, int a, int b,
@@ -733,7 +755,7 @@ int ksmm_factor_backward_input(const void *dy, const void *w, void *dx, int64_t 
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
     const int64_t nnz = (int64_t)a * b * c * d;
     char *wt = (char *)workspace;
-    char *fwd_ws = wt + align256(nnz * (int64_t)dtype_size(dtype)) + align256(nnz * 4);
+    char *fwd_ws = wt + align256(nnz * (int64_t)dtype_size(dtype)) + wgrad_partial_bytes(batch, a, b, c, d, dtype);
     int rc = block_transpose_run(w, wt, a, b, c, d, dtype, (hipStream_t)stream);
     if (rc != KSMM_OK) return rc;
     // dX = K^T dY: the factor with pattern (a, c, b, d) and transposed blocks
@@ -751,6 +773,21 @@ int ksmm_factor_backward_weight(const void *dy, const void *x, void *dw, int64_t
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return KSMM_ERR_WORKSPACE;
     const int64_t nnz = (int64_t)a * b * c * d;
     float *acc = (float *)((char *)workspace + align256(nnz * (int64_t)dtype_size(dtype)));
+    if (!bs_last && wgrad_transposed_bytes(batch, a, b, c, d, dtype, 0) > 0) {
+        // Batch-size-first: the operands of one block are d elements apart along the features, and
+        // the sum runs over the rows.  Both operands are transposed once into the workspace (rows
+        // padded to 16 columns, the padding cleared) and the batch-size-last kernel reduces them.
+        const int64_t es = (int64_t)dtype_size(dtype), bp = padded_batch(batch);
+        const int64_t fwd = ksmm_factor_workspace(batch, a, c, b, d, dtype, dtype, dtype, 0);
+        char *tdy = (char *)acc + wgrad_partial_bytes(batch, a, b, c, d, dtype) + align256(fwd);
+        char *tx = tdy + align256((int64_t)a * b * d * bp * es);
+        int rc = transpose_run(dy, tdy, batch, (int64_t)a * b * d, (int)es, (hipStream_t)stream, 0, bp);
+        if (rc == KSMM_OK) rc = zero_pad_run(tdy, (int64_t)a * b * d, batch, bp, (int)es, (hipStream_t)stream);
+        if (rc == KSMM_OK) rc = transpose_run(x, tx, batch, (int64_t)a * c * d, (int)es, (hipStream_t)stream, 0, bp);
+        if (rc == KSMM_OK) rc = zero_pad_run(tx, (int64_t)a * c * d, batch, bp, (int)es, (hipStream_t)stream);
+        if (rc != KSMM_OK) return rc;
+        return wgrad_run(tdy, tx, dw, acc, bp, a, b, c, d, dtype, 1, scale, (hipStream_t)stream, nullptr);
+    }
     return wgrad_run(dy, x, dw, acc, batch, a, b, c, d, dtype, bs_last ? 1 : 0, scale, (hipStream_t)stream, nullptr);
 }
 

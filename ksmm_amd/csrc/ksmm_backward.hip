@@ -6,9 +6,10 @@
 //                 one (b x B) @ (B x c) product per (a_i, d_i) block, reduced over the batch:
 //                 MFMA kernel for batch-size-last (operand rows are batch-contiguous, so both
 //                 operands come straight from global memory in MFMA layout, no LDS), an
-//                 LDS-tiled FMA kernel for everything else; partial sums over batch splits are
-//                 accumulated with fp32 atomics in a workspace and then scaled, converted and
-//                 written in kernel format (a*d*c, b).
+//                 LDS-tiled FMA kernel for everything else; every batch split writes its partial
+//                 sums to a slice of its own in the workspace, and a finish kernel adds the slices
+//                 in a fixed order, scales, converts and writes kernel format (a*d*c, b): the
+//                 result is the same bit for bit from run to run (no atomics).
 //
 // The reference has no backward pass (src/ksmm_py/layer/kronecker_sparse/kernel.py:319-329 refers
 // to an undefined symbol; forward_bmm.py:12-15 is `pass`); the definition above is the adjoint of
@@ -33,18 +34,16 @@ __global__ __launch_bounds__(256) void ks_block_transpose_kernel(const T *__rest
     out[i] = in[(g * c + ci) * b + bi];
 }
 
-__global__ __launch_bounds__(256) void ks_fill_zero_kernel(float *__restrict__ p, int64_t n)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0.f;
-}
-
+// dw[i] = scale * (slice 0 + slice 1 + ... in that order); slices are n floats apart
 template <typename T>
 __global__ __launch_bounds__(256) void ks_wgrad_finish_kernel(const float *__restrict__ acc, T *__restrict__ dw,
-                                                              int64_t n, float scale)
+                                                              int64_t n, int splits, float scale)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) dw[i] = (T)(acc[i] * scale);
+    if (i >= n) return;
+    float s = acc[i];
+    for (int k = 1; k < splits; ++k) s += acc[(int64_t)k * n + i];
+    dw[i] = (T)(s * scale);
 }
 
 template <typename T> struct wg_vec;
@@ -76,7 +75,7 @@ template <typename T, int MT, int NT>
 __global__ __launch_bounds__(256) void ks_wgrad_bl_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                           float *__restrict__ acc_out, int batch, int a, int b,
                                                           int c, int d, int m_tiles, int n_tiles, int splits,
-                                                          int cols_per_split)
+                                                          int cols_per_split, int64_t slice)
 {
     typedef wg_vec<T> V;
     constexpr int STEP = 4 * V::N;  // batch columns per step (4 lane groups)
@@ -144,7 +143,7 @@ __global__ __launch_bounds__(256) void ks_wgrad_bl_kernel(const T *__restrict__ 
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int m = m0 + 16 * i + 4 * q + e;
-                if (m < b) atomicAdd(acc_out + ((size_t)g * c + cc) * b + m, acc[i][j][e]);
+                if (m < b) acc_out[(size_t)split * slice + ((size_t)g * c + cc) * b + m] = acc[i][j][e];
             }
         }
 }
@@ -155,7 +154,7 @@ template <typename T, bool BS_LAST>
 __global__ __launch_bounds__(256) void ks_wgrad_tiled_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                              float *__restrict__ acc_out, int64_t batch, int a,
                                                              int b, int c, int d, int m_tiles, int n_tiles,
-                                                             int splits, int64_t cols_per_split)
+                                                             int splits, int64_t cols_per_split, int64_t slice)
 {
     __shared__ float sa[16][17], sb[16][17];
     int64_t t = blockIdx.x;
@@ -191,7 +190,7 @@ __global__ __launch_bounds__(256) void ks_wgrad_tiled_kernel(const T *__restrict
         __syncthreads();
     }
     const int m = mt * 16 + tx, cc = nt * 16 + ty;  // consecutive threads: consecutive b_i (contiguous in dW)
-    if (m < b && cc < c) atomicAdd(acc_out + ((size_t)g * c + cc) * b + m, acc);
+    if (m < b && cc < c) acc_out[(size_t)split * slice + ((size_t)g * c + cc) * b + m] = acc;
 }
 
 template <typename T> int launch_block_transpose(const void *w, void *wt, int64_t total, int b, int c, hipStream_t s)
@@ -203,49 +202,82 @@ template <typename T> int launch_block_transpose(const void *w, void *wt, int64_
     return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
-template <typename T, int MT, int NT>
-int launch_wgrad_bl(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
-                    hipStream_t s)
+// Batch splits of the two weight-gradient kernels (every split is non-empty and writes a slice of
+// a*b*c*d partial sums of its own): columns per split and their number.
+void wgrad_bl_splits(int64_t batch, int64_t tiles, int step, int64_t *splits_out, int64_t *cols_out)
 {
-    const int m_tiles = (b + 16 * MT - 1) / (16 * MT), n_tiles = (c + 16 * NT - 1) / (16 * NT);
-    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
-    constexpr int STEP = 4 * wg_vec<T>::N;
     // about 16 waves per CU; at least 8 steps per wave
     int64_t splits = (4096 + tiles - 1) / tiles;
-    const int64_t max_splits = (batch + 8 * STEP - 1) / (8 * STEP);
+    const int64_t max_splits = (batch + 8 * step - 1) / (8 * step);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     int64_t cols = (batch + splits - 1) / splits;
-    cols = (cols + STEP - 1) / STEP * STEP;
-    splits = (batch + cols - 1) / cols;
-    const int64_t waves = tiles * splits, blocks = (waves + 3) / 4;
-    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((ks_wgrad_bl_kernel<T, MT, NT>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
-                       (const T *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols);
-    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+    cols = (cols + step - 1) / step * step;
+    *splits_out = (batch + cols - 1) / cols;
+    *cols_out = cols;
 }
 
-template <typename T>
-int launch_wgrad_tiled(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
-                       int bs_last, hipStream_t s)
+void wgrad_tiled_splits(int64_t batch, int64_t tiles, int64_t *splits_out, int64_t *cols_out)
 {
-    const int m_tiles = (b + 15) / 16, n_tiles = (c + 15) / 16;
-    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
     int64_t splits = (2048 + tiles - 1) / tiles;
     const int64_t max_splits = (batch + 255) / 256;
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     int64_t cols = (batch + splits - 1) / splits;
     cols = (cols + 15) / 16 * 16;
-    splits = (batch + cols - 1) / cols;
+    *splits_out = (batch + cols - 1) / cols;
+    *cols_out = cols;
+}
+
+// tile of the MFMA kernel for a block shape: 16 * t rows and columns
+int wgrad_bl_tile(int b, int c)
+{
+    return (b <= 16 && c <= 16) ? 1 : (b <= 32 && c <= 32) ? 2 : (b % 64 && c % 64 && b % 48 == 0 && c % 48 == 0) ? 3 : 4;
+}
+
+bool wgrad_mfma_ok(const void *dy, const void *x, int64_t batch, int b, int c, int d, int dtype, int bs_last)
+{
+    const int vec = 16 / (int)dtype_size(dtype);
+    return bs_last && batch % vec == 0 && ((((uintptr_t)dy | (uintptr_t)x) & 15) == 0) &&
+           (int64_t)(b > c ? b : c) * d * batch < 0x7fffffffLL;
+}
+
+template <typename T, int MT, int NT>
+int launch_wgrad_bl(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
+                    hipStream_t s, int *splits_used)
+{
+    const int m_tiles = (b + 16 * MT - 1) / (16 * MT), n_tiles = (c + 16 * NT - 1) / (16 * NT);
+    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
+    constexpr int STEP = 4 * wg_vec<T>::N;
+    int64_t splits, cols;
+    wgrad_bl_splits(batch, tiles, STEP, &splits, &cols);
+    const int64_t waves = tiles * splits, blocks = (waves + 3) / 4;
+    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    *splits_used = (int)splits;
+    hipLaunchKernelGGL((ks_wgrad_bl_kernel<T, MT, NT>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
+                       (const T *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols,
+                       (int64_t)a * b * c * d);
+    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_wgrad_tiled(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
+                       int bs_last, hipStream_t s, int *splits_used)
+{
+    const int m_tiles = (b + 15) / 16, n_tiles = (c + 15) / 16;
+    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
+    int64_t splits, cols;
+    wgrad_tiled_splits(batch, tiles, &splits, &cols);
     const int64_t blocks = tiles * splits;
     if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    *splits_used = (int)splits;
+    const int64_t slice = (int64_t)a * b * c * d;
     if (bs_last)
         hipLaunchKernelGGL((ks_wgrad_tiled_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
-                           (const T *)x, acc, batch, a, b, c, d, m_tiles, n_tiles, (int)splits, cols);
+                           (const T *)x, acc, batch, a, b, c, d, m_tiles, n_tiles, (int)splits, cols, slice);
     else
         hipLaunchKernelGGL((ks_wgrad_tiled_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
-                           (const T *)x, acc, batch, a, b, c, d, m_tiles, n_tiles, (int)splits, cols);
+                           (const T *)x, acc, batch, a, b, c, d, m_tiles, n_tiles, (int)splits, cols, slice);
     return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
@@ -263,47 +295,60 @@ int block_transpose_run(const void *w, void *wt, int a, int b, int c, int d, int
     }
 }
 
+// Floats of partial sums the weight gradient of this problem writes (slices of a*b*c*d, one per
+// batch split), whichever kernel takes it: the larger of the two kernels' needs, so that the
+// answer does not depend on pointer alignment.
+int64_t wgrad_partial_floats(int64_t batch, int a, int b, int c, int d, int dtype)
+{
+    const int64_t n = (int64_t)a * b * c * d;
+    int64_t splits, cols, most = 1;
+    const int t = wgrad_bl_tile(b, c);
+    const int64_t tiles_bl = (int64_t)a * d * ((b + 16 * t - 1) / (16 * t)) * ((c + 16 * t - 1) / (16 * t));
+    wgrad_bl_splits(batch, tiles_bl, 4 * (16 / (int)dtype_size(dtype)), &splits, &cols);
+    if (splits > most) most = splits;
+    wgrad_tiled_splits(batch, (int64_t)a * d * ((b + 15) / 16) * ((c + 15) / 16), &splits, &cols);
+    if (splits > most) most = splits;
+    return most * n;
+}
+
 // dw (kernel format, type `dtype`) <- scale * sum over the batch of dY x X^T per block; acc is an
-// fp32 buffer of a*b*c*d elements (zeroed here).  tile_query: 1 = MFMA kernel, 0 = tiled kernel.
+// fp32 buffer of wgrad_partial_floats() elements.  kernel_used: 1 = MFMA kernel, 0 = tiled kernel.
 int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch, int a, int b, int c, int d,
               int dtype, int bs_last, float scale, hipStream_t stream, int *kernel_used)
 {
     const int64_t n = (int64_t)a * b * c * d;
-    const int64_t fill_blocks = (n + 255) / 256;
-    if (fill_blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
-    const int vec = 16 / (int)dtype_size(dtype);
-    const bool mfma_ok = bs_last && batch % vec == 0 && ((((uintptr_t)dy | (uintptr_t)x) & 15) == 0) &&
-                         (int64_t)(b > c ? b : c) * d * batch < 0x7fffffffLL;
+    const int64_t fin_blocks = (n + 255) / 256;
+    if (fin_blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    const bool mfma_ok = wgrad_mfma_ok(dy, x, batch, b, c, d, dtype, bs_last);
     if (kernel_used) *kernel_used = mfma_ok ? 1 : 0;
-    hipLaunchKernelGGL(ks_fill_zero_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, stream, acc, n);
-    if (hipGetLastError() != hipSuccess) return KSMM_ERR_LAUNCH;
-    int rc;
+    const int t = wgrad_bl_tile(b, c);
+    int rc, splits = 1;
     if (dtype == KSMM_F32) {
         if (mfma_ok)
-            rc = (b <= 16 && c <= 16) ? launch_wgrad_bl<float, 1, 1>(dy, x, acc, batch, a, b, c, d, stream)
-                 : (b <= 32 && c <= 32) ? launch_wgrad_bl<float, 2, 2>(dy, x, acc, batch, a, b, c, d, stream)
-                 : (b % 64 && c % 64 && b % 48 == 0 && c % 48 == 0) ? launch_wgrad_bl<float, 3, 3>(dy, x, acc, batch, a, b, c, d, stream)
-                                                                    : launch_wgrad_bl<float, 4, 4>(dy, x, acc, batch, a, b, c, d, stream);
+            rc = t == 1   ? launch_wgrad_bl<float, 1, 1>(dy, x, acc, batch, a, b, c, d, stream, &splits)
+                 : t == 2 ? launch_wgrad_bl<float, 2, 2>(dy, x, acc, batch, a, b, c, d, stream, &splits)
+                 : t == 3 ? launch_wgrad_bl<float, 3, 3>(dy, x, acc, batch, a, b, c, d, stream, &splits)
+                          : launch_wgrad_bl<float, 4, 4>(dy, x, acc, batch, a, b, c, d, stream, &splits);
         else
-            rc = launch_wgrad_tiled<float>(dy, x, acc, batch, a, b, c, d, bs_last, stream);
+            rc = launch_wgrad_tiled<float>(dy, x, acc, batch, a, b, c, d, bs_last, stream, &splits);
     } else if (dtype == KSMM_F16) {
         if (mfma_ok)
-            rc = (b <= 16 && c <= 16) ? launch_wgrad_bl<half_t, 1, 1>(dy, x, acc, batch, a, b, c, d, stream)
-                 : (b <= 32 && c <= 32) ? launch_wgrad_bl<half_t, 2, 2>(dy, x, acc, batch, a, b, c, d, stream)
-                 : (b % 64 && c % 64 && b % 48 == 0 && c % 48 == 0) ? launch_wgrad_bl<half_t, 3, 3>(dy, x, acc, batch, a, b, c, d, stream)
-                                                                    : launch_wgrad_bl<half_t, 4, 4>(dy, x, acc, batch, a, b, c, d, stream);
+            rc = t == 1   ? launch_wgrad_bl<half_t, 1, 1>(dy, x, acc, batch, a, b, c, d, stream, &splits)
+                 : t == 2 ? launch_wgrad_bl<half_t, 2, 2>(dy, x, acc, batch, a, b, c, d, stream, &splits)
+                 : t == 3 ? launch_wgrad_bl<half_t, 3, 3>(dy, x, acc, batch, a, b, c, d, stream, &splits)
+                          : launch_wgrad_bl<half_t, 4, 4>(dy, x, acc, batch, a, b, c, d, stream, &splits);
         else
-            rc = launch_wgrad_tiled<half_t>(dy, x, acc, batch, a, b, c, d, bs_last, stream);
+            rc = launch_wgrad_tiled<half_t>(dy, x, acc, batch, a, b, c, d, bs_last, stream, &splits);
     } else {
         return KSMM_ERR_BAD_DTYPE;
     }
     if (rc != KSMM_OK) return rc;
     if (dtype == KSMM_F32)
-        hipLaunchKernelGGL((ks_wgrad_finish_kernel<float>), dim3((unsigned)fill_blocks), dim3(256), 0, stream, acc,
-                           (float *)dw, n, scale);
+        hipLaunchKernelGGL((ks_wgrad_finish_kernel<float>), dim3((unsigned)fin_blocks), dim3(256), 0, stream, acc,
+                           (float *)dw, n, splits, scale);
     else
-        hipLaunchKernelGGL((ks_wgrad_finish_kernel<half_t>), dim3((unsigned)fill_blocks), dim3(256), 0, stream, acc,
-                           (half_t *)dw, n, scale);
+        hipLaunchKernelGGL((ks_wgrad_finish_kernel<half_t>), dim3((unsigned)fin_blocks), dim3(256), 0, stream, acc,
+                           (half_t *)dw, n, splits, scale);
     return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 

@@ -185,8 +185,10 @@ int gemm_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // p
 int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile);  // part of the tile family
 
 // Backward pass pieces (ksmm_backward.hip): blockwise transpose of a kernel-format weight, and the
-// weight gradient (acc: fp32 scratch of a*b*c*d elements; kernel_used: 1 MFMA kernel, 0 tiled).
+// weight gradient (acc: fp32 scratch of wgrad_partial_floats() elements, one slice of a*b*c*d per
+// batch split; kernel_used: 1 MFMA kernel, 0 tiled).
 int block_transpose_run(const void *w, void *wt, int a, int b, int c, int d, int dtype, hipStream_t stream);
+int64_t wgrad_partial_floats(int64_t batch, int a, int b, int c, int d, int dtype);
 int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch, int a, int b, int c, int d,
               int dtype, int bs_last, float scale, hipStream_t stream, int *kernel_used);
 
@@ -194,6 +196,8 @@ int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch
 // out (cols x rows) = transpose of in (rows x cols); pitches in elements per row, 0 = dense
 int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream,
                   int64_t in_pitch = 0, int64_t out_pitch = 0);
+// zeros in columns [cols, pitch) of every row of a (rows x pitch) matrix
+int zero_pad_run(void *p, int64_t rows, int64_t cols, int64_t pitch, int elem_bytes, hipStream_t stream);
 // out (rows x cols_out) = the rows of in (rows x cols_in) cut or zero-filled to cols_out columns
 int repitch_run(const void *in, void *out, int64_t rows, int64_t cols_in, int64_t cols_out, int elem_bytes,
                 hipStream_t stream);

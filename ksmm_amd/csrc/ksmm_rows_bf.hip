@@ -32,9 +32,11 @@ namespace {
 // conflicts whatever the padding); in planes those accesses are conflict-free, and so are
 // the four 4-byte stores / loads per 16-byte global vector that feed and drain them.
 constexpr int plane_floats(int n) { return n + (68 - n % 64) % 64; }
-template <int BB, int CC, int DD, int TN, bool PL = false> struct RowCfg {
-    static constexpr int NW = DD, THREADS = 64 * NW;
-    static constexpr int MT = BB / 16, KS = CC / 4, NT = TN / 16;
+// MS: waves per d_i, each holding BB / MS rows of the block (blocks whose weights do not fit the
+// registers of one wave)
+template <int BB, int CC, int DD, int TN, bool PL = false, int MS = 1> struct RowCfg {
+    static constexpr int NW = DD * MS, THREADS = 64 * NW;
+    static constexpr int MT = BB / 16 / MS, KS = CC / 4, NT = TN / 16;
     static constexpr int XROW = CC * DD, OROW = BB * DD;  // floats per row segment
     static constexpr int LDX = XROW + 4, LDO = OROW + 4;
     static constexpr int LDK = CC + 4, LDM = BB + 4;      // PL: rows of a plane
@@ -44,18 +46,18 @@ template <int BB, int CC, int DD, int TN, bool PL = false> struct RowCfg {
     static constexpr int X_PER_T = (X_VECS + THREADS - 1) / THREADS, O_PER_T = (O_VECS + THREADS - 1) / THREADS;
     static constexpr int LDS_BYTES = (2 * X_FLOATS + O_FLOATS) * 4;
     static_assert(!PL || DD % 4 == 0, "planes: a 16-byte vector is 4 d_i of one k");
-    static_assert(BB % 16 == 0 && CC % 4 == 0 && TN % 16 == 0, "MFMA tiling");
+    static_assert(BB % (16 * MS) == 0 && CC % 4 == 0 && TN % 16 == 0, "MFMA tiling");
     static_assert(NW <= 16 && XROW % 4 == 0 && OROW % 4 == 0, "shape");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-template <int BB, int CC, int DD, int TN, bool NT_STORE, bool PL = false>
-__global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__restrict__ x,
+template <int BB, int CC, int DD, int TN, bool NT_STORE, bool PL = false, int MS = 1>
+__global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a,
                                                             int d, Epi ep, int wgs_per_a, int n_tiles)
 {
-    typedef RowCfg<BB, CC, DD, TN, PL> C;
+    typedef RowCfg<BB, CC, DD, TN, PL, MS> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *const xs = (float *)smem;                // [2][TN][LDX]; PL: [2][DD][PLANE_X]
     float *const os = xs + 2 * C::X_FLOATS;         // [TN][LDO]; PL: [DD][PLANE_O]
@@ -67,24 +69,26 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
-    const int dd = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's d_i
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ms = wv / DD, dd = wv - ms * DD;  // this wave's row group and d_i
+    const int m_off = ms * (BB / MS);
     const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
 
     // weights of block (a_i, dd): element (k, m) at ((a_i*d + dd)*c + k)*b + m -> A operands
     float wreg[C::MT][C::KS];
     {
-        const float *wg = w + (size_t)(a_i * d + d0 + dd) * CC * BB;
+        const float *wg = w + (size_t)(a_i * d + d0 + dd) * CC * BB + m_off;
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
             for (int mt = 0; mt < C::MT; ++mt) wreg[mt][ks] = wg[(4 * ks + q) * BB + 16 * mt + r];
     }
-    float bv[C::MT][4];  // bias of the outputs this lane holds: m = 16*mt + 4*q + i of d_i = d0 + dd
+    float bv[C::MT][4];  // bias of the outputs this lane holds: m = m_off + 16*mt + 4*q + i of d_i = d0 + dd
 #pragma unroll
     for (int mt = 0; mt < C::MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * BB + 16 * mt + 4 * q + i) * d + d0 + dd);
+            bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * BB + m_off + 16 * mt + 4 * q + i) * d + d0 + dd);
 
     // element e of a tile row (e = k * DD + j) lives at k * d + j behind the group's origin
     const float *xg = x + (size_t)a_i * CC * d + d0;
@@ -152,8 +156,8 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_kernel(const float *__rest
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[PL ? dd * C::PLANE_O + (16 * nt + r) * C::LDM + 16 * mt + 4 * q + i
-                          : (16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
+                    os[PL ? dd * C::PLANE_O + (16 * nt + r) * C::LDM + m_off + 16 * mt + 4 * q + i
+                          : (16 * nt + r) * C::LDO + (m_off + 16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -343,11 +347,16 @@ struct RowInst {
     int nt;   // streaming (nontemporal) output stores
     const void *fn;
     int planes;  // fp32: LDS tiles split into one plane per d_i
+    int ms = 1;  // fp32: waves per d_i (row groups of a tall block)
 };
 #define ROW_INST_PL(BB_, CC_, DD_, TN_) \
     {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_, true>::LDS_BYTES, 4, 1, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, true, true>, 1}
 #define ROW_INST(BB_, CC_, DD_, TN_, NT_) \
     {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, 4, NT_, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, NT_>}
+ // two waves per d_i, each with half of the block's rows
+#define ROW_INST_MS(BB_, CC_, DD_, TN_, MS_) \
+    {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_, false, MS_>::LDS_BYTES, 4, 1, \
+     (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, true, false, MS_>, 0, MS_}
 #define ROW_INST_H(BB_, CC_, DD_, TN_)                                                                      \
     {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 8, 1,                          \
      (const void *)ks_rows_bf_h_kernel<half_t, BB_, CC_, DD_, TN_>}
@@ -369,6 +378,7 @@ struct RowInst {
     M(64, 64, 2, 16), M(64, 64, 3, 16), M(64, 64, 4, 16), M(64, 64, 6, 16), M(64, 64, 8, 16), \
     M(96, 96, 2, 16), M(96, 96, 3, 16), M(96, 96, 4, 16), M(192, 48, 2, 16), M(192, 48, 3, 16), \
     M(192, 48, 4, 16), M(48, 192, 3, 16), M(48, 192, 4, 16)
+#define ROW_SET_16C(M) M(128, 128, 3, 16), M(128, 128, 3, 32), M(16, 16, 4, 64), M(16, 16, 4, 128)
 const RowInst row_insts[] = {
     ROW_INST(48, 48, 16, 16, true), ROW_INST(48, 48, 8, 32, true), ROW_INST(48, 48, 4, 64, true),
     ROW_INST(64, 64, 8, 16, true),  ROW_INST(64, 64, 4, 32, true), ROW_INST(16, 16, 16, 32, true),
@@ -396,6 +406,13 @@ const RowInst row_insts[] = {
     ROW_INST_PL(48, 48, 4, 16), ROW_INST_PL(64, 64, 8, 16), ROW_INST_PL(64, 64, 4, 32), ROW_INST_PL(64, 64, 4, 16),
     ROW_INST_PL(16, 16, 16, 32), ROW_INST_PL(16, 16, 4, 128), ROW_INST_PL(32, 32, 8, 32), ROW_INST_PL(32, 32, 16, 16),
     ROW_INST_PL(96, 96, 4, 16), ROW_INST_PL(48, 192, 4, 16), ROW_INST_PL(192, 48, 4, 16),
+    // 16-bit: three 128 x 128 blocks per workgroup (the down factor (1,128,128,3) of the reference's
+    // ViT-S feed-forward, scripts/2_benchmark_ksvit_time.sh:48-50, in its default layout), and
+    // 16 x 16 blocks in groups of four
+    ROW_SET_16C(ROW_INST_H),
+    ROW_SET_16C(ROW_INST_Q),
+    // fp32 128 x 128 blocks: two waves per d_i
+    ROW_INST_MS(128, 128, 3, 16, 2),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 constexpr int ROW_INST_BITS = 10, ROW_INST_ANY = (1 << ROW_INST_BITS) - 1;
@@ -409,8 +426,8 @@ uint32_t rows_inst_id(int i)
 {
     if (i < 0 || i >= N_ROW_INSTS) return 0;
     const RowInst &t = row_insts[i];
-    const int v[7] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt, t.planes};
-    return inst_hash('R', v, t.planes ? 7 : 6);  // (ids of the other instances predate the field)
+    const int v[8] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt, t.planes, t.ms};
+    return inst_hash('R', v, t.ms > 1 ? 8 : t.planes ? 7 : 6);  // (ids of the other instances predate the fields)
 }
 
 // variant: bits 0-9 instance (all ones: first that fits), bits 10.. workgroups per a_i (0: heuristic)
@@ -455,7 +472,8 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
     const int64_t ag = (int64_t)p.a * (p.d / t.dd);  // (a_i, group) pairs
     // one round of workgroups, 8 or more waves per CU
-    const int per_cu_lds = 160 * 1024 / t.lds, per_cu_waves = 16 / t.dd > 0 ? 16 / t.dd : 1;
+    const int nw = t.dd * t.ms;
+    const int per_cu_lds = 160 * 1024 / t.lds, per_cu_waves = 16 / nw > 0 ? 16 / nw : 1;
     // (rounded down: a few workgroups beyond one round would cost a whole second round)
     if (wgs <= 0) wgs = 256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves) / ag;
     if (wgs <= 0) wgs = 1;
@@ -469,7 +487,7 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         tile->tile_n = t.tn;
         tile->tile_k = t.cc;
         tile->tile_d = t.dd;
-        tile->threads = 64 * t.dd;
+        tile->threads = 64 * nw;
         tile->lds_bytes = t.lds;
         tile->grid = grid;
     }
@@ -479,7 +497,7 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     Epi ep = epi_of(p);
     void *args[] = {(void *)&p.x, (void *)&p.w, (void *)&p.y, &batch_i, (void *)&p.a, (void *)&p.d,
                     &ep, &wgs_i, &n_tiles_i};
-    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(64 * t.dd), args, t.lds, p.stream);
+    hipError_t e = hipLaunchKernel(t.fn, dim3((unsigned)grid), dim3(64 * nw), args, t.lds, p.stream);
     return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 

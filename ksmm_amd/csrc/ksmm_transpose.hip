@@ -106,6 +106,19 @@ __global__ __launch_bounds__(256) void ks_transpose_kernel(const void *__restric
     }
 }
 
+// the padding of every row of a pitched matrix: element q of the padding is column cols + q % pad
+// of row q / pad
+template <int ES>
+__global__ __launch_bounds__(256) void ks_zero_pad_kernel(void *__restrict__ p_, int64_t total, int64_t pad, int64_t cols,
+                                                         int64_t pitch)
+{
+    typedef typename elem_of<ES>::type T;
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= total) return;
+    const int64_t row = q / pad;
+    ((T *)p_)[row * pitch + cols + (q - row * pad)] = 0;
+}
+
 template <int ES> const void *transpose_fn(bool vin, bool vout)
 {
     if (vin && vout) return (const void *)ks_transpose_kernel<ES, true, true>;
@@ -191,6 +204,19 @@ int repitch_run(const void *in, void *out, int64_t rows, int64_t cols_in, int64_
 
 // out (cols x rows, out_pitch elements per row) = transpose of in (rows x cols, in_pitch elements
 // per row); elem_bytes in {1, 2, 4}; a pitch of 0 means the dense one
+// zeros in columns [cols, pitch) of every row of a (rows x pitch) matrix of 1-, 2- or 4-byte elements
+int zero_pad_run(void *p, int64_t rows, int64_t cols, int64_t pitch, int elem_bytes, hipStream_t stream)
+{
+    if (pitch <= cols) return KSMM_OK;
+    const int64_t pad = pitch - cols, total = rows * pad;
+    if ((total + 255) / 256 > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    const void *fn = elem_bytes == 4 ? (const void *)ks_zero_pad_kernel<4>
+                                     : elem_bytes == 2 ? (const void *)ks_zero_pad_kernel<2> : (const void *)ks_zero_pad_kernel<1>;
+    void *args[] = {(void *)&p, (void *)&total, (void *)&pad, (void *)&cols, (void *)&pitch};
+    hipError_t e = hipLaunchKernel(fn, dim3((unsigned)((total + 255) / 256)), dim3(256), args, 0, stream);
+    return e == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
 int transpose_run(const void *in, void *out, int64_t rows, int64_t cols, int elem_bytes, hipStream_t stream,
                   int64_t in_pitch, int64_t out_pitch)
 {

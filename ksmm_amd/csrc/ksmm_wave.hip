@@ -40,13 +40,13 @@ template <> struct hvec<8> { typedef half8_t type; };
 template <typename TX, int VEC> struct row_io;
 template <int VEC> struct row_io<half_t, VEC> {
     static constexpr int RAW = VEC / 2;  // dwords per row load
-    __device__ static __forceinline__ void load(const half_t *p, uint32_t (&o)[RAW])
+    template <bool NT> __device__ static __forceinline__ void load(const half_t *p, uint32_t (&o)[RAW])
     {
         if constexpr (VEC == 8) {
-            uint4_t v = *(const uint4_t *)p;
+            uint4_t v = NT ? __builtin_nontemporal_load((const uint4_t *)p) : *(const uint4_t *)p;
             o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
         } else {
-            uint2_t v = *(const uint2_t *)p;
+            uint2_t v = NT ? __builtin_nontemporal_load((const uint2_t *)p) : *(const uint2_t *)p;
             o[0] = v[0]; o[1] = v[1];
         }
     }
@@ -58,13 +58,13 @@ template <int VEC> struct row_io<half_t, VEC> {
 };
 template <int VEC> struct row_io<fp8_t, VEC> {
     static constexpr int RAW = VEC / 4;
-    __device__ static __forceinline__ void load(const fp8_t *p, uint32_t (&o)[RAW])
+    template <bool NT> __device__ static __forceinline__ void load(const fp8_t *p, uint32_t (&o)[RAW])
     {
         if constexpr (VEC == 16) {
-            uint4_t v = *(const uint4_t *)p;
+            uint4_t v = NT ? __builtin_nontemporal_load((const uint4_t *)p) : *(const uint4_t *)p;
             o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
         } else {
-            uint2_t v = *(const uint2_t *)p;
+            uint2_t v = NT ? __builtin_nontemporal_load((const uint2_t *)p) : *(const uint2_t *)p;
             o[0] = v[0]; o[1] = v[1];
         }
     }
@@ -286,12 +286,18 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
     }
 }
 
-__device__ __forceinline__ void ring_dma16(const void *sbase, uint32_t voff, uint32_t lds_addr)
+template <bool NT> __device__ __forceinline__ void ring_dma16(const void *sbase, uint32_t voff, uint32_t lds_addr)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(voff), "s"(sbase), "s"(lds_addr)
-                 : "memory", "m0");
+    if constexpr (NT)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                     :
+                     : "v"(voff), "s"(sbase), "s"(lds_addr)
+                     : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(voff), "s"(sbase), "s"(lds_addr)
+                     : "memory", "m0");
 }
 
 // the lane's own 16 bytes of a slot, complete when the function returns
@@ -302,7 +308,7 @@ template <int OFF> __device__ __forceinline__ float4_t ring_read16(uint32_t lds_
     return v;
 }
 
-template <int MT, int KS, bool DEFER, bool EPI>
+template <int MT, int KS, bool DEFER, bool NT, bool EPI>
 __global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a, int b,
@@ -366,7 +372,7 @@ __global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restri
     {
         const uint32_t off = x_lane + col_off(0);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) ring_dma16(xg + ks * x_step, off, lds_wave + ks * 1024);
+        for (int ks = 0; ks < KS; ++ks) ring_dma16<NT>(xg + ks * x_step, off, lds_wave + ks * 1024);
     }
     auto store_one = [&](const float4_t(&acc)[MT][VEC], int s, uint32_t off) {
         const int mt = s >> 2, i = s & 3;
@@ -376,7 +382,11 @@ __global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restri
                          epi_finish(ep, acc[mt][2][i], bv[mt][i]), epi_finish(ep, acc[mt][3][i], bv[mt][i])};
         else
             o = float4_t{acc[mt][0][i] * scale, acc[mt][1][i] * scale, acc[mt][2][i] * scale, acc[mt][3][i] * scale};
-        *(float4_t *)(yg + (size_t)(16 * mt + i) * row_stride * 4 + off) = o;
+        float4_t *const dst = (float4_t *)(yg + (size_t)(16 * mt + i) * row_stride * 4 + off);
+        if constexpr (NT)
+            __builtin_nontemporal_store(o, dst);
+        else
+            *dst = o;
     };
     // One tile: k-step ks waits for slot ks, reads it, hands the slot to the next tile's load,
     // multiplies, and issues the stores of the previous tile that fall to this step.
@@ -402,7 +412,7 @@ __global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restri
             constexpr int after = (KS - 1 - ks) + (HAS_NEXT ? ks : 0) + (STEADY ? NST : 0);
             __builtin_amdgcn_s_waitcnt(vmcnt_enc(after));
             const float4_t xv = ring_read16<ks * 1024>(lds_lane);
-            if constexpr (HAS_NEXT) ring_dma16(xg + ks * x_step, noff, lds_wave + ks * 1024);
+            if constexpr (HAS_NEXT) ring_dma16<NT>(xg + ks * x_step, noff, lds_wave + ks * 1024);
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
 #pragma unroll
@@ -477,7 +487,9 @@ __global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restri
 // 16-bit MFMA path: x is fp16 or e4m3fn (decoded to fp16, exact), w is fp16 or e4m3fn,
 // y is fp16.  MT = b / 16, KS = c / (4 * KL).  Each wave iteration covers 16 * VEC columns.
 // ------------------------------------------------------------------------------------------
-template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC, bool ROLL, bool EPI>
+// NT: non-temporal loads of the input rows and stores of the output rows (streams that are not read
+// again by this kernel: they need not stay in the caches)
+template <typename TX, typename TW, int MT, int KS, int KL, int VEC, int OCC, bool ROLL, bool EPI, bool NT>
 __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ x,
                                                    const TW *__restrict__ w,
                                                    half_t *__restrict__ y, int batch, int a, int b,
@@ -548,8 +560,8 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
             for (int jj = 0; jj < KL; ++jj)
-                io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + off),
-                         raw[ks][jj]);
+                io::template load<NT>((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + off),
+                                      raw[ks][jj]);
     }
     float bv[EPI ? MT : 1][4];  // bias of the output rows this lane holds
     if constexpr (EPI) {
@@ -575,8 +587,8 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
             if constexpr (ROLL) {
 #pragma unroll
                 for (int jj = 0; jj < KL; ++jj)
-                    io::load((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + next_off),
-                             raw[ks][jj]);
+                    io::template load<NT>((const TX *)(xg + (size_t)(KSTEP * ks + jj) * row_stride * sizeof(TX) + next_off),
+                                          raw[ks][jj]);
             }
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
@@ -615,7 +627,10 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_h(const TX *__restrict__ 
                             else
                                 o[v] = (half_t)(acc[mt][v0 + v][i] * scale);
                         }
-                        *(typename hvec<W>::type *)(dst + v0) = o;
+                        if constexpr (NT)
+                            __builtin_nontemporal_store(o, (typename hvec<W>::type *)(dst + v0));
+                        else
+                            *(typename hvec<W>::type *)(dst + v0) = o;
                     }
                 }
         }
@@ -635,6 +650,8 @@ struct WaveInst {
     // reloaded); [2], [3]: the same with bias / activation
     const void *fn[4];
     int ring = 0;  // > 0: the ring form, with at most this many waves per workgroup (LDS: c / 4 KB each)
+    int nt = 0;    // non-temporal loads of the input and stores of the output
+    int pref = 0;  // the automatic choice looks at these first (measured faster than the older forms)
 };
 
 typedef void (*f32_fn)(const float *, const float *, float *, int, int, int, int, int, Epi, int, int, int);
@@ -647,10 +664,12 @@ using h_fn = void (*)(const TX *, const TW *, half_t *, int, int, int, int, int,
     {B_, C_, 4, 1, OCC_, {F32_FN(B_, C_, OCC_, true, false), F32_FN(B_, C_, OCC_, false, false), \
                           F32_FN(B_, C_, OCC_, true, true), F32_FN(B_, C_, OCC_, false, true)}}
 // DEFER_: a second set of accumulators, the stores of a tile spread over the next one
-#define F32_RING_FN(B_, C_, DEFER_, EPI_) (const void *)(f32_fn)ks_wave_ring_f32<B_ / 16, C_ / 4, DEFER_, EPI_>
-#define F32_RING(B_, C_, DEFER_, WAVES_) \
-    {B_, C_, 4, 1, DEFER_ ? 1 : 2, {F32_RING_FN(B_, C_, DEFER_, false), F32_RING_FN(B_, C_, DEFER_, false), \
-                                    F32_RING_FN(B_, C_, DEFER_, true), F32_RING_FN(B_, C_, DEFER_, true)}, WAVES_}
+// NT_: non-temporal loads and stores (the `nt` field tells such instances apart)
+#define F32_RING_FN(B_, C_, DEFER_, NT_, EPI_) (const void *)(f32_fn)ks_wave_ring_f32<B_ / 16, C_ / 4, DEFER_, NT_, EPI_>
+#define F32_RING(B_, C_, DEFER_, NT_, WAVES_) \
+    {B_, C_, 4, 1, DEFER_ ? 1 : 2, {F32_RING_FN(B_, C_, DEFER_, NT_, false), F32_RING_FN(B_, C_, DEFER_, NT_, false), \
+                                    F32_RING_FN(B_, C_, DEFER_, NT_, true), F32_RING_FN(B_, C_, DEFER_, NT_, true)}, WAVES_, NT_, \
+     (B_) == 48 && (C_) == 48 && NT_ && DEFER_}
 const WaveInst f32_insts[] = {
     F32_INST(48, 48, 2), F32_INST(48, 48, 3), F32_INST(64, 64, 2), F32_INST(64, 64, 1),
     F32_INST(16, 16, 4), F32_INST(32, 32, 3), F32_INST(48, 192, 1),
@@ -659,23 +678,31 @@ const WaveInst f32_insts[] = {
     // (6,64,64,1) at batch 25088 (groups of 16 rows were 15-40 % slower there and on 48 x 48)
     F32_INST(32, 64, 3),
     // ring form (input through a per-wave LDS ring, stores spread over the next tile)
-    F32_RING(48, 48, true, 8), F32_RING(64, 64, false, 8), F32_RING(32, 64, true, 8), F32_RING(16, 16, true, 8),
-    F32_RING(32, 32, true, 8), F32_RING(48, 48, false, 8),
+    F32_RING(48, 48, true, false, 8), F32_RING(64, 64, false, false, 8), F32_RING(32, 64, true, false, 8),
+    F32_RING(16, 16, true, false, 8), F32_RING(32, 32, true, false, 8), F32_RING(48, 48, false, false, 8),
+    // the same with non-temporal loads and stores
+    F32_RING(48, 48, true, true, 8), F32_RING(64, 64, false, true, 8), F32_RING(32, 64, true, true, 8),
+    F32_RING(16, 16, true, true, 8), F32_RING(32, 32, true, true, 8),
 };
 
-#define H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, ROLL_, EPI_) \
-    (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, ROLL_, EPI_>
-#define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_)                                                          \
+#define H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, ROLL_, EPI_, NT_) \
+    (const void *)(h_fn<TX_, TW_>)ks_wave_bl_h<TX_, TW_, B_ / 16, C_ / (4 * KL_), KL_, VEC_, OCC_, ROLL_, EPI_, NT_>
+#define H_INST_N(TX_, TW_, B_, C_, KL_, VEC_, OCC_, NT_)                                                   \
     {B_, C_, VEC_, KL_, OCC_,                                                                              \
-     {H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, true, false), H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false, false), \
-      H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, true, true), H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false, true)}}
+     {H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, true, false, NT_), H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false, false, NT_), \
+      H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, true, true, NT_), H_FN(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false, true, NT_)}, 0, NT_, \
+     NT_ && (B_) == 16 && sizeof(TX_) == 2}
+#define H_INST(TX_, TW_, B_, C_, KL_, VEC_, OCC_) H_INST_N(TX_, TW_, B_, C_, KL_, VEC_, OCC_, false)
 #define H_SET(TX_, TW_)                                                                      \
     H_INST(TX_, TW_, 64, 64, 8, 4, 2), H_INST(TX_, TW_, 64, 64, 8, 8, 2),                    \
         H_INST(TX_, TW_, 64, 64, 8, 8, 1), H_INST(TX_, TW_, 48, 48, 4, 4, 3),                \
         H_INST(TX_, TW_, 48, 48, 4, 8, 2), H_INST(TX_, TW_, 16, 16, 4, 8, 4),                \
         H_INST(TX_, TW_, 16, 16, 4, 4, 4), H_INST(TX_, TW_, 32, 32, 8, 8, 3),                \
         H_INST(TX_, TW_, 96, 96, 8, 4, 1), H_INST(TX_, TW_, 48, 192, 8, 4, 1),              \
-        H_INST(TX_, TW_, 192, 48, 4, 4, 1)
+        H_INST(TX_, TW_, 192, 48, 4, 4, 1),                                                 \
+        H_INST_N(TX_, TW_, 16, 16, 4, 8, 4, true), H_INST_N(TX_, TW_, 16, 16, 4, 4, 4, true), \
+        H_INST_N(TX_, TW_, 48, 48, 4, 8, 2, true), H_INST_N(TX_, TW_, 64, 64, 8, 8, 2, true), \
+        H_INST_N(TX_, TW_, 32, 32, 8, 8, 3, true)
 const WaveInst h_insts[] = {H_SET(half_t, half_t)};
 const WaveInst hq_insts[] = {H_SET(half_t, fp8_t)};
 const WaveInst q_insts[] = {
@@ -683,10 +710,10 @@ const WaveInst q_insts[] = {
     H_INST(fp8_t, fp8_t, 48, 48, 4, 8, 2),  H_INST(fp8_t, fp8_t, 16, 16, 4, 8, 4),
     H_INST(fp8_t, fp8_t, 16, 16, 4, 16, 3), H_INST(fp8_t, fp8_t, 32, 32, 8, 16, 2),
     H_INST(fp8_t, fp8_t, 32, 32, 8, 8, 3),  H_INST(fp8_t, fp8_t, 48, 192, 8, 8, 1),
+    H_INST_N(fp8_t, fp8_t, 16, 16, 4, 8, 4, true), H_INST_N(fp8_t, fp8_t, 16, 16, 4, 16, 3, true),
+    H_INST_N(fp8_t, fp8_t, 48, 48, 4, 8, 2, true), H_INST_N(fp8_t, fp8_t, 64, 64, 8, 8, 2, true),
+    H_INST_N(fp8_t, fp8_t, 32, 32, 8, 16, 2, true),
 };
-
-// whether the automatic choice may take ring instances (listed behind the register forms)
-constexpr bool RING_BY_DEFAULT = false;
 
 const WaveInst *wave_table(int combo, int *n)
 {
@@ -713,8 +740,8 @@ uint32_t wave_inst_id(int combo, int i)
     int n;
     const WaveInst *t = wave_table(combo, &n);
     if (i < 0 || i >= n) return 0;
-    const int v[7] = {combo, t[i].b, t[i].c, t[i].vec, t[i].kl, t[i].occ, t[i].ring};
-    return inst_hash('W', v, t[i].ring ? 7 : 6);  // (ids of the register-form instances predate the field)
+    const int v[8] = {combo, t[i].b, t[i].c, t[i].vec, t[i].kl, t[i].occ, t[i].ring, t[i].nt};
+    return inst_hash('W', v, t[i].nt ? 8 : t[i].ring ? 7 : 6);  // (ids of the older instances predate the fields)
 }
 
 int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
@@ -735,16 +762,20 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     int rr = variant < 0 ? -1 : ((variant >> 16) & 3);
     if (rr == 3) return KSMM_ERR_BAD_ALGO;
     int pick = -1;
-    for (int i = 0; i < n_insts; ++i) {
-        // fp32: a forced instance also takes blocks whose b is a multiple of its rows (row groups)
-        const bool rows_ok = insts[i].b == p.b || (combo == 0 && want == i && p.b % insts[i].b == 0);
-        if (!rows_ok || insts[i].c != p.c) continue;
-        if (p.batch % insts[i].vec) continue;
-        if (want != 0xff && want != i) continue;
-        if (want == 0xff && insts[i].ring && !RING_BY_DEFAULT) continue;
-        pick = i;
-        break;
-    }
+    // automatic choice: the preferred instances first, then the others in table order (ring and
+    // non-temporal forms that are not marked preferred are taken only when forced or named by the
+    // measured table)
+    for (int pass = 0; pass < 2 && pick < 0; ++pass)
+        for (int i = 0; i < n_insts; ++i) {
+            // fp32: a forced instance also takes blocks whose b is a multiple of its rows (row groups)
+            const bool rows_ok = insts[i].b == p.b || (combo == 0 && want == i && p.b % insts[i].b == 0);
+            if (!rows_ok || insts[i].c != p.c) continue;
+            if (p.batch % insts[i].vec) continue;
+            if (want != 0xff && want != i) continue;
+            if (want == 0xff && (pass == 0 ? !insts[i].pref : (insts[i].ring || insts[i].nt))) continue;
+            pick = i;
+            break;
+        }
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
     const WaveInst &in = insts[pick];
     // The per-lane byte offsets must fit in 32 bits.  The largest ones formed are row 3*KL of a
@@ -759,28 +790,26 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int tn = 16 * in.vec;
     const int64_t n_tiles = (p.batch + tn - 1) / tn;
     if (in.ring) {
-        // Ring form: every wave takes every n_slabs-th tile of its block's row of tiles.  Tiles per
-        // wave (bits 8-15, 0: automatic): the smallest number with which all waves are resident at
-        // once (at most in.ring waves per CU, and what the LDS holds: c / 4 KB per wave), so that
-        // all of them share the work evenly; bits 18-21: waves per workgroup (0: as many as spread
-        // the waves over one workgroup per CU).
+        // Ring form: every wave takes every n_slabs-th tile of its block's row of tiles.  Bits
+        // 18-21: waves per workgroup (0: four, one per SIMD; at most in.ring and what the LDS
+        // holds, c / 4 KB per wave); tiles per wave (bits 8-15, 0: automatic): the smallest number
+        // with which all workgroups are resident at once, one per CU.
         const int64_t groups = (int64_t)p.a * p.d * (p.b / in.b);
         const int ks = p.c / 4;
         int wmax = in.ring;
         if (wmax * ks > 160) wmax = 160 / ks;
         int wpw = variant < 0 ? 0 : ((variant >> 18) & 15);
         if (wpw > wmax || wmax < 1) return KSMM_ERR_BAD_ALGO;
+        // (measured on (1,48,48,16) at batch 25088: one wave per SIMD, 7 tiles per wave, 224
+        // workgroups 30.4 us; 7 or 8 waves per workgroup with 4 tiles each 31.1-31.3; workgroups
+        // beyond one round 32-34)
+        if (wpw == 0) wpw = wmax < 4 ? wmax : 4;
         if (iters == 0) {
             iters = 1;
-            while (iters < 255 && groups * ((n_tiles + iters - 1) / iters) > 256 * (int64_t)(wpw ? wpw : wmax)) ++iters;
+            while (iters < 255 && groups * ((n_tiles + iters - 1) / iters) > 256 * (int64_t)wpw) ++iters;
         }
         const int64_t n_slabs = (n_tiles + iters - 1) / iters;
         const int64_t waves = groups * n_slabs;
-        if (wpw == 0) {
-            wpw = (int)((waves + 255) / 256);
-            if (wpw < 4) wpw = 4;  // (small problems: fewer, fuller workgroups)
-            if (wpw > wmax) wpw = wmax;
-        }
         const int64_t blocks = (waves + wpw - 1) / wpw;
         if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
         const int lds = wpw * ks * 1024;

