@@ -71,7 +71,9 @@ template <> struct wg_vec<half_t> {
 // q = lane / 16) loads N consecutive batch elements of operand row r at column n + N*q; MFMA e
 // multiplies element group e of every lane, i.e. its k-set is {n + N*q + e ...}: the same set for
 // both operands, and the order of a sum's terms is free.
-template <typename T, int MT, int NT>
+// NTL: non-temporal loads, for blocks of a single tile (every operand row is read by one wave only;
+// with several tiles per block the rows are shared through the caches)
+template <typename T, int MT, int NT, bool NTL>
 __global__ __launch_bounds__(256) void ks_wgrad_bl_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                           float *__restrict__ acc_out, int batch, int a, int b,
                                                           int c, int d, int m_tiles, int n_tiles, int splits,
@@ -107,31 +109,42 @@ __global__ __launch_bounds__(256) void ks_wgrad_bl_kernel(const T *__restrict__ 
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
     typedef typename V::type vec_t;
-    for (int n = n_begin; n < n_end; n += STEP) {
-        const int col = n + V::N * q;
-        const bool live = col < n_end;             // whole vectors: batch and the split are multiples of N
-        const int lcol = live ? col : n_begin;     // (a valid address; the value is zeroed)
-        vec_t av[MT], bv[NT];
+    // U sub-steps per iteration, all their loads issued before the first MFMA: a row is then read
+    // in runs of U * 64 bytes, and the loads of the whole iteration are in flight together
+    constexpr int U = (MT + NT) * 4 <= 24 ? 4 : 2;
+    for (int n = n_begin; n < n_end; n += U * STEP) {
+        vec_t av[U][MT], bv[U][NT];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) av[i] = *(const vec_t *)(ap[i] + lcol);
-#pragma unroll
-        for (int j = 0; j < NT; ++j) bv[j] = *(const vec_t *)(bp[j] + lcol);
-        if (!live) {
+        for (int u = 0; u < U; ++u) {
+            const int col = n + u * STEP + V::N * q;
+            const bool live = col < n_end;          // whole vectors: batch and the split are multiples of N
+            const int lcol = live ? col : n_begin;  // (a valid address; the value is zeroed)
 #pragma unroll
             for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int e = 0; e < V::N; ++e) av[i][e] = 0;
+                av[u][i] = NTL ? __builtin_nontemporal_load((const vec_t *)(ap[i] + lcol)) : *(const vec_t *)(ap[i] + lcol);
 #pragma unroll
             for (int j = 0; j < NT; ++j)
-#pragma unroll
-                for (int e = 0; e < V::N; ++e) bv[j][e] = 0;
+                bv[u][j] = NTL ? __builtin_nontemporal_load((const vec_t *)(bp[j] + lcol)) : *(const vec_t *)(bp[j] + lcol);
         }
 #pragma unroll
-        for (int e = 0; e < V::MFMAS; ++e)
+        for (int u = 0; u < U; ++u) {
+            if (n + u * STEP + V::N * q >= n_end) {
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+                for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < NT; ++j) acc[i][j] = V::mfma(e, av[i], bv[j], acc[i][j]);
+                    for (int e = 0; e < V::N; ++e) av[u][i][e] = 0;
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+#pragma unroll
+                    for (int e = 0; e < V::N; ++e) bv[u][j][e] = 0;
+            }
+#pragma unroll
+            for (int e = 0; e < V::MFMAS; ++e)
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) acc[i][j] = V::mfma(e, av[u][i], bv[u][j], acc[i][j]);
+        }
     }
     // D: lane holds column (c index) r and rows (b index) 4*q .. 4*q + 3 of each 16 x 16 tile
 #pragma unroll
@@ -206,9 +219,9 @@ template <typename T> int launch_block_transpose(const void *w, void *wt, int64_
 // a*b*c*d partial sums of its own): columns per split and their number.
 void wgrad_bl_splits(int64_t batch, int64_t tiles, int step, int64_t *splits_out, int64_t *cols_out)
 {
-    // about 16 waves per CU; at least 8 steps per wave
+    // about 16 waves per CU; at least 4 loop iterations per wave
     int64_t splits = (4096 + tiles - 1) / tiles;
-    const int64_t max_splits = (batch + 8 * step - 1) / (8 * step);
+    const int64_t max_splits = (batch + 4 * step - 1) / (4 * step);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     int64_t cols = (batch + splits - 1) / splits;
@@ -248,15 +261,20 @@ int launch_wgrad_bl(const void *dy, const void *x, float *acc, int64_t batch, in
 {
     const int m_tiles = (b + 16 * MT - 1) / (16 * MT), n_tiles = (c + 16 * NT - 1) / (16 * NT);
     const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
-    constexpr int STEP = 4 * wg_vec<T>::N;
+    constexpr int STEP = 16 * wg_vec<T>::N;  // columns per loop iteration of the kernel (four sub-steps)
     int64_t splits, cols;
     wgrad_bl_splits(batch, tiles, STEP, &splits, &cols);
     const int64_t waves = tiles * splits, blocks = (waves + 3) / 4;
     if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     *splits_used = (int)splits;
-    hipLaunchKernelGGL((ks_wgrad_bl_kernel<T, MT, NT>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
-                       (const T *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols,
-                       (int64_t)a * b * c * d);
+    if (m_tiles == 1 && n_tiles == 1)
+        hipLaunchKernelGGL((ks_wgrad_bl_kernel<T, MT, NT, true>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
+                           (const T *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols,
+                           (int64_t)a * b * c * d);
+    else
+        hipLaunchKernelGGL((ks_wgrad_bl_kernel<T, MT, NT, false>), dim3((unsigned)blocks), dim3(256), 0, s, (const T *)dy,
+                           (const T *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols,
+                           (int64_t)a * b * c * d);
     return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
@@ -304,7 +322,7 @@ int64_t wgrad_partial_floats(int64_t batch, int a, int b, int c, int d, int dtyp
     int64_t splits, cols, most = 1;
     const int t = wgrad_bl_tile(b, c);
     const int64_t tiles_bl = (int64_t)a * d * ((b + 16 * t - 1) / (16 * t)) * ((c + 16 * t - 1) / (16 * t));
-    wgrad_bl_splits(batch, tiles_bl, 4 * (16 / (int)dtype_size(dtype)), &splits, &cols);
+    wgrad_bl_splits(batch, tiles_bl, 16 * (16 / (int)dtype_size(dtype)), &splits, &cols);
     if (splits > most) most = splits;
     wgrad_tiled_splits(batch, (int64_t)a * d * ((b + 15) / 16) * ((c + 15) / 16), &splits, &cols);
     if (splits > most) most = splits;

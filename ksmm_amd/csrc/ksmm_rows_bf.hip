@@ -456,8 +456,12 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         }
         if (t.dd == p.d) {
             // all d blocks in one workgroup: the smallest batch tile (more workgroups per CU;
-            // measured 10-55 % faster than the 32- and 64-row tiles for d <= 8)
-            if (pick < 0 || row_insts[pick].dd != p.d || t.tn < row_insts[pick].tn) pick = i;
+            // measured 10-55 % faster than the 32- and 64-row tiles for d <= 8), except for
+            // 128 x 128 blocks, whose weights take longer to read than a small tile to multiply
+            // ((1,128,128,3) at batch 25088: fp16 28.8 us with 16 rows, 23.9 with 32; e4m3 42.2 / 33.3)
+            const bool larger = t.bb * t.cc >= 128 * 128;
+            if (pick < 0 || row_insts[pick].dd != p.d || (larger ? t.tn > row_insts[pick].tn : t.tn < row_insts[pick].tn))
+                pick = i;
         } else if (pick >= 0 && row_insts[pick].dd == p.d) {
             // an exact match was found already
         } else if (grouped_ok && (run_bytes >= 32 || (combo == 0 && p.b <= p.c)) &&

@@ -13,6 +13,7 @@ which is compiled into the library, named by its stable instance id.
     python -m ksmm_amd.tune --patterns FILE [--dtypes fp32,fp16,fp8] [--layouts last,first]
                             [--batch 25088] [--json OUT.json] [--merge A.json B.json ...]
                             [--emit ksmm_amd/csrc/ksmm_tuned.inc] [--emit-best ksmm_amd/tuned]
+                            [--update ksmm_amd/csrc/ksmm_tuned.inc] [--update-best ksmm_amd/tuned]
 
 ``FILE`` holds one ``a,b,c,d`` per line (the reference's patterns.in has that format).  Several
 runs (e.g. one per element type) can be merged with ``--merge`` before ``--emit``.
@@ -103,7 +104,7 @@ def _sample_cols(batch, n=48):
     return np.array(sorted(idx))
 
 
-def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
+def tune_pattern(pattern, prec, bs_last, batch, lib_mod, rotation_bytes=1.3e9):
     from . import Kernel, generate_factor, quantize_fp8
     from .kernel import query_tile, variant_id
     from .layer import from_kernel_format_to_abcd
@@ -120,7 +121,10 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, budget_bytes=1.5e9):
     es_out = 2 if prec != "fp32" else 4
     in_size, out_size = a * c * d, a * b * d
     per_set = batch * (in_size * es_in + out_size * es_out)
-    n_sets = max(2, min(4, int(budget_bytes // max(per_set, 1))))
+    # Consecutive launches rotate over distinct input/output sets of at least 1.2 GB in total (at
+    # most 24 sets), as bench.py does: the 256 MB last-level cache cannot hand a set back to the
+    # launch that uses it next, so candidates are ranked cold, the way they are used.
+    n_sets = max(2, min(24, int(math.ceil(rotation_bytes / max(per_set, 1)))))
     g = torch.Generator(device="cuda").manual_seed(1)
     w4 = (torch.rand(a, b, c, d, generator=g, device="cuda") * 2 - 1) / math.sqrt(c)
     if prec == "fp8":
@@ -262,6 +266,61 @@ def emit(entries, path, batch):
     return len(rows)
 
 
+def update_inc(entries, path, batch):
+    """Re-measured patterns into an existing table: the rows of every (pattern, type, layout) in
+    ``entries`` are replaced by what ``emit`` would write for them (or dropped when the heuristic
+    is now within 3 %); all other rows stay as they are."""
+    import re
+    import tempfile
+
+    keep = []
+    redone = {(tuple(e["pattern"]), COMBO[e["prec"]], 1 if e["bs_last"] else 0) for e in entries}
+    row_re = re.compile(r"^\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)u, (-?\d+)\},\s*//\s*([\d.]+) \(([\d.]+)\)")
+    for line in open(path):
+        m = row_re.match(line)
+        if not m:
+            continue
+        v = [int(g) for g in m.groups()[:9]]
+        if (tuple(v[:4]), v[4], v[5]) in redone:
+            continue
+        keep.append(tuple(v) + (float(m.group(10)), float(m.group(11))))
+    with tempfile.NamedTemporaryFile("r", suffix=".inc") as tmp:
+        emit(entries, tmp.name, batch)
+        for line in open(tmp.name):
+            m = row_re.match(line)
+            if m:
+                keep.append(tuple(int(g) for g in m.groups()[:9]) + (float(m.group(10)), float(m.group(11))))
+    keep.sort(key=lambda r: r[:6])
+    head = [l for l in open(path) if l.startswith("//")]
+    with open(path, "w") as f:
+        f.writelines(head)
+        for r in keep:
+            f.write("{%d, %d, %d, %d, %d, %d, %d, %du, %d},  // %.1f (%.1f)\n" % r)
+    return len(keep)
+
+
+def update_best(entries, directory):
+    """The same for the ``*.best`` text files: lines of re-measured patterns are replaced."""
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        written = emit_best(entries, tmp)
+        for name in written:
+            new_lines = [l for l in open(os.path.join(tmp, name)) if not l.startswith("#")]
+            key = lambda l: tuple(l.split()[:5])
+            fresh = {key(l): l for l in new_lines}
+            old_path = os.path.join(directory, name)
+            old_lines = [l for l in open(old_path)] if os.path.exists(old_path) else []
+            head = [l for l in old_lines if l.startswith("#")] or [open(os.path.join(tmp, name)).readline()]
+            body = {key(l): l for l in old_lines if not l.startswith("#")}
+            body.update(fresh)
+            with open(old_path, "w") as f:
+                f.writelines(head[:1])
+                for k in sorted(body, key=lambda k: tuple(int(v) for v in k)):
+                    f.write(body[k])
+    return written
+
+
 BEST_NAME = {"fp32": "float", "fp16": "half", "fp8": "fp8e4m3"}
 FAMILY = {0: "auto", 1: "generic", 2: "wave", 3: "tile"}
 
@@ -317,6 +376,8 @@ def main():
     ap.add_argument("--merge", nargs="*", default=[])
     ap.add_argument("--emit")
     ap.add_argument("--emit-best", help="directory for the kernel_bs_*_*.best text files")
+    ap.add_argument("--update", help="an existing table (.inc): replace the rows of the measured patterns, keep the rest")
+    ap.add_argument("--update-best", help="directory of existing *.best files: replace the lines of the measured patterns")
     ap.add_argument("--shard", default="0/1", help="i/n: take every n-th pattern starting at i")
     ap.add_argument("--time-limit", type=float, default=1e9, help="stop (and save) after this many seconds")
     args = ap.parse_args()
@@ -366,6 +427,11 @@ def main():
     if args.emit:
         n = emit(entries, args.emit, args.batch)
         print("wrote %d rows to %s" % (n, args.emit))
+    if args.update:
+        print("%s now holds %d rows" % (args.update, update_inc(entries, args.update, args.batch)))
+    if args.update_best:
+        for name, n in update_best(entries, args.update_best).items():
+            print("updated %d patterns in %s" % (n, os.path.join(args.update_best, name)))
     if args.emit_best:
         for name, n in emit_best(entries, args.emit_best).items():
             print("wrote %d patterns to %s" % (n, os.path.join(args.emit_best, name)))
