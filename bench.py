@@ -166,6 +166,8 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
 
         copy_us = pattern_copy_us(p, bs_last, cur, outs, steps, warmup)
         sec = time_launches(run, n_sets, steps, warmup)
+        stream_us = same_bytes_stream_copy_us(cur[0].numel() * cur[0].element_size()
+                                              + outs[0].numel() * outs[0].element_size(), steps, warmup)
         x_dt = cur[0].dtype
         roof = factor_roofline(BATCH, p, x_dt, facs[i].dtype, out_dt, sec)
         tile = query_tile(BATCH, p, x_dt, facs[i].dtype, bs_last)
@@ -174,7 +176,11 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
             "bound": roof["bound"], "roofline_frac": roof["frac"], "floor_us": roof["floor_us"],
             "x_dtype": str(x_dt).replace("torch.", ""), "algo": tile["algo"], "variant": tile["variant"],
             # a tile-at-a-time copy with this factor's addresses and no arithmetic (None: no such copy)
-            "pattern_copy_us": copy_us})
+            "pattern_copy_us": copy_us,
+            # the streaming copy (non-temporal, persistent grid) moving as many bytes as this factor
+            # reads and writes, half of them each way: what the memory system gives a kernel that
+            # does nothing else
+            "stream_copy_us": stream_us, "frac_of_stream_copy": stream_us / (sec * 1e6)})
         cur = outs
     # ---- whole KSLinear (chain launcher) ----------------------------------------------------
     if len(patterns) > 1:
@@ -285,6 +291,32 @@ def bench_backward(name, pattern, prec, bs_last, steps, warmup):
         out[key + "_gbs"] = nbytes / sec / 1e9
         out[key + "_tflops"] = flops / sec / 1e12
     return out
+
+
+_STREAM_COPY_US = {}
+
+
+def same_bytes_stream_copy_us(total_bytes, steps, warmup):
+    """µs the streaming copy of the benchmark library takes to move `total_bytes` (half read,
+    half written) with the buffer rotation of the factor timings; one measurement per size."""
+    import ctypes
+
+    from ksmm_amd import _lib, bench_lib
+
+    half = (total_bytes // 2 + 15) // 16 * 16
+    if half not in _STREAM_COPY_US:
+        lib = bench_lib.load()
+        n_sets = max(2, min(8, int(math.ceil(1.2e9 / (2 * half)))))
+        src = [torch.empty(half, dtype=torch.uint8, device="cuda").random_() for _ in range(n_sets)]
+        dst = [torch.empty_like(t) for t in src]
+
+        def run(j):
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            _lib.check(lib.ksbench_stream_copy(src[j].data_ptr(), dst[j].data_ptr(), half, 2048, stream))
+
+        _STREAM_COPY_US[half] = time_launches(run, n_sets, max(20, steps // 2), max(5, warmup // 2)) * 1e6
+        del src, dst
+    return _STREAM_COPY_US[half]
 
 
 def copy_reference(steps, warmup):

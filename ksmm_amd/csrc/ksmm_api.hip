@@ -395,6 +395,10 @@ bool chain_wants_transposed(const ksmm_factor_desc *f, int n, int64_t batch, int
                             int bs_last)
 {
     if (bs_last) return false;
+    // a chain the fused kernel takes in batch-size-last layout: one pass over the data between two
+    // transposes instead of one pass per factor
+    if (chain16_run(f, n, nullptr, nullptr, padded_batch(batch), x_dtype, y_dtype, 1, false, nullptr, nullptr) == KSMM_OK)
+        return true;
     for (int i = 0; i < n; ++i) {
         Problem p{nullptr, nullptr, nullptr, batch, f[i].a, f[i].b, f[i].c, f[i].d, i == 0 ? x_dtype : y_dtype,
                   f[i].w_dtype, y_dtype, 0, 1.f, nullptr};

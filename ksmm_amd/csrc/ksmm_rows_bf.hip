@@ -1,4 +1,5 @@
-// "Row" kernels: batch-size-first layout, d > 1, small b x c blocks.  The fp32 kernel first; the
+// "Row" kernels: batch-size-first layout, small b x c blocks, d > 1 (and d == 1 in groups of
+// consecutive a_i, at the end of this comment).  The fp32 kernel first; the
 // fp16 / e4m3 one further down has the same structure.
 //
 // In this layout a batch row holds, for one a_i, the c*d inputs of all d blocks interleaved
@@ -14,6 +15,10 @@
 // The loads of the next two tiles are in flight (in registers) while a tile is multiplied and
 // stored; tiles are dealt round-robin to the workgroups of an a_i, so that at any time they
 // work on one compact window of memory.
+//
+// d == 1 with blocks of 16 x 16 or 32 x 32 (the last factor of a butterfly chain, (64,16,16,1)):
+// the same kernel with the waves of a workgroup taking DD consecutive a_i, whose inputs are one
+// contiguous run of DD * c elements per batch row; only the index arithmetic differs.
 //
 // Reference counterpart: kernel_bs_first_float
 // (src/ksmm_py/layer/kronecker_sparse/template_kernels_float.cuh:85-286), whose strided scalar
@@ -51,21 +56,24 @@ template <int BB, int CC, int DD, int TN, bool PL = false, int MS = 1> struct Ro
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-template <int BB, int CC, int DD, int TN, bool NT_STORE, bool PL = false, int MS = 1>
+// AG: d == 1 and the DD waves take DD consecutive a_i instead (their inputs are one contiguous run
+// of DD * c elements of a batch row, block after block: the "stride" of a block's inputs is 1).
+template <int BB, int CC, int DD, int TN, bool NT_STORE, bool PL = false, int MS = 1, bool AG = false>
 __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ w,
                                                             float *__restrict__ y, int batch, int a,
                                                             int d, Epi ep, int wgs_per_a, int n_tiles)
 {
     typedef RowCfg<BB, CC, DD, TN, PL, MS> C;
+    static_assert(!(AG && PL), "planes are for interleaved blocks");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *const xs = (float *)smem;                // [2][TN][LDX]; PL: [2][DD][PLANE_X]
     float *const os = xs + 2 * C::X_FLOATS;         // [TN][LDO]; PL: [DD][PLANE_O]
-    // blockIdx -> (a_i, group of DD d_i, share of the tiles)
-    const int groups = d / DD;
+    // blockIdx -> (a_i, group of DD d_i, share of the tiles); AG: a_i is the group's first block
+    const int groups = AG ? 1 : d / DD;
     const int ag = blockIdx.x / wgs_per_a;
     const int s = blockIdx.x - ag * wgs_per_a;
-    const int a_i = ag / groups, d0 = (ag - a_i * groups) * DD;
+    const int a_i = AG ? ag * DD : ag / groups, d0 = AG ? 0 : (ag - a_i * groups) * DD;
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
@@ -77,7 +85,7 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *_
     // weights of block (a_i, dd): element (k, m) at ((a_i*d + dd)*c + k)*b + m -> A operands
     float wreg[C::MT][C::KS];
     {
-        const float *wg = w + (size_t)(a_i * d + d0 + dd) * CC * BB + m_off;
+        const float *wg = w + (size_t)(AG ? a_i + dd : a_i * d + d0 + dd) * CC * BB + m_off;
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
@@ -88,12 +96,14 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *_
     for (int mt = 0; mt < C::MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            bv[mt][i] = epi_bias<float>(ep, ((size_t)a_i * BB + m_off + 16 * mt + 4 * q + i) * d + d0 + dd);
+            bv[mt][i] = epi_bias<float>(ep, AG ? (size_t)(a_i + dd) * BB + m_off + 16 * mt + 4 * q + i
+                                               : ((size_t)a_i * BB + m_off + 16 * mt + 4 * q + i) * d + d0 + dd);
 
     // element e of a tile row (e = k * DD + j) lives at k * d + j behind the group's origin
+    // (AG: e = j * c + k, at e)
     const float *xg = x + (size_t)a_i * CC * d + d0;
     float *yg = y + (size_t)a_i * BB * d + d0;
-    auto row_off = [&](int e0) { return (e0 / DD) * d + e0 % DD; };
+    auto row_off = [&](int e0) { return AG ? e0 : (e0 / DD) * d + e0 % DD; };
     float4_t xreg[2][C::X_PER_T];
     auto gload = [&](int t, auto P) {
 #pragma unroll
@@ -140,8 +150,9 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *_
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
             for (int nt = 0; nt < C::NT; ++nt)
-                xf[ks][nt] = PL ? xb[dd * C::PLANE_X + (16 * nt + r) * C::LDK + 4 * ks + q]
-                                : xb[(16 * nt + r) * C::LDX + (4 * ks + q) * DD + dd];
+                xf[ks][nt] = PL   ? xb[dd * C::PLANE_X + (16 * nt + r) * C::LDK + 4 * ks + q]
+                             : AG ? xb[(16 * nt + r) * C::LDX + dd * CC + 4 * ks + q]
+                                  : xb[(16 * nt + r) * C::LDX + (4 * ks + q) * DD + dd];
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
@@ -156,8 +167,9 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *_
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[PL ? dd * C::PLANE_O + (16 * nt + r) * C::LDM + m_off + 16 * mt + 4 * q + i
-                          : (16 * nt + r) * C::LDO + (m_off + 16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
+                    os[PL   ? dd * C::PLANE_O + (16 * nt + r) * C::LDM + m_off + 16 * mt + 4 * q + i
+                       : AG ? (16 * nt + r) * C::LDO + dd * BB + m_off + 16 * mt + 4 * q + i
+                            : (16 * nt + r) * C::LDO + (m_off + 16 * mt + 4 * q + i) * DD + dd] = epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -217,7 +229,7 @@ template <typename TX, int BB, int CC, int DD, int TN> struct RowCfgH {
 __device__ __forceinline__ half_t row_to_half(half_t v) { return v; }
 __device__ __forceinline__ half_t row_to_half(fp8_t v) { return fp8_to_half(v.bits); }
 
-template <typename TX, int BB, int CC, int DD, int TN>
+template <typename TX, int BB, int CC, int DD, int TN, bool AG = false>
 __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restrict__ x, const TX *__restrict__ w,
                                                               half_t *__restrict__ y, int batch, int a, int d,
                                                               Epi ep, int wgs_per_a, int n_tiles)
@@ -226,10 +238,10 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     TX *const xs = (TX *)smem;                         // [2][TN][LDX]
     half_t *const os = (half_t *)(smem + C::X_BYTES);  // [TN][LDO]
-    const int groups = d / DD;
+    const int groups = AG ? 1 : d / DD;
     const int ag = blockIdx.x / wgs_per_a;
     const int s = blockIdx.x - ag * wgs_per_a;
-    const int a_i = ag / groups, d0 = (ag - a_i * groups) * DD;
+    const int a_i = AG ? ag * DD : ag / groups, d0 = AG ? 0 : (ag - a_i * groups) * DD;
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
@@ -240,7 +252,7 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
     // A operand of sub-step ks: lane (r, q) holds k = 16*ks + 4*q .. + 3 of row m = 16*mt + r
     half4_t wreg[C::MT][C::KS];
     {
-        const TX *wg = w + (size_t)(a_i * d + d0 + dd) * CC * BB;
+        const TX *wg = w + (size_t)(AG ? a_i + dd : a_i * d + d0 + dd) * CC * BB;
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
@@ -253,11 +265,12 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
     for (int mt = 0; mt < C::MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            bv[mt][i] = epi_bias<half_t>(ep, ((size_t)a_i * BB + 16 * mt + 4 * q + i) * d + d0 + dd);
+            bv[mt][i] = epi_bias<half_t>(ep, AG ? (size_t)(a_i + dd) * BB + 16 * mt + 4 * q + i
+                                                : ((size_t)a_i * BB + 16 * mt + 4 * q + i) * d + d0 + dd);
 
     const TX *xg = x + (size_t)a_i * CC * d + d0;
     half_t *yg = y + (size_t)a_i * BB * d + d0;
-    auto row_off = [&](int e0) { return (e0 / DD) * d + e0 % DD; };
+    auto row_off = [&](int e0) { return AG ? e0 : (e0 / DD) * d + e0 % DD; };
     uint4_t xreg[2][C::X_PER_T];
     auto gload = [&](int t, auto P) {
 #pragma unroll
@@ -297,7 +310,8 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    xf[ks][nt][j] = row_to_half(xb[(16 * nt + r) * C::LDX + (16 * ks + 4 * q + j) * DD + dd]);
+                    xf[ks][nt][j] = row_to_half(AG ? xb[(16 * nt + r) * C::LDX + dd * CC + 16 * ks + 4 * q + j]
+                                                   : xb[(16 * nt + r) * C::LDX + (16 * ks + 4 * q + j) * DD + dd]);
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
@@ -312,7 +326,8 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[(16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = (half_t)epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
+                    os[AG ? (16 * nt + r) * C::LDO + dd * BB + 16 * mt + 4 * q + i
+                          : (16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = (half_t)epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -348,6 +363,7 @@ struct RowInst {
     const void *fn;
     int planes;  // fp32: LDS tiles split into one plane per d_i
     int ms = 1;  // fp32: waves per d_i (row groups of a tall block)
+    int ag = 0;  // d == 1: the waves take dd consecutive a_i
 };
 #define ROW_INST_PL(BB_, CC_, DD_, TN_) \
     {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_, true>::LDS_BYTES, 4, 1, (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, true, true>, 1}
@@ -357,6 +373,26 @@ struct RowInst {
 #define ROW_INST_MS(BB_, CC_, DD_, TN_, MS_) \
     {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_, false, MS_>::LDS_BYTES, 4, 1, \
      (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, true, false, MS_>, 0, MS_}
+// d == 1: groups of DD_ consecutive blocks
+#define ROW_INST_AG(BB_, CC_, DD_, TN_) \
+    {0, BB_, CC_, DD_, TN_, RowCfg<BB_, CC_, DD_, TN_>::LDS_BYTES, 4, 1, \
+     (const void *)ks_rows_bf_kernel<BB_, CC_, DD_, TN_, true, false, 1, true>, 0, 1, 1}
+#define ROW_INST_AG_H(BB_, CC_, DD_, TN_) \
+    {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 8, 1, \
+     (const void *)ks_rows_bf_h_kernel<half_t, BB_, CC_, DD_, TN_, true>, 0, 1, 1}
+#define ROW_INST_AG_Q(BB_, CC_, DD_, TN_) \
+    {2, BB_, CC_, DD_, TN_, RowCfgH<fp8_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 16, 1, \
+     (const void *)ks_rows_bf_h_kernel<fp8_t, BB_, CC_, DD_, TN_, true>, 0, 1, 1}
+#define ROW_SET_AG(M) M(16, 16, 16, 32), M(16, 16, 16, 64), M(16, 16, 8, 64), M(16, 16, 4, 128), M(32, 32, 8, 32), M(32, 32, 4, 64), \
+    M(16, 16, 2, 128), M(16, 16, 1, 128)
+#define ROW_SET_AG32(M) M(16, 16, 16, 16), M(16, 16, 16, 32), M(16, 16, 8, 32), M(16, 16, 4, 64), M(32, 32, 8, 16), M(32, 32, 4, 32), \
+    M(16, 16, 2, 64), M(16, 16, 1, 128)
+#define ROW_SET_AG_B(M) \
+    M(48, 48, 4, 32), M(48, 48, 2, 64), M(48, 48, 1, 64), M(64, 64, 4, 32), M(64, 64, 2, 64), M(64, 64, 4, 64), \
+    M(96, 96, 2, 32), M(96, 96, 4, 16), M(64, 64, 1, 64), M(32, 32, 2, 64), M(32, 32, 1, 128)
+#define ROW_SET_AG32_B(M) \
+    M(48, 48, 4, 16), M(48, 48, 2, 32), M(48, 48, 1, 64), M(64, 64, 4, 16), M(64, 64, 2, 32), M(64, 64, 4, 32), \
+    M(64, 64, 1, 64), M(32, 32, 2, 64), M(32, 32, 1, 64)
 #define ROW_INST_H(BB_, CC_, DD_, TN_)                                                                      \
     {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_>::LDS_BYTES, 8, 1,                          \
      (const void *)ks_rows_bf_h_kernel<half_t, BB_, CC_, DD_, TN_>}
@@ -413,6 +449,13 @@ const RowInst row_insts[] = {
     ROW_SET_16C(ROW_INST_Q),
     // fp32 128 x 128 blocks: two waves per d_i
     ROW_INST_MS(128, 128, 3, 16, 2),
+    // d == 1, small blocks: groups of consecutive a_i
+    ROW_SET_AG32(ROW_INST_AG),
+    ROW_SET_AG(ROW_INST_AG_H),
+    ROW_SET_AG(ROW_INST_AG_Q),
+    ROW_SET_AG32_B(ROW_INST_AG),
+    ROW_SET_AG_B(ROW_INST_AG_H),
+    ROW_SET_AG_B(ROW_INST_AG_Q),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 constexpr int ROW_INST_BITS = 10, ROW_INST_ANY = (1 << ROW_INST_BITS) - 1;
@@ -426,8 +469,8 @@ uint32_t rows_inst_id(int i)
 {
     if (i < 0 || i >= N_ROW_INSTS) return 0;
     const RowInst &t = row_insts[i];
-    const int v[8] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt, t.planes, t.ms};
-    return inst_hash('R', v, t.ms > 1 ? 8 : t.planes ? 7 : 6);  // (ids of the other instances predate the fields)
+    const int v[9] = {t.combo, t.bb, t.cc, t.dd, t.tn, t.nt, t.planes, t.ms, t.ag};
+    return inst_hash('R', v, t.ag ? 9 : t.ms > 1 ? 8 : t.planes ? 7 : 6);  // (ids of the other instances predate the fields)
 }
 
 // variant: bits 0-9 instance (all ones: first that fits), bits 10.. workgroups per a_i (0: heuristic)
@@ -447,6 +490,25 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         // row segments start on 16-byte boundaries (output vectors: 4 floats / 8 halves)
         const int ovec = combo == 0 ? 4 : 8;
         if (((int64_t)p.a * p.c * p.d) % t.vec || ((int64_t)p.a * p.b * p.d) % ovec) continue;
+        if (t.ag) {
+            // d == 1: dd consecutive blocks per workgroup; the largest group that divides a (the
+            // smallest tile among equals: more workgroups)
+            if (p.d != 1 || p.a % t.dd) continue;
+            // blocks up to 48 x 48 always; 64 x 64 in groups of four for fp32 and e4m3 and 96 x 96
+            // for fp16 (measured against the tile and stream kernels these shapes had: fp32
+            // (12,64,64,1) 53 -> 46 us, fp16 (8,96,96,1) 27 -> 20 us, fp32 (16,48,48,1) 122 -> 38 us;
+            // fp16 64 x 64 stays on the stream kernel, 15 against 19 us); the rest when named
+            const bool take = t.bb * t.cc <= 48 * 48 || (t.bb == 64 && t.cc == 64 && t.dd == 4 && combo != 1) ||
+                              (t.bb == 96 && t.cc == 96 && combo == 1);
+            if (want == ROW_INST_ANY && !take) continue;
+            if (want != ROW_INST_ANY) {
+                pick = i;
+                break;
+            }
+            if (pick < 0 || t.dd > row_insts[pick].dd) pick = i;
+            continue;
+        }
+        if (p.d == 1) continue;
         // all d blocks in one workgroup, or groups of dd whose runs keep the 16-byte alignment
         const bool grouped_ok = t.dd % t.vec == 0 && t.dd % ovec == 0 && p.d % t.dd == 0;
         const int run_bytes = t.dd * (combo == 0 ? 4 : 2);  // output run of a group
@@ -474,7 +536,7 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if (pick < 0) return KSMM_ERR_BAD_ALGO;
     const RowInst &t = row_insts[pick];
     const int64_t n_tiles = (p.batch + t.tn - 1) / t.tn;
-    const int64_t ag = (int64_t)p.a * (p.d / t.dd);  // (a_i, group) pairs
+    const int64_t ag = t.ag ? p.a / t.dd : (int64_t)p.a * (p.d / t.dd);  // (a_i, group) pairs
     // one round of workgroups, 8 or more waves per CU
     const int nw = t.dd * t.ms;
     const int per_cu_lds = 160 * 1024 / t.lds, per_cu_waves = 16 / nw > 0 ? 16 / nw : 1;

@@ -283,6 +283,15 @@ def test_row_kernel_instances_forced():
     for prec in ("fp32", "fp16", "fp8"):
         _forced_sweep([(prec, False, p, batch) for p in late for batch in (512, 203)], [1000 + i for i in range(158, 172)], 2,
                       4 if prec == "fp32" else 16)
+    # d = 1: groups of consecutive a_i (16 x 16 and 32 x 32 blocks), every group size that divides a
+    ag = [(64, 16, 16, 1), (48, 16, 16, 1), (12, 16, 16, 1), (6, 16, 16, 1), (3, 16, 16, 1), (16, 32, 32, 1),
+          (4, 32, 32, 1), (6, 32, 32, 1), (3, 32, 32, 1), (12, 64, 64, 1), (6, 64, 64, 1), (3, 64, 64, 1),
+          (4, 48, 48, 1), (2, 48, 48, 1), (1, 48, 48, 1), (4, 96, 96, 1), (2, 96, 96, 1)]
+    for prec in ("fp32", "fp16", "fp8"):
+        _forced_sweep([(prec, False, p, batch) for p in ag for batch in (512, 203)], [1000 + i for i in range(167, 222)],
+                      2, 60)
+        # and as the automatic choice
+        _forced_sweep([(prec, False, p, 1000) for p in ag], [-1], 0, len(ag))
 
 
 def test_tile_subfamilies_forced():
