@@ -248,6 +248,88 @@ def bench_config(name, patterns, prec, bs_last, bound, steps, warmup, check=True
     return result
 
 
+FFN_UP = [(6, 64, 64, 1), (1, 768, 192, 2)]      # 384 -> 1536
+FFN_DOWN = [(6, 64, 256, 1), (1, 128, 128, 3)]   # 1536 -> 384
+
+
+def bench_ffn(steps, warmup, prec="fp16", bs_last=False):
+    """The feed-forward block of the reference's ViT-S benchmark (scripts/2_benchmark_ksvit_time.sh:5,
+    48-50; src/ksmm_py/model/vit.py:416-431) at B = 25 088 rows (196 tokens x 128 images), in its
+    default layout: up-projection + bias + GELU (both inside the last factor's kernel), then
+    down-projection + bias, two chain launches; per factor of the down-projection as well.  Checked
+    against the float64 oracle on sampled rows."""
+    from ksmm_amd import Kernel, generate_factor
+    from ksmm_amd.roofline import factor_roofline
+
+    dt = DT[prec]
+    gen = torch.Generator().manual_seed(SEED + 11)
+    w_up, w_dn = make_weights(FFN_UP, None, gen), make_weights(FFN_DOWN, None, gen)
+    f_up = [generate_factor(*p, "kernel", w, dt, "cuda") for p, w in zip(FFN_UP, w_up)]
+    f_dn = [generate_factor(*p, "kernel", w, dt, "cuda") for p, w in zip(FFN_DOWN, w_dn)]
+    n_in, n_hid = 384, 1536
+    b_up = (torch.randn(n_hid, generator=gen) * 0.1).to(dt).cuda()
+    b_dn = (torch.randn(n_in, generator=gen) * 0.1).to(dt).cuda()
+    n_sets = 8
+    shape = lambda n: (n, BATCH) if bs_last else (BATCH, n)
+    xs = []
+    for i in range(n_sets):
+        x = torch.randn(BATCH, n_in, generator=gen)
+        xs.append((x.t().contiguous() if bs_last else x).to(dt).cuda())
+    hid = [torch.empty(shape(n_hid), dtype=dt, device="cuda") for _ in range(n_sets)]
+    outs = [torch.empty(shape(n_in), dtype=dt, device="cuda") for _ in range(n_sets)]
+    ws = torch.empty(2 * (n_hid * BATCH * 4 + 256), dtype=torch.uint8, device="cuda")
+
+    def up(j):
+        return Kernel.chain_forward(xs[j], f_up, FFN_UP, bs_last, fuse=True, workspace=ws, bias=b_up, act="gelu",
+                                    out=hid[j])
+
+    def down(j):
+        return Kernel.chain_forward(hid[j], f_dn, FFN_DOWN, bs_last, fuse=True, workspace=ws, bias=b_dn, out=outs[j])
+
+    def ffn(j):
+        up(j)
+        return down(j)
+
+    res = {"name": "ffn_vit_s", "precision": prec, "bs_last": bs_last, "patterns_up": FFN_UP,
+           "patterns_down": FFN_DOWN, "batch": BATCH}
+    res["ffn_us"] = time_launches(ffn, n_sets, steps, warmup) * 1e6
+    res["up_bias_gelu_us"] = time_launches(up, n_sets, steps, warmup) * 1e6
+    res["down_bias_us"] = time_launches(down, n_sets, steps, warmup) * 1e6
+    # the down-projection's factors on their own (input of the second = output of the first)
+    mid = [torch.empty(shape(FFN_DOWN[0][0] * FFN_DOWN[0][1] * FFN_DOWN[0][3]), dtype=dt, device="cuda")
+           for _ in range(n_sets)]
+    res["down_factors"] = []
+    for i, (p, src, dst) in enumerate(((FFN_DOWN[0], hid, mid), (FFN_DOWN[1], mid, outs))):
+        def run(j, p=p, src=src, dst=dst, i=i):
+            Kernel.forward(src[j], f_dn[i], bs_last, *p, out=dst[j])
+
+        sec = time_launches(run, n_sets, steps, warmup)
+        roof = factor_roofline(BATCH, p, dt, dt, dt, sec)
+        res["down_factors"].append({"pattern": p, "us": sec * 1e6, "bound": roof["bound"],
+                                    "roofline_frac": roof["frac"], "floor_us": roof["floor_us"]})
+    # parity of the whole block on sampled rows
+    from oracle import ks_oracle as O
+    import numpy as np
+
+    ffn(0)
+    torch.cuda.synchronize()
+    rows = np.unique(np.concatenate([np.arange(0, BATCH, 397), np.arange(BATCH - 2, BATCH)]))
+    xr = xs[0].cpu().double().numpy()
+    xsub = xr[:, rows] if bs_last else xr[rows, :]
+    wr_up = [w.to(dt).double().numpy() for w in w_up]
+    wr_dn = [w.to(dt).double().numpy() for w in w_dn]
+    bu, bd = b_up.cpu().double().numpy(), b_dn.cpu().double().numpy()
+    h = O.chain_apply(wr_up, xsub, bs_last) + (bu[:, None] if bs_last else bu)
+    h = torch.nn.functional.gelu(torch.from_numpy(h)).to(dt).double().numpy()  # the hidden tensor is stored in `dt`
+    z = O.chain_apply(wr_dn, h, bs_last) + (bd[:, None] if bs_last else bd)
+    yh = outs[0].float().cpu().numpy()
+    ysub = yh[:, rows] if bs_last else yh[rows, :]
+    res["rel_fro_error"] = O.rel_fro_error(ysub, z)
+    res["tolerance"] = TOL[prec]
+    res["parity_ok"] = bool(res["rel_fro_error"] <= TOL[prec])
+    return res
+
+
 def bench_backward(name, pattern, prec, bs_last, steps, warmup):
     """µs of the input gradient (dX = K^T dY, on the forward kernels with transposed blocks) and of
     the weight gradient (dW = sum over the batch of dY x X^T per block, per-split partial sums added
@@ -512,6 +594,9 @@ def main():
     ap.add_argument("--backward", type=int, default=1,
                     help="also time the backward pass (input and weight gradients) of the headline factor and of "
                          "the ViT-B up-projection factors")
+    ap.add_argument("--ffn", type=int, default=1,
+                    help="also time the feed-forward block of the reference's ViT-S benchmark (up + bias + GELU, "
+                         "down + bias) in its default layout")
     ap.add_argument("--factor", default=None,
                     help="time one factor only, e.g. fp16:last:1,768,192,16 (per-kernel profiling runs); "
                          "prints that configuration's JSON instead of the headline line")
@@ -561,6 +646,7 @@ def main():
         backward.append(bench_backward("C2_bs_last", (1, 48, 48, 16), "fp32", True, bsteps, bwarm))
         backward.append(bench_backward("C4_vit_b_up_f0", (12, 64, 64, 1), "fp16", False, bsteps, bwarm))
         backward.append(bench_backward("C4_vit_b_up_f1", (1, 1536, 384, 2), "fp16", False, bsteps, bwarm))
+    ffn = bench_ffn(max(10, args.steps // 4), max(3, args.warmup // 4)) if args.ffn else None
     cpu = cpu_baseline(CONFIGS[0][1], True) if args.cpu else None
     if args.cpu:
         # the same CPU algorithm beside every other configuration (fp32 on the host, whatever the
@@ -595,6 +681,7 @@ def main():
                    "ok": head.get("parity_ok")},
         "configs": [head] + others,
         "backward": backward,
+        "ffn": ffn,
         "wall_s": time.time() - t_start,
     }
     print(json.dumps(line))

@@ -28,11 +28,13 @@ template <typename CT, int N> struct alignas(N * sizeof(CT)) pack_t {
     CT e[N];
 };
 
-template <typename CT, typename TW, int DD, int TM, int TN, int TK, int WM, int WN> struct BfCfg {
+// TX: the input's type in memory when it is not the compute type (e4m3fn, decoded to fp16 while the
+// vectors are split into the planes)
+template <typename CT, typename TW, int DD, int TM, int TN, int TK, int WM, int WN, typename TX = CT> struct BfCfg {
     static constexpr int THREADS = 64 * WM * WN;
     static constexpr int KSTEP = compute<CT>::KSTEP;
     static constexpr int MT = TM / WM / 32, NT = TN / WN / 32;
-    static constexpr int EPV = 16 / (int)sizeof(CT);  // elements per 16-byte input vector
+    static constexpr int EPV = 16 / (int)sizeof(TX);  // elements per 16-byte input vector
     static constexpr int KPV = EPV / DD;              // consecutive k per input vector
     static constexpr int LDW = pads<CT>::outer(TM);
     static constexpr int LDK = pads<CT>::inner(TK);
@@ -47,14 +49,18 @@ template <typename CT, typename TW, int DD, int TM, int TN, int TK, int WM, int 
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-template <typename CT, typename TW, typename TY, int DD, int TM, int TN, int TK, int WM, int WN>
-__global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__restrict__ x,
+__device__ __forceinline__ half_t bf_decode(half_t v) { return v; }
+__device__ __forceinline__ float bf_decode(float v) { return v; }
+__device__ __forceinline__ half_t bf_decode(fp8_t v) { return fp8_to_half(v.bits); }
+
+template <typename CT, typename TW, typename TY, int DD, int TM, int TN, int TK, int WM, int WN, typename TX = CT>
+__global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const TX *__restrict__ x,
                                                                  const TW *__restrict__ w,
                                                                  TY *__restrict__ y, int batch, int a,
                                                                  int b, int c, int d, Epi ep,
                                                                  int m_tiles, int n_tiles, int blocks)
 {
-    typedef BfCfg<CT, TW, DD, TM, TN, TK, WM, WN> C;
+    typedef BfCfg<CT, TW, DD, TM, TN, TK, WM, WN, TX> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     CT *const lds = (CT *)smem;
     auto ws = [&](int buf, int dd) { return lds + buf * C::W_ELEMS + dd * TK * C::LDW; };
@@ -76,7 +82,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
-    const CT *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
+    const TX *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
 
     stage<TW, CT> wreg[C::W_PER_T];
     uint4_t xreg[C::X_PER_T];
@@ -121,12 +127,12 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const CT *__re
                 const int vpr = TK * DD / C::EPV;
                 const int nn = v / vpr, kk = (v % vpr) * C::KPV;
                 // split the vector by d_i: element e is (k = kk + e / DD, d_i = e % DD)
-                pack_t<CT, C::EPV> all = __builtin_bit_cast(pack_t<CT, C::EPV>, xreg[i]);
+                pack_t<TX, C::EPV> all = __builtin_bit_cast(pack_t<TX, C::EPV>, xreg[i]);
 #pragma unroll
                 for (int dd = 0; dd < DD; ++dd) {
                     pack_t<CT, C::KPV> part;
 #pragma unroll
-                    for (int q = 0; q < C::KPV; ++q) part.e[q] = all.e[q * DD + dd];
+                    for (int q = 0; q < C::KPV; ++q) part.e[q] = bf_decode(all.e[q * DD + dd]);
                     *(pack_t<CT, C::KPV> *)(xs(buf, dd) + nn * C::LDK + kk) = part;
                 }
             }
@@ -653,6 +659,10 @@ struct BfInst {
 #define BF_INST(COMBO_, CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_)                                  \
     {COMBO_, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, BfCfg<CT_, TW_, DD_, TM_, TN_, TK_, WM_, WN_>::LDS_BYTES, WM_, \
      (const void *)ks_tile_bf_kernel<CT_, TW_, CT_, DD_, TM_, TN_, TK_, WM_, WN_>}
+// e4m3fn input and weights, fp16 planes and output
+#define BF_INST_Q(DD_, TM_, TN_, TK_, WM_, WN_)                                                   \
+    {2, DD_, TM_, TN_, TK_, 64 * WM_ * WN_, BfCfg<half_t, fp8_t, DD_, TM_, TN_, TK_, WM_, WN_, fp8_t>::LDS_BYTES, WM_, \
+     (const void *)ks_tile_bf_kernel<half_t, fp8_t, half_t, DD_, TM_, TN_, TK_, WM_, WN_, fp8_t>}
 #define BF_SET_H(COMBO_, TW_)                                                                    \
     BF_INST(COMBO_, half_t, TW_, 2, 128, 128, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 2, 256, 128, 32, 2, 2), \
         BF_INST(COMBO_, half_t, TW_, 2, 128, 256, 32, 2, 2), BF_INST(COMBO_, half_t, TW_, 2, 64, 128, 32, 1, 4), \
@@ -690,6 +700,11 @@ const BfInst bf_insts[] = {
     BF4_INST(64, 128, 2, 4, 2, 2),
     // e4m3 input and weights: groups of 8 again (8-byte vectors, decoded on their way to LDS)
     BF8_SET(2, fp8_t, fp8_t),
+    // e4m3 input and weights, d = 2 or 4 whole (a 16-byte vector is 8 or 4 k of every d_i)
+    // ((1,768,192,2) at batch 25088: 62 us on the 64 x 128 tile, 67-71 on the larger ones; about
+    // what the transposed route takes, without its workspace)
+    BF_INST_Q(2, 64, 128, 32, 1, 4), BF_INST_Q(2, 128, 128, 32, 2, 2), BF_INST_Q(2, 256, 128, 32, 2, 2),
+    BF_INST_Q(2, 32, 128, 32, 1, 4), BF_INST_Q(4, 64, 128, 32, 1, 4), BF_INST_Q(4, 32, 128, 32, 1, 4),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
