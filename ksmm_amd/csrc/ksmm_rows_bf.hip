@@ -212,16 +212,16 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *_
 // when an operand is picked out of LDS or loaded as a weight), fp32 accumulation, fp16
 // output.  Row segments travel as 16-byte vectors (8 halves / 16 e4m3), so c * DD and b * DD
 // must be multiples of the vector (and DD itself when d > DD: runs of DD elements).
-template <typename TX, int BB, int CC, int DD, int TN> struct RowCfgH {
-    static constexpr int NW = DD, THREADS = 64 * NW;
+template <typename TX, int BB, int CC, int DD, int TN, int MS = 1> struct RowCfgH {
+    static constexpr int NW = DD * MS, THREADS = 64 * NW;
     static constexpr int ES = (int)sizeof(TX), EPV = 16 / ES;   // input element, elements per vector
-    static constexpr int MT = BB / 16, KS = CC / 16, NT = TN / 16;
+    static constexpr int MT = BB / 16 / MS, KS = CC / 16, NT = TN / 16;
     static constexpr int XROW = CC * DD, OROW = BB * DD;         // elements per row segment
     static constexpr int LDX = XROW + EPV, LDO = OROW + 8;       // padded LDS rows (elements)
     static constexpr int X_VECS = TN * XROW / EPV, O_VECS = TN * OROW / 8;
     static constexpr int X_PER_T = (X_VECS + THREADS - 1) / THREADS, O_PER_T = (O_VECS + THREADS - 1) / THREADS;
     static constexpr int X_BYTES = 2 * TN * LDX * ES, LDS_BYTES = X_BYTES + TN * LDO * 2;
-    static_assert(BB % 16 == 0 && CC % 16 == 0 && TN % 16 == 0, "MFMA tiling");
+    static_assert(BB % (16 * MS) == 0 && CC % 16 == 0 && TN % 16 == 0, "MFMA tiling");
     static_assert(NW <= 16 && XROW % EPV == 0 && OROW % 8 == 0, "shape");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
@@ -229,12 +229,12 @@ template <typename TX, int BB, int CC, int DD, int TN> struct RowCfgH {
 __device__ __forceinline__ half_t row_to_half(half_t v) { return v; }
 __device__ __forceinline__ half_t row_to_half(fp8_t v) { return fp8_to_half(v.bits); }
 
-template <typename TX, int BB, int CC, int DD, int TN, bool AG = false>
-__global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restrict__ x, const TX *__restrict__ w,
+template <typename TX, int BB, int CC, int DD, int TN, bool AG = false, int MS = 1>
+__global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_h_kernel(const TX *__restrict__ x, const TX *__restrict__ w,
                                                               half_t *__restrict__ y, int batch, int a, int d,
                                                               Epi ep, int wgs_per_a, int n_tiles)
 {
-    typedef RowCfgH<TX, BB, CC, DD, TN> C;
+    typedef RowCfgH<TX, BB, CC, DD, TN, MS> C;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     TX *const xs = (TX *)smem;                         // [2][TN][LDX]
     half_t *const os = (half_t *)(smem + C::X_BYTES);  // [TN][LDO]
@@ -245,14 +245,16 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
-    const int dd = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's d_i inside the group
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ms = wv / DD, dd = wv - ms * DD;  // this wave's row group of the block and its d_i inside the group
+    const int m_off = ms * (BB / MS);
     const size_t in_size = (size_t)a * CC * d, out_size = (size_t)a * BB * d;
 
     // weights of block (a_i, d0 + dd): element (k, m) at ((a_i*d + d0 + dd)*c + k)*b + m;
-    // A operand of sub-step ks: lane (r, q) holds k = 16*ks + 4*q .. + 3 of row m = 16*mt + r
+    // A operand of sub-step ks: lane (r, q) holds k = 16*ks + 4*q .. + 3 of row m = m_off + 16*mt + r
     half4_t wreg[C::MT][C::KS];
     {
-        const TX *wg = w + (size_t)(AG ? a_i + dd : a_i * d + d0 + dd) * CC * BB;
+        const TX *wg = w + (size_t)(AG ? a_i + dd : a_i * d + d0 + dd) * CC * BB + m_off;
 #pragma unroll
         for (int ks = 0; ks < C::KS; ++ks)
 #pragma unroll
@@ -265,8 +267,8 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
     for (int mt = 0; mt < C::MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            bv[mt][i] = epi_bias<half_t>(ep, AG ? (size_t)(a_i + dd) * BB + 16 * mt + 4 * q + i
-                                                : ((size_t)a_i * BB + 16 * mt + 4 * q + i) * d + d0 + dd);
+            bv[mt][i] = epi_bias<half_t>(ep, AG ? (size_t)(a_i + dd) * BB + m_off + 16 * mt + 4 * q + i
+                                                : ((size_t)a_i * BB + m_off + 16 * mt + 4 * q + i) * d + d0 + dd);
 
     const TX *xg = x + (size_t)a_i * CC * d + d0;
     half_t *yg = y + (size_t)a_i * BB * d + d0;
@@ -326,8 +328,8 @@ __global__ __launch_bounds__(64 * DD) void ks_rows_bf_h_kernel(const TX *__restr
             for (int nt = 0; nt < C::NT; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    os[AG ? (16 * nt + r) * C::LDO + dd * BB + 16 * mt + 4 * q + i
-                          : (16 * nt + r) * C::LDO + (16 * mt + 4 * q + i) * DD + dd] = (half_t)epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
+                    os[AG ? (16 * nt + r) * C::LDO + dd * BB + m_off + 16 * mt + 4 * q + i
+                          : (16 * nt + r) * C::LDO + (m_off + 16 * mt + 4 * q + i) * DD + dd] = (half_t)epi_finish(ep, acc[mt][nt][i], bv[mt][i]);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::O_PER_T; ++i) {
@@ -387,6 +389,13 @@ struct RowInst {
     M(16, 16, 2, 128), M(16, 16, 1, 128)
 #define ROW_SET_AG32(M) M(16, 16, 16, 16), M(16, 16, 16, 32), M(16, 16, 8, 32), M(16, 16, 4, 64), M(32, 32, 8, 16), M(32, 32, 4, 32), \
     M(16, 16, 2, 64), M(16, 16, 1, 128)
+// 16-bit: MS_ waves per d_i, each with BB_ / MS_ rows of the block
+#define ROW_INST_H_MS(BB_, CC_, DD_, TN_, MS_) \
+    {1, BB_, CC_, DD_, TN_, RowCfgH<half_t, BB_, CC_, DD_, TN_, MS_>::LDS_BYTES, 8, 1, \
+     (const void *)ks_rows_bf_h_kernel<half_t, BB_, CC_, DD_, TN_, false, MS_>, 0, MS_}
+#define ROW_INST_Q_MS(BB_, CC_, DD_, TN_, MS_) \
+    {2, BB_, CC_, DD_, TN_, RowCfgH<fp8_t, BB_, CC_, DD_, TN_, MS_>::LDS_BYTES, 16, 1, \
+     (const void *)ks_rows_bf_h_kernel<fp8_t, BB_, CC_, DD_, TN_, false, MS_>, 0, MS_}
 #define ROW_SET_AG_B(M) \
     M(48, 48, 4, 32), M(48, 48, 2, 64), M(48, 48, 1, 64), M(64, 64, 4, 32), M(64, 64, 2, 64), M(64, 64, 4, 64), \
     M(96, 96, 2, 32), M(96, 96, 4, 16), M(64, 64, 1, 64), M(32, 32, 2, 64), M(32, 32, 1, 128)
@@ -456,6 +465,18 @@ const RowInst row_insts[] = {
     ROW_SET_AG32_B(ROW_INST_AG),
     ROW_SET_AG_B(ROW_INST_AG_H),
     ROW_SET_AG_B(ROW_INST_AG_Q),
+    // 16-bit 128 x 128 blocks, three per workgroup, several waves per block
+    // ((1,128,128,3) at batch 25088, fp16: 24.0 us on one wave per block, 15.6 on four with 32-row
+    // tiles, 18-19 on two; e4m3 33.4 -> 18.8)
+    ROW_INST_H_MS(128, 128, 3, 32, 4), ROW_INST_H_MS(128, 128, 3, 32, 2), ROW_INST_H_MS(128, 128, 3, 16, 2),
+    ROW_INST_H_MS(128, 128, 3, 16, 4),
+    ROW_INST_Q_MS(128, 128, 3, 32, 4), ROW_INST_Q_MS(128, 128, 3, 32, 2), ROW_INST_Q_MS(128, 128, 3, 16, 2),
+    ROW_INST_Q_MS(128, 128, 3, 16, 4),
+    // the same for groups of 4 and 2 blocks
+    ROW_INST_H_MS(128, 128, 4, 16, 4), ROW_INST_H_MS(128, 128, 4, 32, 4), ROW_INST_H_MS(128, 128, 2, 32, 4),
+    ROW_INST_H_MS(128, 128, 2, 32, 8),
+    ROW_INST_Q_MS(128, 128, 4, 16, 4), ROW_INST_Q_MS(128, 128, 4, 32, 4), ROW_INST_Q_MS(128, 128, 2, 32, 4),
+    ROW_INST_Q_MS(128, 128, 2, 32, 8),
 };
 constexpr int N_ROW_INSTS = sizeof(row_insts) / sizeof(RowInst);
 constexpr int ROW_INST_BITS = 10, ROW_INST_ANY = (1 << ROW_INST_BITS) - 1;
@@ -487,6 +508,9 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
         const RowInst &t = row_insts[i];
         if (t.combo != combo || t.bb != p.b || t.cc != p.c) continue;
         if (want == ROW_INST_ANY && t.planes) continue;  // named by the table (or forced) only
+        // 16-bit groups of 2 and 4 blocks on several waves per block: no faster than one wave per
+        // block (fp16 (16,128,128,2) 150 against 138 us, (4,128,128,4) 78 against 70), named only
+        if (want == ROW_INST_ANY && t.ms > 1 && combo != 0 && t.dd != 3) continue;
         // row segments start on 16-byte boundaries (output vectors: 4 floats / 8 halves)
         const int ovec = combo == 0 ? 4 : 8;
         if (((int64_t)p.a * p.c * p.d) % t.vec || ((int64_t)p.a * p.b * p.d) % ovec) continue;
@@ -521,8 +545,11 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             // measured 10-55 % faster than the 32- and 64-row tiles for d <= 8), except for
             // 128 x 128 blocks, whose weights take longer to read than a small tile to multiply
             // ((1,128,128,3) at batch 25088: fp16 28.8 us with 16 rows, 23.9 with 32; e4m3 42.2 / 33.3)
+            // (and more waves per block before larger tiles: 15.6 us on four waves per block)
             const bool larger = t.bb * t.cc >= 128 * 128;
-            if (pick < 0 || row_insts[pick].dd != p.d || (larger ? t.tn > row_insts[pick].tn : t.tn < row_insts[pick].tn))
+            const RowInst *cur = pick >= 0 ? &row_insts[pick] : nullptr;
+            if (!cur || cur->dd != p.d ||
+                (larger ? (t.ms > cur->ms || (t.ms == cur->ms && t.tn > cur->tn)) : t.tn < cur->tn))
                 pick = i;
         } else if (pick >= 0 && row_insts[pick].dd == p.d) {
             // an exact match was found already

@@ -284,9 +284,10 @@ def test_row_kernel_instances_forced():
     cases = [("fp8", False, p, batch) for p in shapes16 for batch in (512, 203)]
     _forced_sweep(cases, [1000 + i for i in list(range(61, 97)) + list(range(125, 143))], 2, 40)
     # three 128 x 128 blocks per workgroup (fp32: two waves per d_i), 16 x 16 blocks in groups of four
-    late = [(2, 128, 128, 3), (1, 128, 128, 3), (3, 16, 16, 4), (16, 16, 16, 4)]
+    late = [(2, 128, 128, 3), (1, 128, 128, 3), (3, 16, 16, 4), (16, 16, 16, 4), (1, 128, 128, 4), (2, 128, 128, 2),
+            (1, 128, 128, 8)]
     for prec in ("fp32", "fp16", "fp8"):
-        _forced_sweep([(prec, False, p, batch) for p in late for batch in (512, 203)], [1000 + i for i in range(158, 172)], 2,
+        _forced_sweep([(prec, False, p, batch) for p in late for batch in (512, 203)], [1000 + i for i in list(range(158, 172)) + list(range(222, 238))], 2,
                       4 if prec == "fp32" else 16)
     # d = 1: groups of consecutive a_i (16 x 16 and 32 x 32 blocks), every group size that divides a
     ag = [(64, 16, 16, 1), (48, 16, 16, 1), (12, 16, 16, 1), (6, 16, 16, 1), (3, 16, 16, 1), (16, 32, 32, 1),
