@@ -287,7 +287,7 @@ def test_row_kernel_instances_forced():
     late = [(2, 128, 128, 3), (1, 128, 128, 3), (3, 16, 16, 4), (16, 16, 16, 4), (1, 128, 128, 4), (2, 128, 128, 2),
             (1, 128, 128, 8)]
     for prec in ("fp32", "fp16", "fp8"):
-        _forced_sweep([(prec, False, p, batch) for p in late for batch in (512, 203)], [1000 + i for i in list(range(158, 172)) + list(range(222, 238))], 2,
+        _forced_sweep([(prec, False, p, batch) for p in late for batch in (512, 203)], [1000 + i for i in list(range(158, 172)) + list(range(222, 240))], 2,
                       4 if prec == "fp32" else 16)
     # d = 1: groups of consecutive a_i (16 x 16 and 32 x 32 blocks), every group size that divides a
     ag = [(64, 16, 16, 1), (48, 16, 16, 1), (12, 16, 16, 1), (6, 16, 16, 1), (3, 16, 16, 1), (16, 32, 32, 1),
