@@ -765,6 +765,15 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             // transposes move each operand once more, the GEMM tiles run at 2-3x its
             // matrix-core rate)
             if (p.d == t.dd && combo != 0 && p.b >= 512 && (int64_t)p.b * p.c >= 512 * 512) continue;
+            // e4m3 input with d = 2 or 4 whole: measured against the transposed route on the 102
+            // such patterns of the reference's list (batch 25088), the direct kernel wins (time
+            // ratio 0.6-0.97) with short c or narrow blocks and loses (1.1-2.3) elsewhere: the
+            // e4m3 GEMM tiles in the middle of the other route multiply at twice the rate
+            if (combo == 2 && !t.pd) {
+                const bool pays = p.d == 2 ? (p.c <= 128 || (p.c <= 256 && p.b <= 512))
+                                           : (p.c <= 96 || (p.b <= 64 && p.a >= 3));
+                if (!pays) continue;
+            }
             if (p.d != t.dd) {
                 const int64_t bd = (int64_t)p.b * p.d;
                 const bool pays = combo == 0 ? ((p.d <= 16 && p.b <= 192) || (bd <= 8192 && (p.d <= 16 || p.c <= 128)))
