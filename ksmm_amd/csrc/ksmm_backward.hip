@@ -34,16 +34,33 @@ __global__ __launch_bounds__(256) void ks_block_transpose_kernel(const T *__rest
     out[i] = in[(g * c + ci) * b + bi];
 }
 
-// dw[i] = scale * (slice 0 + slice 1 + ... in that order); slices are n floats apart
+// dw[i] = scale * (sum of the slices); slices are n floats apart.  A workgroup takes 64 outputs;
+// its four 64-thread groups add a quarter of the slices each, in slice order (eight loads in
+// flight per thread), and the four partial sums are added in group order: the association is
+// fixed by (splits) alone, so the result has the same bits on every run.
 template <typename T>
 __global__ __launch_bounds__(256) void ks_wgrad_finish_kernel(const float *__restrict__ acc, T *__restrict__ dw,
                                                               int64_t n, int splits, float scale)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    float s = acc[i];
-    for (int k = 1; k < splits; ++k) s += acc[(int64_t)k * n + i];
-    dw[i] = (T)(s * scale);
+    __shared__ float part[4][64];
+    const int g = threadIdx.x >> 6, l = threadIdx.x & 63;
+    const int64_t i = (int64_t)blockIdx.x * 64 + l;
+    const int per = (splits + 3) / 4, k0 = g * per, k1 = min(k0 + per, splits);
+    float s = 0.f;
+    if (i < n) {
+        int k = k0;
+        for (; k + 8 <= k1; k += 8) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = acc[(int64_t)(k + j) * n + i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s += v[j];
+        }
+        for (; k < k1; ++k) s += acc[(int64_t)k * n + i];
+    }
+    part[g][l] = s;
+    __syncthreads();
+    if (g == 0 && i < n) dw[i] = (T)((((part[0][l] + part[1][l]) + part[2][l]) + part[3][l]) * scale);
 }
 
 template <typename T> struct wg_vec;
@@ -217,6 +234,125 @@ template <typename T> int launch_block_transpose(const void *w, void *wt, int64_
 
 // Batch splits of the two weight-gradient kernels (every split is non-empty and writes a slice of
 // a*b*c*d partial sums of its own): columns per split and their number.
+// Weight gradient of large fp16 blocks (b and c multiples of 128), batch-size-last operands: a
+// 128 x 128 tile of one block's gradient and a range of batch columns per workgroup (4 waves, 2 x 2,
+// 64 x 64 each on v_mfma_f32_32x32x16_f16).  Both operands have the batch axis contiguous, so a slab
+// of 64 columns is 128 rows x 128 bytes per operand: it goes through registers into LDS (16-byte
+// chunks, the chunk index XORed with row / 2 so that the operand reads of 16 consecutive rows hit
+// different banks), double-buffered, one barrier per slab.  Against the wave-per-tile kernel above,
+// which re-reads every operand row once per 64 x 64 tile through L2 (1.85 GB for (1,1536,384,2) at
+// batch 25088), the traffic drops to a quarter.  D = X-rows x dY-rows^T, so a lane holds one output
+// feature m (contiguous in kernel format) and 16 inputs k.
+constexpr int WG_TM = 128, WG_TN = 128, WG_TK = 64;
+__global__ __launch_bounds__(256, 2) void ks_wgrad_gemm_h_kernel(const half_t *__restrict__ dy,
+                                                                 const half_t *__restrict__ x,
+                                                                 float *__restrict__ acc_out, int batch, int a, int b,
+                                                                 int c, int d, int m_tiles, int n_tiles, int splits,
+                                                                 int cols, int64_t slice)
+{
+    __shared__ __attribute__((aligned(16))) half_t sa[2][WG_TM * WG_TK], sb[2][WG_TN * WG_TK];
+    int id = blockIdx.x;
+    const int split = id % splits;
+    id /= splits;
+    const int mt = id % m_tiles;
+    id /= m_tiles;
+    const int nt = id % n_tiles, g = id / n_tiles;
+    const int a_i = g / d, d_i = g - a_i * d;
+    const int m0 = mt * WG_TM, n0 = nt * WG_TN;
+    const int k_begin = split * cols, k_end = min(k_begin + cols, batch);
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lq = lane >> 5;
+    const int wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    // staging: 4 vectors per operand and thread; vector v = tid + 256 * i is row v / 8, physical
+    // chunk v % 8, which holds the logical chunk (v % 8) ^ ((row / 2) % 8)
+    const half_t *ga[4], *gb[4];
+    int lcol[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int v = tid + 256 * i, row = v >> 3, lc = (v & 7) ^ ((row >> 1) & 7);
+        lcol[i] = lc * 8;
+        ga[i] = dy + ((size_t)(a_i * b + m0 + row) * d + d_i) * batch + lc * 8;
+        gb[i] = x + ((size_t)(a_i * c + n0 + row) * d + d_i) * batch + lc * 8;
+    }
+    uint4_t ra[4], rb[4];
+    auto gload = [&](int k) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool in = k + lcol[i] < k_end;  // (k_end is a multiple of 8)
+            ra[i] = in ? *(const uint4_t *)(ga[i] + k) : uint4_t{0u, 0u, 0u, 0u};
+            rb[i] = in ? *(const uint4_t *)(gb[i] + k) : uint4_t{0u, 0u, 0u, 0u};
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *(uint4_t *)(sa[buf] + (tid + 256 * i) * 8) = ra[i];
+            *(uint4_t *)(sb[buf] + (tid + 256 * i) * 8) = rb[i];
+        }
+    };
+    float16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    if (k_begin < k_end) {
+        gload(k_begin);
+        lstore(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int k = k_begin; k < k_end; k += WG_TK) {
+        const bool more = k + WG_TK < k_end;
+        if (more) gload(k + WG_TK);
+#pragma unroll
+        for (int ks = 0; ks < WG_TK / 16; ++ks) {
+            half8_t fx[2], fy[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int rx = wn * 64 + i * 32 + l32, ry = wm * 64 + i * 32 + l32;
+                fx[i] = *(const half8_t *)(sb[buf] + (rx * 8 + ((2 * ks + lq) ^ ((rx >> 1) & 7))) * 8);
+                fy[i] = *(const half8_t *)(sa[buf] + (ry * 8 + ((2 * ks + lq) ^ ((ry >> 1) & 7))) * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx[i], fy[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) lstore(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    // D[k'][m]: lane l32 = output feature m, rows k' = 8 * (e / 4) + 4 * lq + e % 4
+    float *out = acc_out + (size_t)split * slice + (size_t)g * c * b;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int kk = n0 + wn * 64 + i * 32 + 8 * (e >> 2) + 4 * lq + (e & 3);
+                const int m = m0 + wm * 64 + j * 32 + l32;
+                out[(size_t)kk * b + m] = acc[i][j][e];
+            }
+}
+
+bool wgrad_gemm_ok(int b, int c, int dtype) { return dtype == KSMM_F16 && b % WG_TM == 0 && c % WG_TN == 0; }
+
+// batch ranges of the tiled kernel: two workgroups per CU, at least 8 slabs each
+void wgrad_gemm_splits(int64_t batch, int64_t tiles, int64_t *splits_out, int64_t *cols_out)
+{
+    int64_t splits = (512 + tiles - 1) / tiles;
+    const int64_t max_splits = (batch + 8 * WG_TK - 1) / (8 * WG_TK);
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    int64_t cols = (batch + splits - 1) / splits;
+    cols = (cols + WG_TK - 1) / WG_TK * WG_TK;
+    *splits_out = (batch + cols - 1) / cols;
+    *cols_out = cols;
+}
+
 void wgrad_bl_splits(int64_t batch, int64_t tiles, int step, int64_t *splits_out, int64_t *cols_out)
 {
     // about 16 waves per CU; at least 4 loop iterations per wave
@@ -299,6 +435,22 @@ int launch_wgrad_tiled(const void *dy, const void *x, float *acc, int64_t batch,
     return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
 }
 
+int launch_wgrad_gemm(const void *dy, const void *x, float *acc, int64_t batch, int a, int b, int c, int d,
+                      hipStream_t s, int *splits_used)
+{
+    const int m_tiles = b / WG_TM, n_tiles = c / WG_TN;
+    const int64_t tiles = (int64_t)a * d * m_tiles * n_tiles;
+    int64_t splits, cols;
+    wgrad_gemm_splits(batch, tiles, &splits, &cols);
+    const int64_t blocks = tiles * splits;
+    if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
+    *splits_used = (int)splits;
+    hipLaunchKernelGGL(ks_wgrad_gemm_h_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const half_t *)dy,
+                       (const half_t *)x, acc, (int)batch, a, b, c, d, m_tiles, n_tiles, (int)splits, (int)cols,
+                       (int64_t)a * b * c * d);
+    return hipGetLastError() == hipSuccess ? KSMM_OK : KSMM_ERR_LAUNCH;
+}
+
 }  // namespace
 
 // wt <- the b x c blocks of w transposed: kernel format (a*d*b, c) of pattern (a, c, b, d)
@@ -326,6 +478,10 @@ int64_t wgrad_partial_floats(int64_t batch, int a, int b, int c, int d, int dtyp
     if (splits > most) most = splits;
     wgrad_tiled_splits(batch, (int64_t)a * d * ((b + 15) / 16) * ((c + 15) / 16), &splits, &cols);
     if (splits > most) most = splits;
+    if (wgrad_gemm_ok(b, c, dtype)) {
+        wgrad_gemm_splits(batch, (int64_t)a * d * (b / WG_TM) * (c / WG_TN), &splits, &cols);
+        if (splits > most) most = splits;
+    }
     return most * n;
 }
 
@@ -335,7 +491,7 @@ int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch
               int dtype, int bs_last, float scale, hipStream_t stream, int *kernel_used)
 {
     const int64_t n = (int64_t)a * b * c * d;
-    const int64_t fin_blocks = (n + 255) / 256;
+    const int64_t fin_blocks = (n + 63) / 64;
     if (fin_blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     const bool mfma_ok = wgrad_mfma_ok(dy, x, batch, b, c, d, dtype, bs_last);
     if (kernel_used) *kernel_used = mfma_ok ? 1 : 0;
@@ -350,7 +506,9 @@ int wgrad_run(const void *dy, const void *x, void *dw, float *acc, int64_t batch
         else
             rc = launch_wgrad_tiled<float>(dy, x, acc, batch, a, b, c, d, bs_last, stream, &splits);
     } else if (dtype == KSMM_F16) {
-        if (mfma_ok)
+        if (mfma_ok && wgrad_gemm_ok(b, c, dtype))
+            rc = launch_wgrad_gemm(dy, x, acc, batch, a, b, c, d, stream, &splits);
+        else if (mfma_ok)
             rc = t == 1   ? launch_wgrad_bl<half_t, 1, 1>(dy, x, acc, batch, a, b, c, d, stream, &splits)
                  : t == 2 ? launch_wgrad_bl<half_t, 2, 2>(dy, x, acc, batch, a, b, c, d, stream, &splits)
                  : t == 3 ? launch_wgrad_bl<half_t, 3, 3>(dy, x, acc, batch, a, b, c, d, stream, &splits)

@@ -767,6 +767,8 @@ BACKWARD_CASES = [
     # pattern, batch: MFMA weight-gradient tiles of 16, 32, 48 and 64, ragged b / c, d > 1, odd batch
     ((1, 48, 48, 16), 1040), ((6, 64, 64, 1), 520), ((2, 3, 5, 4), 203), ((1, 96, 48, 2), 264), ((3, 16, 16, 4), 528),
     ((1, 256, 64, 2), 520), ((2, 77, 64, 1), 520), ((1, 17, 33, 2), 64), ((2, 32, 32, 3), 1000), ((1, 192, 192, 16), 264),
+    # fp16: the 128 x 128 tiles of the GEMM-shaped weight gradient (several tiles per block, d > 1, ragged last slab)
+    ((1, 256, 128, 2), 520), ((2, 128, 128, 1), 1000), ((1, 128, 256, 3), 264), ((1, 384, 128, 1), 4168),
 ]
 
 
@@ -803,7 +805,8 @@ def test_weight_gradient_is_bit_reproducible(bs_last):
     from ksmm_amd import Kernel, generate_factor
     from ksmm_amd.layer import from_kernel_format_to_abcd
 
-    for prec, pattern, batch in [("fp32", (1, 48, 48, 16), 25088), ("fp16", (2, 64, 96, 3), 8200), ("fp32", (3, 20, 12, 2), 4099)]:
+    for prec, pattern, batch in [("fp32", (1, 48, 48, 16), 25088), ("fp16", (2, 64, 96, 3), 8200), ("fp32", (3, 20, 12, 2), 4099),
+                                 ("fp16", (1, 256, 128, 2), 8200)]:
         a, b, c, d = pattern
         dt = TORCH_DTYPE[prec]
         (w4,) = seeded_weights([pattern], seed=101)
