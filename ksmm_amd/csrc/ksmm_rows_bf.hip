@@ -69,11 +69,26 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_kernel(const float *_
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *const xs = (float *)smem;                // [2][TN][LDX]; PL: [2][DD][PLANE_X]
     float *const os = xs + 2 * C::X_FLOATS;         // [TN][LDO]; PL: [DD][PLANE_O]
-    // blockIdx -> (a_i, group of DD d_i, share of the tiles); AG: a_i is the group's first block
+    // The d / DD workgroups that take the same tiles of one a_i read the same lines (a group's run
+    // of DD elements is a piece of every line of a row): they get block indices that are equal
+    // mod 8, i.e. one XCD and its L2.  (Dealt without that, whenever the workgroups per a_i are
+    // not a multiple of 8, every XCD fetched the lines for its piece: (3,64,64,64) fp16 took 927 us
+    // where (4,64,64,64) takes 425.)
     const int groups = AG ? 1 : d / DD;
-    const int ag = blockIdx.x / wgs_per_a;
-    const int s = blockIdx.x - ag * wgs_per_a;
-    const int a_i = AG ? ag * DD : ag / groups, d0 = AG ? 0 : (ag - a_i * groups) * DD;
+    int a_i, d0, s;
+    if (AG) {
+        const int ag = blockIdx.x / wgs_per_a;
+        s = blockIdx.x - ag * wgs_per_a;
+        a_i = ag * DD;
+        d0 = 0;
+    } else {
+        const int slot = blockIdx.x >> 3, grp = slot % groups;
+        const int u = (slot / groups) * 8 + (blockIdx.x & 7);  // (a_i, share) pairs, 8 at a time
+        if (u >= a * wgs_per_a) return;
+        a_i = u / wgs_per_a;
+        s = u - a_i * wgs_per_a;
+        d0 = grp * DD;
+    }
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
@@ -238,10 +253,26 @@ __global__ __launch_bounds__(64 * DD * MS) void ks_rows_bf_h_kernel(const TX *__
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     TX *const xs = (TX *)smem;                         // [2][TN][LDX]
     half_t *const os = (half_t *)(smem + C::X_BYTES);  // [TN][LDO]
+    // The d / DD workgroups that take the same tiles of one a_i read the same lines (a group's run
+    // of DD elements is a piece of every line of a row): they get block indices that are equal
+    // mod 8, i.e. one XCD and its L2.  (Dealt without that, whenever the workgroups per a_i are
+    // not a multiple of 8, every XCD fetched the lines for its piece: (3,64,64,64) fp16 took 927 us
+    // where (4,64,64,64) takes 425.)
     const int groups = AG ? 1 : d / DD;
-    const int ag = blockIdx.x / wgs_per_a;
-    const int s = blockIdx.x - ag * wgs_per_a;
-    const int a_i = AG ? ag * DD : ag / groups, d0 = AG ? 0 : (ag - a_i * groups) * DD;
+    int a_i, d0, s;
+    if (AG) {
+        const int ag = blockIdx.x / wgs_per_a;
+        s = blockIdx.x - ag * wgs_per_a;
+        a_i = ag * DD;
+        d0 = 0;
+    } else {
+        const int slot = blockIdx.x >> 3, grp = slot % groups;
+        const int u = (slot / groups) * 8 + (blockIdx.x & 7);  // (a_i, share) pairs, 8 at a time
+        if (u >= a * wgs_per_a) return;
+        a_i = u / wgs_per_a;
+        s = u - a_i * wgs_per_a;
+        d0 = grp * DD;
+    }
     const int t_begin = s, t_end = n_tiles, t_step = wgs_per_a;  // every wgs-th tile
     if (t_begin >= t_end) return;
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r = lane & 15;
@@ -574,7 +605,8 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     if (wgs <= 0) wgs = 256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves) / ag;
     if (wgs <= 0) wgs = 1;
     if (wgs > n_tiles) wgs = n_tiles;
-    const int64_t grid = ag * wgs;
+    // (groups of one a_i that take the same tiles sit 8 block indices apart: see the kernels)
+    const int64_t grid = t.ag ? ag * wgs : 8 * (int64_t)(p.d / t.dd) * (((int64_t)p.a * wgs + 7) / 8);
     if (grid > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
         tile->algo = KSMM_ALGO_WAVE;
