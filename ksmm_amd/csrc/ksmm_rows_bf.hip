@@ -602,7 +602,13 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     const int nw = t.dd * t.ms;
     const int per_cu_lds = 160 * 1024 / t.lds, per_cu_waves = 16 / nw > 0 ? 16 / nw : 1;
     // (rounded down: a few workgroups beyond one round would cost a whole second round)
-    if (wgs <= 0) wgs = 256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves) / ag;
+    if (wgs <= 0) {
+        const int64_t round = 256 * (per_cu_lds < per_cu_waves ? per_cu_lds : per_cu_waves);
+        wgs = round / ag;
+        // the grid below is 8 * groups * ceil(a * wgs / 8) workgroups: keep that within the round too
+        const int64_t groups = t.ag ? 1 : p.d / t.dd, units = 8 * (round / (8 * groups));
+        if (!t.ag && units >= p.a && wgs > units / p.a) wgs = units / p.a;
+    }
     if (wgs <= 0) wgs = 1;
     if (wgs > n_tiles) wgs = n_tiles;
     // (groups of one a_i that take the same tiles sit 8 block indices apart: see the kernels)
