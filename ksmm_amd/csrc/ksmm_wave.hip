@@ -121,7 +121,15 @@ __global__ __launch_bounds__(256, OCC) void ks_wave_bl_f32(const float *__restri
     // row group h of it, the groups of a block then reading the same input rows.
     const int m_split = b / (16 * MT);
     int gh, slab;
-    if (m_split % wpw) {
+    if (m_split > 1 && wpw % m_split == 0) {
+        // two or four row groups: the groups of a (block, share) are neighbouring waves of one
+        // workgroup (one CU reads the rows once)
+        const int unit = (int)blockIdx.x * (wpw / m_split) + wv / m_split;
+        if (unit >= a * d * n_slabs) return;
+        const int gb = unit / n_slabs;
+        slab = unit - gb * n_slabs;
+        gh = gb * m_split + wv % m_split;
+    } else if (m_split % wpw) {
         const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * wpw + wv);
         gh = wave / n_slabs;
         slab = wave - gh * n_slabs;
@@ -340,13 +348,24 @@ __global__ __launch_bounds__(512, 1) void ks_wave_ring_f32(const float *__restri
     const int lane = threadIdx.x & 63;
     const int q = lane >> 4, r = lane & 15;
     const int wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + wave_in_wg);
+    const int wpw = (int)(blockDim.x >> 6);
     const int m_split = b / (16 * MT);
-    const int gh = wave / n_slabs;
+    int gh, slab;
+    if (m_split > 1 && wpw % m_split == 0) {
+        // row groups of a (block, share): neighbouring waves of one workgroup
+        const int unit = (int)blockIdx.x * (wpw / m_split) + wave_in_wg / m_split;
+        if (unit >= a * d * n_slabs) return;
+        const int gb = unit / n_slabs;
+        slab = unit - gb * n_slabs;
+        gh = gb * m_split + wave_in_wg % m_split;
+    } else {
+        const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * wpw + wave_in_wg);
+        gh = wave / n_slabs;
+        slab = wave - gh * n_slabs;
+    }
     const int g = gh / m_split;  // block index a_i * d + d_i
     if (g >= a * d) return;
     const int m_off = (gh - g * m_split) * (16 * MT);
-    const int slab = wave - gh * n_slabs;
     const int a_i = g / d, d_i = g - a_i * d;
     // tiles of this wave: every n_slabs-th tile of the block's row of tiles, so that the waves of
     // a workgroup read neighbouring 256-byte pieces of the same rows at any one time
@@ -885,7 +904,7 @@ int wave_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
     // row groups in multiples of the workgroup: the groups of a (block, share) get workgroup
     // indices that are equal mod 8 (see the kernel); the grid is padded to whole sets of 8
     const int64_t m_split = p.b / in.b;
-    if (combo == 0 && !in.ring && m_split > 1 && m_split % wpb == 0)
+    if (combo == 0 && !in.ring && m_split > wpb && m_split % wpb == 0)
         blocks = 8 * (m_split / wpb) * (((int64_t)p.a * p.d * n_slabs + 7) / 8);
     if (blocks > 0x7fffffffLL) return KSMM_ERR_TOO_LARGE;
     if (tile) {
