@@ -84,6 +84,14 @@ template <> struct frag<half_t> {
         short8_t r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return __builtin_bit_cast(half8_t, r);
     }
+    // the operand of the 8-k step: k = k0 + 4 * (lane / 32) .. + 3 of column lane % 32
+    __device__ static __forceinline__ half4_t k_outer4(const half_t *s, int ld, int idx0, int k0, int lane)
+    {
+        const int kq = lane >> 5, i16 = lane & 15, half_sel = (lane >> 4) & 1;
+        const half_t *p = s + (k0 + 4 * kq + (i16 >> 2)) * ld + idx0 + 16 * half_sel + 4 * (i16 & 3);
+        typedef short4_t __attribute__((address_space(3))) * lds_ptr;
+        return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p)));
+    }
     __device__ static __forceinline__ half8_t k_inner(const half_t *s, int ld, int idx0, int k0, int lane)
     {
         return *(const half8_t *)(s + (idx0 + (lane & 31)) * ld + k0 + 8 * (lane >> 5));

@@ -219,32 +219,57 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const TX *__re
 //  * the planes are unpadded rows of 16 k, their two 16-byte halves swapped for rows 8..15 of
 //    every 16 (the 16 rows a 16-byte operand read covers then fall on distinct banks);
 // which brings LDS to 72 KB: two workgroups per CU, four slabs of 32 KB in flight.
-template <typename TX, typename TW, int TM, int TN, int WM, int WN, int PDX, int PDW>
-__global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_bf8_kernel(const TX *__restrict__ x,
+// NG > 1: the workgroup takes NG neighbouring groups of 8 blocks with NG times the waves (each set
+// of WM x WN waves multiplies one group), in slabs of TK = 8 (planes of 64 or 32 blocks at 16 k
+// would not leave room for two LDS buffers; one 4-k MFMA step per slab and block).  With groups
+// of 8 out of d = 64 a line of x is asked for by 8 workgroups for 16 bytes each, and a line of
+// results is written in 8 pieces at 8 different times: that scatter, not the bytes, is what the
+// groups of 8 wait for (fp16 (6,192,192,64) at batch 25088: 5.3 ms, and 2.5 ms when the same
+// kernel reads and writes the same number of bytes as whole lines).  Here
+//  * neighbouring lanes read the vectors of neighbouring groups: runs of 16 * NG bytes per
+//    (row, k), whole runs of 8 k when the workgroup covers d;
+//  * the results leave through LDS ([n][m][group], 16-byte pieces, the group xor-ed with m so
+//    that neighbouring lanes fall on distinct banks): runs of 16 * NG bytes per (row, m), or of
+//    TM * d * 2 bytes when the workgroup covers d;
+//  * the planes of a group start 256 / NG bytes apart in the banks (the lanes of one 4-byte
+//    store differ in the group first).
+// The accumulators of a workgroup are 8 * NG * TM * TN floats in 128 registers of 512 lanes, so
+// the tile shrinks as NG grows and weights and rows are read again more often: 32 blocks
+// (64-byte runs) on a 64 x 32 tile are the best trade (3.85 ms on the pattern above; 64 blocks
+// on 32 x 32: 4.6 ms; 16 blocks on 64 x 64 without the staged results: 5.4 ms).
+template <typename TX, typename TW, int TM, int TN, int WM, int WN, int PDX, int PDW, int NG = 1, int TK = 16>
+__global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) void ks_tile_bf8_kernel(const TX *__restrict__ x,
                                                                 const TW *__restrict__ w,
                                                                 half_t *__restrict__ y, int batch, int a,
                                                                 int b, int c, int d, Epi ep,
                                                                 int m_tiles, int n_tiles, int blocks)
 {
-    constexpr int DD = 8, TK = 16, THREADS = 64 * WM * WN;
+    constexpr int DD = 8, DDA = DD * NG, KH = TK / 2, THREADS = 64 * WM * WN * NG;
+    constexpr bool FL = NG > 1;  // whole lines: results leave through LDS
+    constexpr int NBUF = 2;
+    static_assert(TK == 16 || TK == 8, "one MFMA step per slab");
     constexpr int MT = TM / WM / 32, NT = TN / WN / 32;
-    constexpr int LDW = pads<half_t>::outer(TM);
-    constexpr int W_ELEMS = DD * TK * LDW, X_ELEMS = DD * TN * TK;
+    constexpr int LDW = TM == 32 ? 32 : pads<half_t>::outer(TM);  // (rows of 64 bytes: 4 k are 256 bytes, no padding needed)
+    // (the chunks of a group start 256 / NG bytes apart in the banks: the lanes of one 4-byte store
+    // differ in the chunk first)
+    constexpr int XPAD = NG > 1 ? 128 / NG : 0;
+    constexpr int W_ELEMS = DDA * TK * LDW, X_ELEMS = DDA * TN * TK + NG * XPAD;
     constexpr int W_EPV = stage<TW, half_t>::EPV;
-    constexpr int W_VECS = DD * TK * TM / W_EPV, W_PER_T = W_VECS / THREADS;
-    constexpr int X_QUADS = TN * TK / 2, XQ_PER_T = X_QUADS / THREADS;  // pairs (k, k + 8) of a row
+    constexpr int W_VECS = DDA * TK * TM / W_EPV, W_PER_T = W_VECS / THREADS;
+    constexpr int X_QUADS = NG * TN * TK / 2, XQ_PER_T = X_QUADS / THREADS;  // pairs (k, k + KH) of a row and chunk
     static_assert(W_VECS % THREADS == 0 && X_QUADS % THREADS == 0, "whole loads per thread");
     static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0, "wave tiling");
-    static_assert(2 * (W_ELEMS + X_ELEMS) * 2 <= (WM * WN >= 8 ? 160 : 80) * 1024, "8 waves per CU");
+    static_assert(NBUF * (W_ELEMS + X_ELEMS) * 2 <= (WM * WN * NG >= 8 ? 160 : 80) * 1024, "8 waves per CU");
+    static_assert((NG & (NG - 1)) == 0 && NG <= 8 && (!FL || TM * TN * DDA * 2 <= 160 * 1024), "chunks of a group");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     half_t *const lds = (half_t *)smem;
     auto ws = [&](int buf, int dd) { return lds + buf * W_ELEMS + dd * TK * LDW; };
-    auto xs = [&](int buf, int dd) { return lds + 2 * W_ELEMS + buf * X_ELEMS + dd * TN * TK; };
+    auto xs = [&](int buf, int dd) { return lds + NBUF * W_ELEMS + buf * X_ELEMS + dd * TN * TK + (dd >> 3) * XPAD; };
 
     const int per_xcd = (blocks + 7) / 8;
     const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (lid >= blocks) return;
-    const int n_dg = d / DD;  // groups of DD blocks
+    const int n_dg = d / DDA;  // groups of DDA blocks
     const int mt_id = lid % m_tiles;
     int rest = lid / m_tiles;
     const int dg = rest % n_dg;
@@ -253,7 +278,7 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     const int a_i = rest / n_tiles;
     const int m0 = mt_id * TM, n0 = nt_id * TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
+    const int wg = wave / (WM * WN), wm = wave / WN % WM, wn = wave % WN;  // wg: the wave's chunk of 8 blocks
     const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
 
     stage<TW, half_t> wreg[PDW][W_PER_T];
@@ -266,8 +291,8 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     // (live == false) every lane reads the first 16 bytes of the tile instead (one line): the
     // offsets are masked, not selected, so that no branch comes back.  Addresses are a uniform
     // base per tile plus a 32-bit offset per lane (the host checks that they fit).
-    const TW *const wt = w + ((size_t)(a_i * d + dg * DD) * c) * b + m0;
-    const TX *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DD;
+    const TW *const wt = w + ((size_t)(a_i * d + dg * DDA) * c) * b + m0;
+    const TX *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DDA;
     uint32_t woff[W_PER_T], xoff[XQ_PER_T];
 #pragma unroll
     for (int i = 0; i < W_PER_T; ++i) {
@@ -280,8 +305,9 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
 #pragma unroll
     for (int i = 0; i < XQ_PER_T; ++i) {
         const int v = tid + i * THREADS;
-        const int nn = v >> 3, k8 = v & 7;
-        xoff[i] = (uint32_t)(min(nn, batch - 1 - n0) * (uint32_t)in_size + k8 * d);
+        // the chunk runs fastest: neighbouring lanes read neighbouring vectors of one line
+        const int g = v % NG, k8 = v / NG % KH, nn = v / (KH * NG);
+        xoff[i] = (uint32_t)(min(nn, batch - 1 - n0) * (uint32_t)in_size + k8 * d + g * DD);
     }
     auto live_mask = [](bool live) {
         int lv = live;
@@ -299,7 +325,7 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
         for (int i = 0; i < XQ_PER_T; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                xreg[slot][i][j] = *(const xvec_t *)(xt + ((xoff[i] + (uint32_t)((k0 + 8 * j) * d)) & mk));
+                xreg[slot][i][j] = *(const xvec_t *)(xt + ((xoff[i] + (uint32_t)((k0 + KH * j) * d)) & mk));
     };
     auto lstore = [&](int wslot, int slot, int buf) {
 #pragma unroll
@@ -308,15 +334,17 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
             constexpr int per_dd = TK * TM / W_EPV;
             const int dd = v / per_dd, r = v % per_dd;
             const int kk = r / (TM / W_EPV), mm = (r % (TM / W_EPV)) * W_EPV;
-            wreg[wslot][i].store(ws(buf, dd) + (2 * (kk & 7) + (kk >> 3)) * LDW + mm);
+            wreg[wslot][i].store(ws(buf, dd) + (2 * (kk % KH) + kk / KH) * LDW + mm);
         }
 #pragma unroll
         for (int i = 0; i < XQ_PER_T; ++i) {
             const int v = tid + i * THREADS;
-            const int nn = v >> 3, k8 = v & 7;
+            const int g = v % NG, k8 = v / NG % KH, nn = v / (KH * NG);
             // k = k8 and k8 + 8 of row nn: positions 2 * k8 and 2 * k8 + 1, i.e. 4-byte piece k8 & 3
             // of the 16-byte half k8 >> 2 (swapped for rows 8..15 of every 16)
-            half_t *const dst = xs(buf, 0) + nn * TK + ((((k8 >> 2) ^ ((nn >> 3) & 1)) << 3) | ((k8 & 3) << 1));
+            // (TK = 8: k = k8 and k8 + 4 at positions 2 * k8 and 2 * k8 + 1 of a 16-byte row)
+            half_t *const dst = xs(buf, g * DD) + nn * TK +
+                                (TK == 16 ? ((((k8 >> 2) ^ ((nn >> 3) & 1)) << 3) | ((k8 & 3) << 1)) : (k8 << 1));
             uint4_t c0, c1;  // register p: d_i = 2p (low half) and 2p + 1 (high half), as fp16
             if constexpr (sizeof(TX) == 2) {
                 c0 = xreg[slot][i][0];
@@ -354,21 +382,35 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int n = (wn * NT + j) * 32 + l32;
-        xrow[j] = n * TK + ((lq ^ ((n >> 3) & 1)) << 3);
+        xrow[j] = TK == 16 ? n * TK + ((lq ^ ((n >> 3) & 1)) << 3) : n * TK + 4 * lq;
     }
     auto multiply = [&](int buf) {
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd) {
-            const half_t *wb = ws(buf, dd), *xb = xs(buf, dd);
-            half8_t fw[MT], fx[NT];
+            const half_t *wb = ws(buf, wg * DD + dd), *xb = xs(buf, wg * DD + dd);
+            if constexpr (TK == 16) {
+                half8_t fw[MT], fx[NT];
 #pragma unroll
-            for (int i = 0; i < MT; ++i) fw[i] = frag<half_t>::k_outer(wb, LDW, (wm * MT + i) * 32, 0, lane);
+                for (int i = 0; i < MT; ++i) fw[i] = frag<half_t>::k_outer(wb, LDW, (wm * MT + i) * 32, 0, lane);
 #pragma unroll
-            for (int j = 0; j < NT; ++j) fx[j] = *(const half8_t *)(xb + xrow[j]);
+                for (int j = 0; j < NT; ++j) fx[j] = *(const half8_t *)(xb + xrow[j]);
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+                for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < NT; ++j) acc[dd][i][j] = frag<half_t>::mfma(fx[j], fw[i], acc[dd][i][j]);
+                    for (int j = 0; j < NT; ++j) acc[dd][i][j] = frag<half_t>::mfma(fx[j], fw[i], acc[dd][i][j]);
+            } else {
+                // 8 k per slab: the lane's operand is 4 k (one transpose load, one 8-byte read)
+                half4_t fw[MT], fx[NT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i) fw[i] = frag<half_t>::k_outer4(wb, LDW, (wm * MT + i) * 32, 0, lane);
+#pragma unroll
+                for (int j = 0; j < NT; ++j) fx[j] = *(const half4_t *)(xb + xrow[j]);
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        acc[dd][i][j] = __builtin_amdgcn_mfma_f32_32x32x8f16(fx[j], fw[i], acc[dd][i][j], 0, 0, 0);
+            }
         }
     };
 
@@ -408,6 +450,40 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
 
     // D tile: lane holds output column m = lane % 32, batch rows 8*(e/4) + 4*(lane/32) + e%4;
     // the 8 results of one (n, m) are adjacent in y: one 16-byte store
+    if constexpr (FL) {
+        // the NG chunks of one (n, m) sit in NG waves and are adjacent in y, as are the m of one
+        // row when the group is all of d
+        uint4_t *const ot = (uint4_t *)smem;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const int ml = (wm * MT + i) * 32 + l32;
+                float bv[DD];
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd)
+                    bv[dd] = epi_bias<half_t>(ep, ((size_t)a_i * b + m0 + ml) * d + dg * DDA + wg * DD + dd);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int nl = (wn * NT + j) * 32 + 8 * (e >> 2) + 4 * lq + (e & 3);
+                    pack_t<half_t, DD> o;
+#pragma unroll
+                    for (int dd = 0; dd < DD; ++dd) o.e[dd] = (half_t)epi_finish(ep, acc[dd][i][j][e], bv[dd]);
+                    ot[(nl * TM + ml) * NG + (wg ^ (ml & (NG - 1)))] = __builtin_bit_cast(uint4_t, o);
+                }
+            }
+        __syncthreads();
+        constexpr int PIECES = TN * TM * NG;
+        static_assert(PIECES % THREADS == 0, "whole pieces per thread");
+#pragma unroll 4
+        for (int q = tid; q < PIECES; q += THREADS) {
+            const int ch = q % NG, ml = q / NG % TM, nl = q / (NG * TM);
+            if (n0 + nl < batch)
+                *(uint4_t *)(y + (size_t)(n0 + nl) * out_size + ((size_t)a_i * b + m0 + ml) * d + dg * DDA + ch * DD) =
+                    ot[(nl * TM + ml) * NG + (ch ^ (ml & (NG - 1)))];
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -651,6 +727,13 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
         }
 }
 
+// LDS of the whole-d form: one buffer of planes, or the staged result tile if that is larger
+constexpr int bf8l_lds(int ng, int tk, int tm, int tn)
+{
+    const int ldw = tm == 32 ? 32 : pads<half_t>::outer(tm);
+    const int planes = 2 * (2 * 8 * ng * (tk * ldw + tn * tk) + 256), out = tm * tn * 8 * ng * 2;
+    return planes > out ? planes : out;
+}
 struct BfInst {
     int combo, dd, tm, tn, tk, threads, lds, wm;
     const void *fn;
@@ -679,6 +762,10 @@ struct BfInst {
 #define BF4_INST(TM_, TN_, WM_, WN_, PDX_, PDW_)                                                 \
     {0, 4, TM_, TN_, 16, 64 * WM_ * WN_, 2 * 4 * (4 * 16 * TM_ + 4 * TN_ * 16), WM_,                 \
      (const void *)ks_tile_bf4_kernel<TM_, TN_, WM_, WN_, PDX_, PDW_>, PDX_ * 16 + PDW_}
+#define BF8L_INST(COMBO_, TX_, TW_, NG_, TK_, TM_, TN_, WM_, WN_, PDX_, PDW_)                         \
+    {COMBO_, 8 * NG_, TM_, TN_, TK_, 64 * WM_ * WN_ * NG_,                                       \
+     bf8l_lds(NG_, TK_, TM_, TN_), WM_,                                                          \
+     (const void *)ks_tile_bf8_kernel<TX_, TW_, TM_, TN_, WM_, WN_, PDX_, PDW_, NG_, TK_>, 256 + PDX_ * 16 + PDW_}
 #define BF8_SET(COMBO_, TX_, TW_)                                                                \
     BF8_INST(COMBO_, TX_, TW_, 64, 64, 2, 2, 2, 2), BF8_INST(COMBO_, TX_, TW_, 64, 128, 2, 4, 2, 2)
 const BfInst bf_insts[] = {
@@ -705,6 +792,13 @@ const BfInst bf_insts[] = {
     // what the transposed route takes, without its workspace)
     BF_INST_Q(2, 64, 128, 32, 1, 4), BF_INST_Q(2, 128, 128, 32, 2, 2), BF_INST_Q(2, 256, 128, 32, 2, 2),
     BF_INST_Q(2, 32, 128, 32, 1, 4), BF_INST_Q(4, 64, 128, 32, 1, 4), BF_INST_Q(4, 32, 128, 32, 1, 4),
+    // 32 or 16 blocks per workgroup (pipelined kernel with slabs of 8 k, 8 waves, one workgroup per CU)
+    BF8L_INST(1, half_t, half_t, 4, 8, 64, 32, 2, 1, 2, 2), BF8L_INST(1, half_t, half_t, 4, 8, 32, 64, 1, 2, 2, 2),
+    BF8L_INST(1, half_t, half_t, 2, 8, 64, 64, 2, 2, 2, 2),
+    BF8L_INST(3, half_t, fp8_t, 4, 8, 64, 32, 2, 1, 2, 2), BF8L_INST(3, half_t, fp8_t, 4, 8, 32, 64, 1, 2, 2, 2),
+    BF8L_INST(3, half_t, fp8_t, 2, 8, 64, 64, 2, 2, 2, 2),
+    BF8L_INST(2, fp8_t, fp8_t, 4, 8, 64, 32, 2, 1, 2, 2), BF8L_INST(2, fp8_t, fp8_t, 4, 8, 32, 64, 1, 2, 2, 2),
+    BF8L_INST(2, fp8_t, fp8_t, 2, 8, 64, 64, 2, 2, 2, 2),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
@@ -716,7 +810,7 @@ bool bf_fits(const BfInst &t, const Problem &p, int combo)
     // d > DD: the DD elements of one (row, k) must fill the 16-byte vector
     // (the pipelined e4m3 instances read 8-byte vectors: groups of 8 out of any multiple of 8)
     const int vec = (t.pd && combo == 2) ? 8 : x_epv;
-    if (p.d != t.dd && t.dd != vec) return false;
+    if (p.d != t.dd && (t.pd ? t.dd % vec != 0 : t.dd != vec)) return false;
     if (p.b % w_epv) return false;
     // rows of x start at multiples of in_size, slabs at multiples of TK * d: keep 16-byte alignment
     if (((int64_t)p.a * p.c * p.d) % vec || ((int64_t)p.c * p.d) % vec) return false;
@@ -774,10 +868,24 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
                                            : (p.c <= 96 || (p.b <= 64 && p.a >= 3));
                 if (!pays) continue;
             }
+            const bool wide = t.pd >= 256;  // 32 or 16 blocks per workgroup
+            if (wide) {
+                // Measured against the groups of 8 and the row kernel on the 141 patterns of the
+                // reference's lists with d a multiple of 16 (batch 25088, fp16 and e4m3): 32 blocks
+                // win from d = 64 on (time ratio 0.62-0.93) and, fp16, at d = 32 with short c
+                // (0.88-0.90); 16 blocks win where d is not a multiple of 32 (d = 48: 0.79-0.98),
+                // fp16 at d = 32 with longer c (0.77-0.90) and at d = 16 on wide short blocks
+                // (0.90-0.97); elsewhere the groups of 8 stay within 3 %.
+                const bool fits32 = p.d % 32 == 0 && (p.d >= 64 || (combo != 2 && p.c <= 128));
+                const bool pays = t.dd == 32 ? fits32
+                                             : (!fits32 && ((p.d % 32 != 0 && p.d >= 48) || (combo != 2 && p.d == 32) ||
+                                                            (p.d == 16 && p.b >= 384 && p.c <= 192)));
+                if (!pays) continue;
+            }
             if (p.d != t.dd) {
                 const int64_t bd = (int64_t)p.b * p.d;
                 const bool pays = combo == 0 ? ((p.d <= 16 && p.b <= 192) || (bd <= 8192 && (p.d <= 16 || p.c <= 128)))
-                                             : (t.tm >= 64 && ((p.d <= 32 && p.b <= 384) ||
+                                             : ((t.tm >= 64 || wide) && ((p.d <= 32 && p.b <= 384) ||
                                                                (p.c <= 256 && (p.b <= 192 ? p.d <= 128 : bd <= 12288))));
                 if (!pays) continue;
             }
@@ -785,7 +893,8 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             int64_t score = (int64_t)t.tm * 1000 + t.tn;
             // the pipelined 64 x 64 form first (1.1-1.3x the plain instances on (1,192,192,8..16),
             // (4,128,128,8), (1,64,64,64) at batch 25088)
-            if (t.pd && t.tn == 64 && wgs >= 512) score += 500000;
+            if (t.pd && !wide && t.tn == 64 && wgs >= 512) score += 500000;
+            if (wide && wgs >= 512) score += 600000;
             if (wgs < 512) score -= 100000;
             if (score > best) {
                 best = score;

@@ -104,7 +104,7 @@ def _sample_cols(batch, n=48):
     return np.array(sorted(idx))
 
 
-def tune_pattern(pattern, prec, bs_last, batch, lib_mod, rotation_bytes=1.3e9):
+def tune_pattern(pattern, prec, bs_last, batch, lib_mod, rotation_bytes=1.3e9, tile_subs=None):
     from . import Kernel, generate_factor, quantize_fp8
     from .kernel import query_tile, variant_id
     from .layer import from_kernel_format_to_abcd
@@ -163,7 +163,16 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, rotation_bytes=1.3e9):
     steps = int(min(40, max(6, 1.5e-3 / max(t_auto, 1e-6))))
     results = []
     tried_any = False
-    for pool in (candidates(bs_last, combo), kloop_candidates(combo, bs_last)):
+    pools = (candidates(bs_last, combo), kloop_candidates(combo, bs_last))
+    if tile_subs is not None:
+        # a retune after instances were added to some tile sub-families: only those, against what
+        # the present table (or, without a row, the heuristic) picks
+        now = query_tile(batch, pattern, dt, dt, bs_last)
+        pool = [(al, v) for al, v in pools[0] if al == 3 and (v >> 24) in tile_subs]
+        if now["algo"] in (2, 3) and (now["algo"], now["variant"]) not in pool:
+            pool.append((now["algo"], now["variant"]))
+        pools = (pool,)
+    for pool in pools:
         for algo, variant in pool:
             try:
                 y = run(algo, variant)
@@ -380,6 +389,8 @@ def main():
     ap.add_argument("--update-best", help="directory of existing *.best files: replace the lines of the measured patterns")
     ap.add_argument("--shard", default="0/1", help="i/n: take every n-th pattern starting at i")
     ap.add_argument("--time-limit", type=float, default=1e9, help="stop (and save) after this many seconds")
+    ap.add_argument("--tile-subs", help="comma-separated tile sub-families (2 stream, 4 GEMM, 1 weight-stationary, "
+                    "3 d > 1 tiles): try only their instances and the present table's pick")
     args = ap.parse_args()
     entries = []
     for p in args.merge:
@@ -407,7 +418,8 @@ def main():
                     if time.time() - t_start > args.time_limit:
                         break
                     try:
-                        e = tune_pattern(p, prec, bs_last, args.batch, _lib)
+                        e = tune_pattern(p, prec, bs_last, args.batch, _lib,
+                                         tile_subs=[int(v) for v in args.tile_subs.split(",")] if args.tile_subs else None)
                     except torch.cuda.OutOfMemoryError:
                         print("  OOM", p, prec, layout, flush=True)
                         torch.cuda.empty_cache()

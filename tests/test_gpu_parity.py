@@ -133,6 +133,35 @@ def test_tile_bf_groups_of_blocks_forced():
     assert ran >= 30 and strided >= 12, (ran, strided)
 
 
+def test_tile_bf_wide_groups_forced():
+    """Batch-size-first tile kernel on 32 or 16 neighbouring blocks per workgroup (instances 41..49:
+    slabs of 8 k, results staged through LDS): d whole and a multiple of the group, 32- and 64-row
+    tiles, several a_i, ragged batches (the last batch tile partly empty, fewer rows than a tile),
+    1 to 24 slabs; fp16, fp16 with e4m3 weights, e4m3 input and weights; with a bias."""
+    from ksmm_amd import Kernel, generate_factor
+
+    shapes = [((1, 64, 64, 32), 520), ((2, 64, 8, 32), 77), ((1, 32, 24, 64), 203), ((3, 96, 40, 32), 100),
+              ((1, 64, 192, 16), 264), ((2, 128, 16, 48), 31), ((1, 192, 96, 64), 130), ((1, 64, 72, 128), 65)]
+    variants = [(3 << 24) | i for i in range(41, 50)]
+    for prec, min_ran in (("fp16", 14), ("hq", 14), ("fp8", 14)):
+        _forced_sweep([(prec, False, p, n) for p, n in shapes], variants, 3, min_ran)
+    # the automatic choice with a bias (applied before the results are staged)
+    from ksmm_amd.kernel import query_tile
+
+    a, b, c, d = 1, 128, 48, 64
+    batch = 4100
+    pick = query_tile(batch, (a, b, c, d), torch.float16, torch.float16, False)
+    assert pick["algo"] == 3 and pick["tile_d"] == 32 and pick["threads"] == 512, pick
+    (w4,) = seeded_weights([(a, b, c, d)], seed=61)
+    x = seeded_input(a * c * d, batch, False, seed=62)
+    bias = (torch.rand(a * b * d, generator=torch.Generator().manual_seed(6)) - 0.5).half()
+    fac = generate_factor(a, b, c, d, "kernel", w4, torch.float16, "cuda")
+    z = O.ks_apply_einsum(round_to(w4, "fp16")[0], round_to(x, "fp16")[0], False) + bias.double().numpy()[None, :]
+    y = Kernel.forward(x.half().cuda(), fac, False, a, b, c, d, bias=bias.cuda())
+    err = O.rel_fro_error(y.float().cpu().numpy(), z)
+    assert err <= TOL["fp16"], err
+
+
 def test_wave_row_groups_forced():
     """fp32 wave instance for 32-row blocks forced on 64-row blocks (two row groups per block,
     variant 7 | tiles-per-wave << 8 | dealing << 16), with a_i, d_i > 1, ragged batches and a bias."""
