@@ -566,6 +566,15 @@ int rows_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             continue;
         }
         if (p.d == 1) continue;
+        // 96 x 96 blocks and larger with d a multiple of 16 from 32 on (fp32) or of 32 from 64 on
+        // (16-bit input): the tile kernel's groups of 16 / 32 blocks are faster at large batches
+        // (fp32 (a,96,96,64) 0.64-0.82 of this kernel's time at batch 25088, (1,96,96,96) 0.61; fp16
+        // (12,96,96,64) 0.68)
+        // (within what that kernel takes before the transposed route: b * d <= 8192 in fp32, d <= 128)
+        if (want == ROW_INST_ANY && t.bb >= 96 && t.bb <= 192 && t.cc >= 96 && t.cc <= 256 && p.batch >= 8192 &&
+            (combo == 0 ? p.d >= 32 && p.d % 16 == 0 && (int64_t)p.b * p.d <= 8192
+                        : p.d >= 64 && p.d % 32 == 0 && p.d <= 128))
+            continue;
         // all d blocks in one workgroup, or groups of dd whose runs keep the 16-byte alignment
         const bool grouped_ok = t.dd % t.vec == 0 && t.dd % ovec == 0 && p.d % t.dd == 0;
         const int run_bytes = t.dd * (combo == 0 ? 4 : 2);  // output run of a group

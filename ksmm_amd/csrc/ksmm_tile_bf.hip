@@ -513,33 +513,40 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
 // 16 floats, element k of row n at k ^ 2 * ((n / 4) % 8): the 32 rows an operand read covers
 // fall on distinct banks.  Weight rows are unpadded too: the columns of odd k are XORed with 32,
 // so the two rows an operand read covers use different bank halves.
-template <int TM, int TN, int WM, int WN, int PDX, int PDW>
-__global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_bf4_kernel(const float *__restrict__ x,
+// NG > 1: NG neighbouring groups of 4 blocks per workgroup with NG times the waves, slabs of 8 k,
+// results staged through LDS, as in the 16-bit kernel above (runs of 16 * NG bytes both ways).
+template <int TM, int TN, int WM, int WN, int PDX, int PDW, int NG = 1, int TK = 16>
+__global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) void ks_tile_bf4_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ w,
                                                                 float *__restrict__ y, int batch, int a,
                                                                 int b, int c, int d, Epi ep,
                                                                 int m_tiles, int n_tiles, int blocks)
 {
     typedef float TW;
-    constexpr int DD = 4, TK = 16, THREADS = 64 * WM * WN;
+    constexpr int DD = 4, DDA = DD * NG, KH = TK / 2, THREADS = 64 * WM * WN * NG;
+    constexpr bool FL = NG > 1;  // several groups per workgroup: results leave through LDS
+    constexpr int XPAD = NG > 1 ? 64 / NG : 0;  // the groups start 256 / NG bytes apart in the banks
+    static_assert(TK == 16 || TK == 8, "slab depth");
     constexpr int MT = TM / WM / 32, NT = TN / WN / 32;
     constexpr int LDW = TM;  // unpadded: columns of odd rows are XORed with 32 instead
-    constexpr int W_ELEMS = DD * TK * LDW, X_ELEMS = DD * TN * TK;
+    constexpr int WSW = TM >= 64 ? 32 : 0;  // (rows of 32 floats: two rows are the two bank halves as they are)
+    constexpr int W_ELEMS = DDA * TK * LDW, X_ELEMS = DDA * TN * TK + NG * XPAD;
     constexpr int W_EPV = stage<float, float>::EPV;
-    constexpr int W_VECS = DD * TK * TM / W_EPV, W_PER_T = W_VECS / THREADS;
-    constexpr int X_QUADS = TN * TK / 2, XQ_PER_T = X_QUADS / THREADS;  // pairs (k, k + 8) of a row
+    constexpr int W_VECS = DDA * TK * TM / W_EPV, W_PER_T = W_VECS / THREADS;
+    constexpr int X_QUADS = NG * TN * TK / 2, XQ_PER_T = X_QUADS / THREADS;  // pairs (k, k + KH) of a row and group
     static_assert(W_VECS % THREADS == 0 && X_QUADS % THREADS == 0, "whole loads per thread");
     static_assert(TM % (32 * WM) == 0 && TN % (32 * WN) == 0, "wave tiling");
-    static_assert(2 * (W_ELEMS + X_ELEMS) * 4 <= (WM * WN >= 8 ? 160 : 80) * 1024, "8 waves per CU");
+    static_assert(2 * (W_ELEMS + X_ELEMS) * 4 <= (WM * WN * NG >= 8 ? 160 : 80) * 1024, "8 waves per CU");
+    static_assert((NG & (NG - 1)) == 0 && NG <= 8 && (!FL || TM * TN * DDA * 4 <= 160 * 1024), "groups of a workgroup");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *const lds = (float *)smem;
     auto ws = [&](int buf, int dd) { return lds + buf * W_ELEMS + dd * TK * LDW; };
-    auto xs = [&](int buf, int dd) { return lds + 2 * W_ELEMS + buf * X_ELEMS + dd * TN * TK; };
+    auto xs = [&](int buf, int dd) { return lds + 2 * W_ELEMS + buf * X_ELEMS + dd * TN * TK + (dd >> 2) * XPAD; };
 
     const int per_xcd = (blocks + 7) / 8;
     const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (lid >= blocks) return;
-    const int n_dg = d / DD;  // groups of DD blocks
+    const int n_dg = d / DDA;  // groups of DDA blocks
     const int mt_id = lid % m_tiles;
     int rest = lid / m_tiles;
     const int dg = rest % n_dg;
@@ -548,9 +555,8 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     const int a_i = rest / n_tiles;
     const int m0 = mt_id * TM, n0 = nt_id * TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
+    const int wg = wave / (WM * WN), wm = wave / WN % WM, wn = wave % WN;  // wg: the wave's group of 4 blocks
     const size_t in_size = (size_t)a * c * d, out_size = (size_t)a * b * d;
-    const float *xg = x + (size_t)a_i * c * d + dg * DD;  // + n * in_size + k * d + dd
 
     stage<float, float> wreg[PDW][W_PER_T];
     uint4_t xreg[PDX][XQ_PER_T][2];
@@ -560,8 +566,8 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     // (live == false) every lane reads the first 16 bytes of the tile instead (one line): the
     // offsets are masked, not selected, so that no branch comes back.  Addresses are a uniform
     // base per tile plus a 32-bit offset per lane (the host checks that they fit).
-    const TW *const wt = w + ((size_t)(a_i * d + dg * DD) * c) * b + m0;
-    const float *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DD;
+    const TW *const wt = w + ((size_t)(a_i * d + dg * DDA) * c) * b + m0;
+    const float *const xt = x + (size_t)n0 * in_size + (size_t)a_i * c * d + dg * DDA;
     uint32_t woff[W_PER_T], xoff[XQ_PER_T];
 #pragma unroll
     for (int i = 0; i < W_PER_T; ++i) {
@@ -574,8 +580,9 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
 #pragma unroll
     for (int i = 0; i < XQ_PER_T; ++i) {
         const int v = tid + i * THREADS;
-        const int nn = v >> 3, k8 = v & 7;
-        xoff[i] = (uint32_t)(min(nn, batch - 1 - n0) * (uint32_t)in_size + k8 * d);
+        // the group runs fastest: neighbouring lanes read neighbouring vectors of one line
+        const int g = v % NG, k8 = v / NG % KH, nn = v / (KH * NG);
+        xoff[i] = (uint32_t)(min(nn, batch - 1 - n0) * (uint32_t)in_size + k8 * d + g * DD);
     }
     auto live_mask = [](bool live) {
         int lv = live;
@@ -593,7 +600,7 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
         for (int i = 0; i < XQ_PER_T; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                xreg[slot][i][j] = *(const uint4_t *)(xt + ((xoff[i] + (uint32_t)((k0 + 8 * j) * d)) & mk));
+                xreg[slot][i][j] = *(const uint4_t *)(xt + ((xoff[i] + (uint32_t)((k0 + KH * j) * d)) & mk));
     };
     auto lstore = [&](int wslot, int slot, int buf) {
 #pragma unroll
@@ -602,20 +609,20 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
             constexpr int per_dd = TK * TM / W_EPV;
             const int dd = v / per_dd, r = v % per_dd;
             const int kk = r / (TM / W_EPV), mm = (r % (TM / W_EPV)) * W_EPV;
-            wreg[wslot][i].store(ws(buf, dd) + kk * LDW + (mm ^ (32 * (kk & 1))));
+            wreg[wslot][i].store(ws(buf, dd) + kk * LDW + (mm ^ (WSW * (kk & 1))));
         }
 #pragma unroll
         for (int i = 0; i < XQ_PER_T; ++i) {
             const int v = tid + i * THREADS;
-            const int nn = v >> 3, k8 = v & 7;
-            // k = k8 and k8 + 8 of row nn, element k at k ^ 2 * ((nn / 4) % 8)
-            float *const dst = xs(buf, 0) + nn * TK;
-            const int fn = 2 * ((nn >> 2) & 7);
+            const int g = v % NG, k8 = v / NG % KH, nn = v / (KH * NG);
+            // k = k8 and k8 + KH of row nn, element k at k ^ 2 * ((nn / 4) % 8) (rows of 8 k: k ^ 2 * ((nn / 8) % 4))
+            float *const dst = xs(buf, g * DD) + nn * TK;
+            const int fn = TK == 16 ? 2 * ((nn >> 2) & 7) : 2 * ((nn >> 3) & 3);
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const uint4_t cj = xreg[slot][i][j];
 #pragma unroll
-                for (int dd = 0; dd < DD; ++dd) *(uint32_t *)(dst + dd * TN * TK + ((k8 + 8 * j) ^ fn)) = cj[dd];
+                for (int dd = 0; dd < DD; ++dd) *(uint32_t *)(dst + dd * TN * TK + ((k8 + KH * j) ^ fn)) = cj[dd];
             }
         }
     };
@@ -636,7 +643,7 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
     for (int j = 0; j < NT; ++j) {
         const int n = (wn * NT + j) * 32 + l32;
         xrow[j] = n * TK;
-        xfn[j] = 2 * ((n >> 2) & 7);
+        xfn[j] = TK == 16 ? 2 * ((n >> 2) & 7) : 2 * ((n >> 3) & 3);
     }
     // operands of MFMA step k0 + 2 are requested before the MFMAs of step k0 are issued
     auto multiply = [&](int buf) {
@@ -647,9 +654,9 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
             for (int j = 0; j < NT; ++j) xcol[j] = xrow[j] + ((k0 + lq) ^ xfn[j]);
 #pragma unroll
             for (int dd = 0; dd < DD; ++dd) {
-                const float *wb = ws(buf, dd), *xb = xs(buf, dd);
+                const float *wb = ws(buf, wg * DD + dd), *xb = xs(buf, wg * DD + dd);
 #pragma unroll
-                for (int i = 0; i < MT; ++i) rw[dd][i] = wb[(k0 + lq) * LDW + (((wm * MT + i) * 32 + l32) ^ (32 * lq))];
+                for (int i = 0; i < MT; ++i) rw[dd][i] = wb[(k0 + lq) * LDW + (((wm * MT + i) * 32 + l32) ^ (WSW * lq))];
 #pragma unroll
                 for (int j = 0; j < NT; ++j) rx[dd][j] = xb[xcol[j]];
             }
@@ -706,6 +713,40 @@ __global__ __launch_bounds__(64 * WM * WN, (WM * WN >= 8 ? 1 : 2)) void ks_tile_
 
     // D tile: lane holds output column m = lane % 32, batch rows 8*(e/4) + 4*(lane/32) + e%4;
     // the 4 results of one (n, m) are adjacent in y: one 16-byte store
+    if constexpr (FL) {
+        // the NG groups of one (n, m) sit in NG waves and are adjacent in y: the tile goes to LDS
+        // as [n][m][group] (16-byte pieces, the group xor-ed with m) and leaves in whole runs
+        uint4_t *const ot = (uint4_t *)smem;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const int ml = (wm * MT + i) * 32 + l32;
+                float bv[DD];
+#pragma unroll
+                for (int dd = 0; dd < DD; ++dd)
+                    bv[dd] = epi_bias<float>(ep, ((size_t)a_i * b + m0 + ml) * d + dg * DDA + wg * DD + dd);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int nl = (wn * NT + j) * 32 + 8 * (e >> 2) + 4 * lq + (e & 3);
+                    pack_t<float, DD> o;
+#pragma unroll
+                    for (int dd = 0; dd < DD; ++dd) o.e[dd] = epi_finish(ep, acc[dd][i][j][e], bv[dd]);
+                    ot[(nl * TM + ml) * NG + (wg ^ (ml & (NG - 1)))] = __builtin_bit_cast(uint4_t, o);
+                }
+            }
+        __syncthreads();
+        constexpr int PIECES = TN * TM * NG;
+        static_assert(PIECES % THREADS == 0, "whole pieces per thread");
+#pragma unroll 4
+        for (int q = tid; q < PIECES; q += THREADS) {
+            const int ch = q % NG, ml = q / NG % TM, nl = q / (NG * TM);
+            if (n0 + nl < batch)
+                *(uint4_t *)(y + (size_t)(n0 + nl) * out_size + ((size_t)a_i * b + m0 + ml) * d + dg * DDA + ch * DD) =
+                    ot[(nl * TM + ml) * NG + (ch ^ (ml & (NG - 1)))];
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -732,6 +773,11 @@ constexpr int bf8l_lds(int ng, int tk, int tm, int tn)
 {
     const int ldw = tm == 32 ? 32 : pads<half_t>::outer(tm);
     const int planes = 2 * (2 * 8 * ng * (tk * ldw + tn * tk) + 256), out = tm * tn * 8 * ng * 2;
+    return planes > out ? planes : out;
+}
+constexpr int bf4l_lds(int ng, int tk, int tm, int tn)
+{
+    const int planes = 2 * 4 * (4 * ng * (tk * tm + tn * tk) + 64), out = tm * tn * 4 * ng * 4;
     return planes > out ? planes : out;
 }
 struct BfInst {
@@ -766,6 +812,9 @@ struct BfInst {
     {COMBO_, 8 * NG_, TM_, TN_, TK_, 64 * WM_ * WN_ * NG_,                                       \
      bf8l_lds(NG_, TK_, TM_, TN_), WM_,                                                          \
      (const void *)ks_tile_bf8_kernel<TX_, TW_, TM_, TN_, WM_, WN_, PDX_, PDW_, NG_, TK_>, 256 + PDX_ * 16 + PDW_}
+#define BF4L_INST(NG_, TK_, TM_, TN_, WM_, WN_, PDX_, PDW_)                                           \
+    {0, 4 * NG_, TM_, TN_, TK_, 64 * WM_ * WN_ * NG_, bf4l_lds(NG_, TK_, TM_, TN_), WM_,            \
+     (const void *)ks_tile_bf4_kernel<TM_, TN_, WM_, WN_, PDX_, PDW_, NG_, TK_>, 256 + PDX_ * 16 + PDW_}
 #define BF8_SET(COMBO_, TX_, TW_)                                                                \
     BF8_INST(COMBO_, TX_, TW_, 64, 64, 2, 2, 2, 2), BF8_INST(COMBO_, TX_, TW_, 64, 128, 2, 4, 2, 2)
 const BfInst bf_insts[] = {
@@ -799,6 +848,8 @@ const BfInst bf_insts[] = {
     BF8L_INST(3, half_t, fp8_t, 2, 8, 64, 64, 2, 2, 2, 2),
     BF8L_INST(2, fp8_t, fp8_t, 4, 8, 64, 32, 2, 1, 2, 2), BF8L_INST(2, fp8_t, fp8_t, 4, 8, 32, 64, 1, 2, 2, 2),
     BF8L_INST(2, fp8_t, fp8_t, 2, 8, 64, 64, 2, 2, 2, 2),
+    // fp32: 16 or 8 blocks per workgroup (32 blocks on a 32 x 32 tile never won)
+    BF4L_INST(4, 8, 64, 32, 2, 1, 2, 2), BF4L_INST(4, 8, 32, 64, 1, 2, 2, 2), BF4L_INST(2, 8, 64, 64, 2, 2, 2, 2),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
@@ -869,7 +920,12 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
                 if (!pays) continue;
             }
             const bool wide = t.pd >= 256;  // 32 or 16 blocks per workgroup
-            if (wide) {
+            if (wide && combo == 0) {
+                // fp32, measured the same way on the 161 patterns with d a multiple of 8: the
+                // wider groups win from d = 16 on (0.61-0.98 of the time of the groups of 4; 8
+                // blocks on 64 x 64 where b allows, else 16 blocks on 32 x 64), not at d = 8
+                if (p.d < 16) continue;
+            } else if (wide) {
                 // Measured against the groups of 8 and the row kernel on the 141 patterns of the
                 // reference's lists with d a multiple of 16 (batch 25088, fp16 and e4m3): 32 blocks
                 // win from d = 64 on (time ratio 0.62-0.93) and, fp16, at d = 32 with short c

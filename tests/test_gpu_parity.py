@@ -134,7 +134,7 @@ def test_tile_bf_groups_of_blocks_forced():
 
 
 def test_tile_bf_wide_groups_forced():
-    """Batch-size-first tile kernel on 32 or 16 neighbouring blocks per workgroup (instances 41..49:
+    """Batch-size-first tile kernel on 32 or 16 neighbouring blocks per workgroup (instances 41..52:
     slabs of 8 k, results staged through LDS): d whole and a multiple of the group, 32- and 64-row
     tiles, several a_i, ragged batches (the last batch tile partly empty, fewer rows than a tile),
     1 to 24 slabs; fp16, fp16 with e4m3 weights, e4m3 input and weights; with a bias."""
@@ -145,6 +145,9 @@ def test_tile_bf_wide_groups_forced():
     variants = [(3 << 24) | i for i in range(41, 50)]
     for prec, min_ran in (("fp16", 14), ("hq", 14), ("fp8", 14)):
         _forced_sweep([(prec, False, p, n) for p, n in shapes], variants, 3, min_ran)
+    # fp32: 16 or 8 blocks per workgroup (instances 50..52), 32- and 64-row tiles
+    _forced_sweep([("fp32", False, p, n) for p, n in shapes + [((2, 64, 24, 8), 150), ((1, 96, 16, 16), 77)]],
+                  [(3 << 24) | i for i in range(50, 53)], 3, 16)
     # the automatic choice with a bias (applied before the results are staged)
     from ksmm_amd.kernel import query_tile
 
