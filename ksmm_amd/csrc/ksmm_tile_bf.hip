@@ -228,7 +228,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const TX *__re
 // kernel reads and writes the same number of bytes as whole lines).  Here
 //  * neighbouring lanes read the vectors of neighbouring groups: runs of 16 * NG bytes per
 //    (row, k), whole runs of 8 k when the workgroup covers d;
-//  * the results leave through LDS ([n][m][group], 16-byte pieces, the group xor-ed with m so
+//  * the results leave through LDS ([n][m][group], 16-byte pieces, the group xor-ed with bits of m so
 //    that neighbouring lanes fall on distinct banks): runs of 16 * NG bytes per (row, m), or of
 //    TM * d * 2 bytes when the workgroup covers d;
 //  * the planes of a group start 256 / NG bytes apart in the banks (the lanes of one 4-byte
@@ -342,9 +342,12 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
             const int g = v % NG, k8 = v / NG % KH, nn = v / (KH * NG);
             // k = k8 and k8 + 8 of row nn: positions 2 * k8 and 2 * k8 + 1, i.e. 4-byte piece k8 & 3
             // of the 16-byte half k8 >> 2 (swapped for rows 8..15 of every 16)
-            // (TK = 8: k = k8 and k8 + 4 at positions 2 * k8 and 2 * k8 + 1 of a 16-byte row)
+            // (TK = 8: k = k8 and k8 + 4 at positions 2 * k8 and 2 * k8 + 1 of a 16-byte row, its two
+            // 8-byte halves swapped for rows 16..31 of every 32: the 32 rows an 8-byte operand read
+            // covers then fall on distinct banks)
             half_t *const dst = xs(buf, g * DD) + nn * TK +
-                                (TK == 16 ? ((((k8 >> 2) ^ ((nn >> 3) & 1)) << 3) | ((k8 & 3) << 1)) : (k8 << 1));
+                                (TK == 16 ? ((((k8 >> 2) ^ ((nn >> 3) & 1)) << 3) | ((k8 & 3) << 1))
+                                          : ((k8 ^ (2 * ((nn >> 4) & 1))) << 1));
             uint4_t c0, c1;  // register p: d_i = 2p (low half) and 2p + 1 (high half), as fp16
             if constexpr (sizeof(TX) == 2) {
                 c0 = xreg[slot][i][0];
@@ -382,7 +385,7 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int n = (wn * NT + j) * 32 + l32;
-        xrow[j] = TK == 16 ? n * TK + ((lq ^ ((n >> 3) & 1)) << 3) : n * TK + 4 * lq;
+        xrow[j] = TK == 16 ? n * TK + ((lq ^ ((n >> 3) & 1)) << 3) : n * TK + 4 * (lq ^ ((n >> 4) & 1));
     }
     auto multiply = [&](int buf) {
 #pragma unroll
@@ -454,6 +457,9 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
         // the NG chunks of one (n, m) sit in NG waves and are adjacent in y, as are the m of one
         // row when the group is all of d
         uint4_t *const ot = (uint4_t *)smem;
+        // (rows of m are 16 * NG bytes apart: 16 / NG consecutive m cover the banks once, so the
+        // group is xor-ed with m / (16 / NG))
+        auto okey = [](int ml) { return (ml * NG >> 4) & (NG - 1); };
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -469,7 +475,7 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
                     pack_t<half_t, DD> o;
 #pragma unroll
                     for (int dd = 0; dd < DD; ++dd) o.e[dd] = (half_t)epi_finish(ep, acc[dd][i][j][e], bv[dd]);
-                    ot[(nl * TM + ml) * NG + (wg ^ (ml & (NG - 1)))] = __builtin_bit_cast(uint4_t, o);
+                    ot[(nl * TM + ml) * NG + (wg ^ okey(ml))] = __builtin_bit_cast(uint4_t, o);
                 }
             }
         __syncthreads();
@@ -480,7 +486,7 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
             const int ch = q % NG, ml = q / NG % TM, nl = q / (NG * TM);
             if (n0 + nl < batch)
                 *(uint4_t *)(y + (size_t)(n0 + nl) * out_size + ((size_t)a_i * b + m0 + ml) * d + dg * DDA + ch * DD) =
-                    ot[(nl * TM + ml) * NG + (ch ^ (ml & (NG - 1)))];
+                    ot[(nl * TM + ml) * NG + (ch ^ okey(ml))];
         }
         return;
     }
@@ -715,8 +721,11 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
     // the 4 results of one (n, m) are adjacent in y: one 16-byte store
     if constexpr (FL) {
         // the NG groups of one (n, m) sit in NG waves and are adjacent in y: the tile goes to LDS
-        // as [n][m][group] (16-byte pieces, the group xor-ed with m) and leaves in whole runs
+        // as [n][m][group] (16-byte pieces, the group xor-ed with bits of m) and leaves in whole runs
         uint4_t *const ot = (uint4_t *)smem;
+        // (rows of m are 16 * NG bytes apart: 16 / NG consecutive m cover the banks once, so the
+        // group is xor-ed with m / (16 / NG))
+        auto okey = [](int ml) { return (ml * NG >> 4) & (NG - 1); };
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -732,7 +741,7 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
                     pack_t<float, DD> o;
 #pragma unroll
                     for (int dd = 0; dd < DD; ++dd) o.e[dd] = epi_finish(ep, acc[dd][i][j][e], bv[dd]);
-                    ot[(nl * TM + ml) * NG + (wg ^ (ml & (NG - 1)))] = __builtin_bit_cast(uint4_t, o);
+                    ot[(nl * TM + ml) * NG + (wg ^ okey(ml))] = __builtin_bit_cast(uint4_t, o);
                 }
             }
         __syncthreads();
@@ -743,7 +752,7 @@ __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) voi
             const int ch = q % NG, ml = q / NG % TM, nl = q / (NG * TM);
             if (n0 + nl < batch)
                 *(uint4_t *)(y + (size_t)(n0 + nl) * out_size + ((size_t)a_i * b + m0 + ml) * d + dg * DDA + ch * DD) =
-                    ot[(nl * TM + ml) * NG + (ch ^ (ml & (NG - 1)))];
+                    ot[(nl * TM + ml) * NG + (ch ^ okey(ml))];
         }
         return;
     }
