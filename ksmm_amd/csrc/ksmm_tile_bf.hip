@@ -236,7 +236,7 @@ __global__ __launch_bounds__(64 * WM * WN) void ks_tile_bf_kernel(const TX *__re
 // The accumulators of a workgroup are 8 * NG * TM * TN floats in 128 registers of 512 lanes, so
 // the tile shrinks as NG grows and weights and rows are read again more often: 32 blocks
 // (64-byte runs) on a 64 x 32 tile are the best trade (3.85 ms on the pattern above; 64 blocks
-// on 32 x 32: 4.6 ms; 16 blocks on 64 x 64 without the staged results: 5.4 ms).
+// on 32 x 32: 4.6 ms; 16 blocks on 64 x 64: 4.4 ms).
 template <typename TX, typename TW, int TM, int TN, int WM, int WN, int PDX, int PDW, int NG = 1, int TK = 16>
 __global__ __launch_bounds__(64 * WM * WN * NG, (WM * WN * NG >= 8 ? 1 : 2)) void ks_tile_bf8_kernel(const TX *__restrict__ x,
                                                                 const TW *__restrict__ w,
