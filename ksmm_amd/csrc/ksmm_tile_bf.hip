@@ -863,7 +863,8 @@ const BfInst bf_insts[] = {
     BF8L_INST(3, half_t, fp8_t, 2, 8, 64, 64, 2, 2, 2, 2),
     BF8L_INST(2, fp8_t, fp8_t, 4, 8, 64, 32, 2, 1, 2, 2), BF8L_INST(2, fp8_t, fp8_t, 4, 8, 32, 64, 1, 2, 2, 2),
     BF8L_INST(2, fp8_t, fp8_t, 2, 8, 64, 64, 2, 2, 2, 2),
-    // fp32: 16 or 8 blocks per workgroup (32 blocks on a 32 x 32 tile never won)
+    // fp32: 16 or 8 blocks per workgroup (32 blocks on a 32 x 32 tile never won; 8 blocks in slabs of
+    // 16 k, which fit, were 2-8 % slower than in slabs of 8)
     BF4L_INST(4, 8, 64, 32, 2, 1, 2, 2), BF4L_INST(4, 8, 32, 64, 1, 2, 2, 2), BF4L_INST(2, 8, 64, 64, 2, 2, 2, 2),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
