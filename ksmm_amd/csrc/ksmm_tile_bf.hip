@@ -866,6 +866,16 @@ const BfInst bf_insts[] = {
     // fp32: 16 or 8 blocks per workgroup (32 blocks on a 32 x 32 tile never won; 8 blocks in slabs of
     // 16 k, which fit, were 2-8 % slower than in slabs of 8)
     BF4L_INST(4, 8, 64, 32, 2, 1, 2, 2), BF4L_INST(4, 8, 32, 64, 1, 2, 2, 2), BF4L_INST(2, 8, 64, 64, 2, 2, 2, 2),
+    // 16-bit d = 4 and 2 whole on 8 waves (the 4-wave instances above leave one wave per SIMD when
+    // their planes fill the LDS: fp16 (48,384,384,4) 4265 -> 3091 us on the 128 x 128 tile,
+    // (64,256,256,4) 3246 -> 2204, (96,192,192,4) 2888 -> 2218 on 64 x 128 with slabs of 16)
+    BF_INST(1, half_t, half_t, 4, 64, 128, 16, 2, 4), BF_INST(1, half_t, half_t, 4, 128, 128, 32, 2, 4),
+    BF_INST(1, half_t, half_t, 4, 128, 128, 16, 2, 4), BF_INST(1, half_t, half_t, 4, 64, 64, 16, 2, 2),
+    BF_INST(1, half_t, half_t, 2, 128, 128, 32, 2, 4), BF_INST(1, half_t, half_t, 2, 128, 256, 32, 2, 4),
+    BF_INST(1, half_t, half_t, 2, 256, 128, 32, 4, 2),
+    BF_INST(3, half_t, fp8_t, 4, 64, 128, 16, 2, 4), BF_INST(3, half_t, fp8_t, 4, 128, 128, 32, 2, 4),
+    BF_INST(3, half_t, fp8_t, 2, 128, 128, 32, 2, 4),
+    BF_INST_Q(4, 64, 128, 32, 2, 4), BF_INST_Q(4, 128, 128, 32, 2, 4), BF_INST_Q(2, 128, 128, 32, 2, 4),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 
@@ -925,14 +935,23 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             // the batch-size-last GEMM tiles between two transposes beat this kernel (the
             // transposes move each operand once more, the GEMM tiles run at 2-3x its
             // matrix-core rate)
-            if (p.d == t.dd && combo != 0 && p.b >= 512 && (int64_t)p.b * p.c >= 512 * 512) continue;
+            // (e4m3 input: the bounds measured for it below)
+            if (p.d == t.dd && combo != 0 && combo != 2 && p.b >= 512 && (int64_t)p.b * p.c >= 512 * 512) continue;
             // e4m3 input with d = 2 or 4 whole: measured against the transposed route on the 102
             // such patterns of the reference's list (batch 25088), the direct kernel wins (time
             // ratio 0.6-0.97) with short c or narrow blocks and loses (1.1-2.3) elsewhere: the
             // e4m3 GEMM tiles in the middle of the other route multiply at twice the rate
+            // (with the instances on 8 waves, measured again on the 110 patterns that had stayed on
+            // the other route: the direct kernel also wins, ratio 0.66-0.94, for d = 4 on blocks up to
+            // 384 x 384 / 768 x 192 with b a multiple of 64 and c <= 384, and for d = 2 with b a
+            // multiple of 128 up to 512 x 512 / 256 x 1024 / 1536 x 384; it loses, 1.1-1.8, on 96-row
+            // blocks, c = 768 and blocks of 768 x 768 and more)
             if (combo == 2 && !t.pd) {
-                const bool pays = p.d == 2 ? (p.c <= 128 || (p.c <= 256 && p.b <= 512))
-                                           : (p.c <= 96 || (p.b <= 64 && p.a >= 3));
+                const int64_t bc = (int64_t)p.b * p.c;
+                const bool pays = p.d == 2 ? (p.c <= 128 || (p.c <= 256 && p.b <= 512) ||
+                                              (p.b % 128 == 0 && (bc <= 262144 || (bc <= 589824 && p.c <= 384))))
+                                           : (p.c <= 96 || (p.b <= 64 && p.a >= 3) ||
+                                              (p.b % 64 == 0 && p.c <= 384 && (bc < 147456 || (bc == 147456 && (p.a >= 4 || p.c <= 192)))));
                 if (!pays) continue;
             }
             const bool wide = t.pd >= 256;  // 32 or 16 blocks per workgroup
@@ -962,7 +981,9 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
                 if (!pays) continue;
             }
             const int64_t wgs = (int64_t)p.a * (p.d / t.dd) * (p.b / t.tm) * ((p.batch + t.tn - 1) / t.tn);
-            int64_t score = (int64_t)t.tm * 1000 + t.tn;
+            // (between equal tiles the instance on more waves: two waves per SIMD where the planes
+            // leave room for one workgroup per CU)
+            int64_t score = (int64_t)t.tm * 1000 + t.tn + t.threads / 256;
             // the pipelined 64 x 64 form first (1.1-1.3x the plain instances on (1,192,192,8..16),
             // (4,128,128,8), (1,64,64,64) at batch 25088)
             if (t.pd && !wide && t.tn == 64 && wgs >= 512) score += 500000;

@@ -88,7 +88,9 @@ def test_tile_bf_groups_of_blocks_forced():
              ("fp32", (1, 128, 32, 2)), ("fp8", (1, 128, 64, 16)),
              # 5, 7 and 12 slabs of 16: whole and partial rounds of the two-slab register pipeline
              ("fp16", (1, 64, 80, 8)), ("fp16", (1, 192, 192, 16)), ("fp8", (2, 64, 112, 8)),
-             ("fp32", (1, 64, 80, 8)), ("fp32", (1, 192, 192, 4)), ("fp32", (2, 64, 112, 12))]
+             ("fp32", (1, 64, 80, 8)), ("fp32", (1, 192, 192, 4)), ("fp32", (2, 64, 112, 12)),
+             # d = 4 and 2 whole on the 8-wave instances (128-row tiles too)
+             ("fp16", (1, 128, 48, 4)), ("fp16", (2, 256, 32, 2)), ("fp8", (2, 128, 32, 4)), ("fp8", (1, 128, 64, 2))]
     ran, strided = 0, 0
     for prec, pattern in cases:
         a, b, c, d = pattern
@@ -105,7 +107,7 @@ def test_tile_bf_groups_of_blocks_forced():
             x = seeded_input(a * c * d, batch, False, seed=32)
             z = O.ks_apply_einsum(wr, round_to(x, xprec)[0], False)
             zb = z + bias.double().numpy()[None, :]
-            for inst in range(40):
+            for inst in list(range(40)) + list(range(53, 63)):
                 try:
                     y = Kernel.forward(x.to(x_dt).cuda(), fac, False, a, b, c, d, scale=scale, algo=3,
                                        variant=(3 << 24) | inst)
@@ -130,7 +132,11 @@ def test_tile_bf_groups_of_blocks_forced():
                    ("fp8", False, (1, 64, 128, 4), 203), ("fp8", False, (3, 32, 32, 4), 1000),
                    ("fp8", False, (1, 768, 192, 2), 264)],
                   [(3 << 24) | i for i in range(35, 41)] + [-1], 3, 14)
-    assert ran >= 30 and strided >= 12, (ran, strided)
+    # the same on 8 waves (instances 63..65)
+    _forced_sweep([("fp8", False, (1, 256, 64, 2), 520), ("fp8", False, (2, 128, 96, 2), 77),
+                   ("fp8", False, (1, 64, 128, 4), 203), ("fp8", False, (2, 128, 64, 4), 1000)],
+                  [(3 << 24) | i for i in range(63, 66)], 3, 5)
+    assert ran >= 40 and strided >= 12, (ran, strided)
 
 
 def test_tile_bf_wide_groups_forced():
