@@ -586,6 +586,26 @@ const TileInst tile_insts[] = {
     TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, true, 128, 256, 32, 2, 2, true),
     TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, false, 64, 256, 64, 1, 4, true),
     TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, false, 128, 256, 32, 2, 2, true),
+    // the 16-bit ones on 8 waves (the planes of the instances above leave one workgroup of 4 waves per CU)
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, true, 128, 256, 32, 2, 4, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, true, 64, 256, 64, 2, 4, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, false, 128, 256, 32, 2, 4, true),
+    TILE_INST_R(1, half_t, half_t, half_t, half_t, false, 64, 256, 64, 2, 4, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, true, 128, 256, 32, 2, 4, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, true, 64, 256, 64, 2, 4, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, false, 128, 256, 32, 2, 4, true),
+    TILE_INST_R(2, half_t, fp8_t, fp8_t, half_t, false, 64, 256, 64, 2, 4, true),
+    TILE_INST_R(0, float, float, float, float, true, 128, 256, 16, 2, 4, true),
+    TILE_INST_R(0, float, float, float, float, true, 64, 256, 16, 2, 4, true),
+    TILE_INST_R(0, float, float, float, float, false, 128, 256, 16, 2, 4, true),
+    TILE_INST_R(0, float, float, float, float, false, 64, 256, 16, 2, 4, true),
+    // aligned b on 8 waves
+    TILE_INST(1, half_t, half_t, half_t, half_t, true, 128, 256, 32, 2, 4),
+    TILE_INST(1, half_t, half_t, half_t, half_t, false, 128, 256, 32, 2, 4),
+    TILE_INST(2, half_t, fp8_t, fp8_t, half_t, true, 128, 256, 32, 2, 4),
+    TILE_INST(2, half_t, fp8_t, fp8_t, half_t, false, 128, 256, 32, 2, 4),
+    TILE_INST(0, float, float, float, float, true, 128, 256, 16, 2, 4),
+    TILE_INST(0, float, float, float, float, false, 128, 256, 16, 2, 4),
 };
 constexpr int N_TILE_INSTS = sizeof(tile_insts) / sizeof(TileInst);
 
@@ -676,7 +696,9 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             const TileInst &t = tile_insts[i];
             if (!tile_fits(t, p, combo)) continue;
             const int64_t wgs = (int64_t)p.a * p.d * ((p.b + t.tm - 1) / t.tm) * ((p.batch + t.tn - 1) / t.tn);
-            int64_t score = (int64_t)t.tm * 1000 + t.tn;
+            // (between equal tiles the instance on 8 waves: with 4, the planes of the large tiles leave
+            // one wave per SIMD; (16,1855,256,1) fp16 1343 -> 821 us, (64,455,64,1) 933 -> 533)
+            int64_t score = (int64_t)t.tm * 1000 + t.tn + t.threads / 256;
             if (wgs < 512) score -= 100000;
             if (score > best_score) {
                 best_score = score;

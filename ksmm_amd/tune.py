@@ -168,7 +168,7 @@ def tune_pattern(pattern, prec, bs_last, batch, lib_mod, rotation_bytes=1.3e9, t
         # a retune after instances were added to some tile sub-families: only those, against what
         # the present table (or, without a row, the heuristic) picks
         now = query_tile(batch, pattern, dt, dt, bs_last)
-        pool = [(al, v) for al, v in pools[0] if al == 3 and (v >> 24) in tile_subs]
+        pool = [(al, v) for al, v in pools[0] + pools[1] if al == 3 and (v >> 24) in tile_subs]
         if now["algo"] in (2, 3) and (now["algo"], now["variant"]) not in pool:
             pool.append((now["algo"], now["variant"]))
         pools = (pool,)
@@ -389,8 +389,8 @@ def main():
     ap.add_argument("--update-best", help="directory of existing *.best files: replace the lines of the measured patterns")
     ap.add_argument("--shard", default="0/1", help="i/n: take every n-th pattern starting at i")
     ap.add_argument("--time-limit", type=float, default=1e9, help="stop (and save) after this many seconds")
-    ap.add_argument("--tile-subs", help="comma-separated tile sub-families (2 stream, 4 GEMM, 1 weight-stationary, "
-                    "3 d > 1 tiles): try only their instances and the present table's pick")
+    ap.add_argument("--tile-subs", help="comma-separated tile sub-families (0 k-loop tiles, 2 stream, 4 GEMM, "
+                    "1 weight-stationary, 3 d > 1 tiles): try only their instances and the present table's pick")
     args = ap.parse_args()
     entries = []
     for p in args.merge:

@@ -356,7 +356,7 @@ def test_tile_subfamilies_forced():
               ("fp16", True, (2, 70, 64, 2), 520), ("fp16", False, (2, 77, 64, 1), 520), ("fp32", True, (1, 45, 48, 3), 520),
               ("fp32", False, (1, 130, 32, 1), 520), ("fp8", True, (1, 50, 64, 2), 528), ("fp8", False, (2, 200, 64, 1), 528),
               ("fp16", True, (1, 449, 64, 1), 264)]
-    _forced_sweep(kcases, [(0 << 24) | i for i in range(72)], 3, 40)                     # k-loop
+    _forced_sweep(kcases, [(0 << 24) | i for i in range(90)], 3, 52)                     # k-loop
     wcases = [("fp32", True, (2, 64, 64, 2), 520), ("fp32", False, (2, 96, 96, 1), 520),
               ("fp16", True, (2, 64, 64, 2), 520), ("fp16", False, (3, 64, 64, 1), 520),
               ("fp8", True, (2, 64, 64, 1), 528), ("hq", False, (2, 96, 96, 1), 520)]
