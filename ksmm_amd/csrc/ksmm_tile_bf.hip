@@ -876,6 +876,9 @@ const BfInst bf_insts[] = {
     BF_INST(3, half_t, fp8_t, 4, 64, 128, 16, 2, 4), BF_INST(3, half_t, fp8_t, 4, 128, 128, 32, 2, 4),
     BF_INST(3, half_t, fp8_t, 2, 128, 128, 32, 2, 4),
     BF_INST_Q(4, 64, 128, 32, 2, 4), BF_INST_Q(4, 128, 128, 32, 2, 4), BF_INST_Q(2, 128, 128, 32, 2, 4),
+    // fp32 groups of 4 on 128-row tiles, 8 waves (one slab in flight in registers: two spill); big d = 4
+    // blocks 4-9 % faster than on 64 x 128 ((64,256,256,4) 8419 -> 7900 us, (32,128,128,4) 1240 -> 1122)
+    BF4_INST(128, 64, 4, 2, 2, 2), BF4_INST(128, 128, 2, 4, 1, 1), BF4_INST(128, 128, 4, 2, 1, 1),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 

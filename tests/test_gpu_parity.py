@@ -154,6 +154,9 @@ def test_tile_bf_wide_groups_forced():
     # fp32: 16 or 8 blocks per workgroup (instances 50..52), 32- and 64-row tiles
     _forced_sweep([("fp32", False, p, n) for p, n in shapes + [((2, 64, 24, 8), 150), ((1, 96, 16, 16), 77)]],
                   [(3 << 24) | i for i in range(50, 53)], 3, 16)
+    # fp32 groups of 4 on 128-row tiles (instances 66..68)
+    _forced_sweep([("fp32", False, (1, 128, 48, 4), 520), ("fp32", False, (2, 256, 32, 8), 77),
+                   ("fp32", False, (1, 128, 80, 12), 300)], [(3 << 24) | i for i in range(66, 69)], 3, 9)
     # the automatic choice with a bias (applied before the results are staged)
     from ksmm_amd.kernel import query_tile
 
