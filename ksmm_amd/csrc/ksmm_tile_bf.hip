@@ -879,6 +879,9 @@ const BfInst bf_insts[] = {
     // fp32 groups of 4 on 128-row tiles, 8 waves (one slab in flight in registers: two spill); big d = 4
     // blocks 4-9 % faster than on 64 x 128 ((64,256,256,4) 8419 -> 7900 us, (32,128,128,4) 1240 -> 1122)
     BF4_INST(128, 64, 4, 2, 2, 2), BF4_INST(128, 128, 2, 4, 1, 1), BF4_INST(128, 128, 4, 2, 1, 1),
+    // 16-bit groups of 8 on a 128 x 64 tile, 8 waves
+    BF8_INST(1, half_t, half_t, 128, 64, 4, 2, 2, 2), BF8_INST(3, half_t, fp8_t, 128, 64, 4, 2, 2, 2),
+    BF8_INST(2, fp8_t, fp8_t, 128, 64, 4, 2, 2, 2),
 };
 constexpr int N_BF_INSTS = sizeof(bf_insts) / sizeof(BfInst);
 

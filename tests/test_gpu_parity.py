@@ -107,7 +107,7 @@ def test_tile_bf_groups_of_blocks_forced():
             x = seeded_input(a * c * d, batch, False, seed=32)
             z = O.ks_apply_einsum(wr, round_to(x, xprec)[0], False)
             zb = z + bias.double().numpy()[None, :]
-            for inst in list(range(40)) + list(range(53, 63)):
+            for inst in list(range(40)) + list(range(53, 63)) + [69, 70]:
                 try:
                     y = Kernel.forward(x.to(x_dt).cuda(), fac, False, a, b, c, d, scale=scale, algo=3,
                                        variant=(3 << 24) | inst)
@@ -126,7 +126,7 @@ def test_tile_bf_groups_of_blocks_forced():
     # e4m3 input and weights (8-byte vectors of a group, decoded on their way to LDS)
     _forced_sweep([("fp8", False, (1, 128, 64, 16), 520), ("fp8", False, (2, 64, 80, 8), 77),
                    ("fp8", False, (1, 192, 192, 8), 1000), ("fp8", False, (1, 64, 32, 24), 203)],
-                  [(3 << 24) | i for i in range(27, 41)], 3, 8)
+                  [(3 << 24) | i for i in list(range(27, 41)) + [71]], 3, 9)
     # e4m3 input and weights, d = 2 or 4 whole (16-byte vectors of 8 or 4 k of every d_i)
     _forced_sweep([("fp8", False, (1, 256, 64, 2), 520), ("fp8", False, (2, 128, 96, 2), 77),
                    ("fp8", False, (1, 64, 128, 4), 203), ("fp8", False, (3, 32, 32, 4), 1000),
