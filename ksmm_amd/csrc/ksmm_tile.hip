@@ -696,9 +696,10 @@ int tile_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
             const TileInst &t = tile_insts[i];
             if (!tile_fits(t, p, combo)) continue;
             const int64_t wgs = (int64_t)p.a * p.d * ((p.b + t.tm - 1) / t.tm) * ((p.batch + t.tn - 1) / t.tn);
-            // (between equal tiles the instance on 8 waves: with 4, the planes of the large tiles leave
+            // (any b: between equal tiles the instance on 8 waves: with 4, the planes of the large tiles leave
             // one wave per SIMD; (16,1855,256,1) fp16 1343 -> 821 us, (64,455,64,1) 933 -> 533)
-            int64_t score = (int64_t)t.tm * 1000 + t.tn + t.threads / 256;
+            // (the aligned 8-wave instances are named by the measured table only)
+            int64_t score = (int64_t)t.tm * 1000 + t.tn + (t.ragged_b ? t.threads / 256 : 0);
             if (wgs < 512) score -= 100000;
             if (score > best_score) {
                 best_score = score;

@@ -961,6 +961,10 @@ int tile_bf_run(const Problem &p, int variant, bool launch, ksmm_tile *tile)
                 if (!pays) continue;
             }
             const bool wide = t.pd >= 256;  // 32 or 16 blocks per workgroup
+            // fp32 groups of 4 on 128-row tiles: the best choice on half of the patterns they fit and up
+            // to 18 % behind the 64-row tiles on the others, with no simple bound between: named by the
+            // measured table only
+            if (combo == 0 && t.pd && !wide && t.tm == 128) continue;
             if (wide && combo == 0) {
                 // fp32, measured the same way on the 161 patterns with d a multiple of 8: the
                 // wider groups win from d = 16 on (0.61-0.98 of the time of the groups of 4; 8
